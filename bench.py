@@ -1,0 +1,239 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X receive-side unpack path.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One "step" is the unpack of one 8 MiB chunk of the 4-flow workload (about 2155 descriptors of at most 4 KiB,
+byte-unaligned sources in a 256 MiB bounce pool, contiguous destination), cut into two 4 MiB requests the way
+NCCL slices an 8 MiB chunk.  The chunk goes through the persistent engine exactly as the plugin drives it:
+descriptors are copied into a slot of the 16-deep mapped ring, the slot is published, the GPU unpacks it and
+writes a completion word that the host polls -- no kernel launch per request.  Successive steps use different
+descriptor lists and different destinations (a ring of chunks bigger than the 256 MiB Infinity Cache), so the
+figure is HBM traffic, not cache hits.  Bounce pool, descriptor lists and destinations are resident before the
+timed region starts; nothing crosses PCIe during it except descriptors and completion words.
+
+Prints ONE JSON line: payload GB/s (`value`), the HBM roofline of the dominant kernel, p50/p99 request
+completion latency, and a memcpy-per-descriptor CPU baseline timed on this machine's host cores.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+import __graft_entry__ as graft
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+CHUNK_CONFIG = 2
+
+
+def percentile(values, q):
+    return float(np.percentile(np.asarray(values, dtype=np.float64), q))
+
+
+def cpu_baseline(oracle, wl, pool, threads, budget_s):
+    """memcpy-per-descriptor over the same descriptor list, pool and destination in host DRAM."""
+    dst = np.empty(wl.info.dst_bytes + 64, dtype=np.uint8)
+    descs = np.ascontiguousarray(wl.descs)
+    probe = (ctypes.c_double * 3)()
+    rc = oracle.tcpx_oracle_unpack_timed(dst.ctypes.data, pool.ctypes.data, descs.ctypes.data, len(descs), threads, 2, 3, probe)
+    assert rc == 0
+    per_iter = max(min(probe), 1e-6)
+    iters = int(max(20, min(2000, budget_s / per_iter)))
+    secs = (ctypes.c_double * iters)()
+    rc = oracle.tcpx_oracle_unpack_timed(dst.ctypes.data, pool.ctypes.data, descs.ctypes.data, len(descs), threads, 5, iters, secs)
+    assert rc == 0
+    med = float(np.median(np.asarray(secs[:])))
+    return wl.info.payload_bytes / med / 1e9, iters
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=4000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--chunks", type=int, default=48, help="distinct chunks (descriptor lists + destinations) cycled through")
+    ap.add_argument("--depth", type=int, default=16, help="slots of the mapped ring in flight")
+    ap.add_argument("--cpu-seconds", type=float, default=8.0, help="time budget per CPU baseline leg")
+    ap.add_argument("--skip-extras", action="store_true", help="only the headline measurement")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this path runs on one GPU; --gpus %d is not supported (every GPU would run an independent copy)" % args.gpus)
+
+    import torch
+
+    pkg = graft.load_package()
+    hip = pkg.hip_layer()  # raises if the HIP library is missing; there is no fallback
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    dev = 0
+    name = ctypes.create_string_buffer(256)
+    cus = ctypes.c_int()
+    pkg.check(hip.tcpxuDeviceInfo(dev, name, 256, ctypes.byref(cus)), "tcpxuDeviceInfo")
+
+    # ---- inputs: one pool, `chunks` descriptor lists, `chunks` destinations ------------------------------
+    workloads = [pkg.Workload(CHUNK_CONFIG, seed=0xC0FFEE02 + 7919 * i) for i in range(args.chunks)]
+    info0 = workloads[0].info
+    chunk_bytes = info0.payload_bytes
+    pool = np.empty(info0.pool_bytes, dtype=np.uint8)
+    workloads[0].fill_window(0, pool)
+    pool_d = torch.from_numpy(pool).to("cuda:0")
+    dst_d = torch.full((args.chunks * chunk_bytes + 512,), 0xA5, dtype=torch.uint8, device="cuda:0")
+    dst_base = dst_d.data_ptr() + 256
+    torch.cuda.synchronize()
+
+    per_chunk_items = []
+    keep = []
+    for c, wl in enumerate(workloads):
+        items = []
+        for r in wl.requests:
+            d = np.ascontiguousarray(wl.descs[int(r["first_desc"]) : int(r["first_desc"]) + int(r["n_descs"])])
+            keep.append(d)
+            items.append((pool_d.data_ptr(), dst_base + c * chunk_bytes, d.ctypes.data, len(d)))
+        per_chunk_items.append(items)
+    slots_per_step = len(per_chunk_items[0])
+    descs_per_step = float(np.mean([wl.info.n_descs for wl in workloads]))
+
+    def item_array(first_step, n_steps):
+        flat = []
+        for s in range(first_step, first_step + n_steps):
+            flat.extend(per_chunk_items[s % args.chunks])
+        arr = (pkg.StreamItem * len(flat))()
+        for i, (b, d, p, n) in enumerate(flat):
+            arr[i].bounce_base, arr[i].dst_base, arr[i].descs_host, arr[i].n_descs = b, d, p, n
+        return arr
+
+    engine = ctypes.c_void_p()
+    cfg = pkg.EngineConfig(0, 0, 0, 0)
+    pkg.check(hip.tcpxuEngineCreate(dev, ctypes.byref(cfg), ctypes.byref(engine)), "tcpxuEngineCreate")
+
+    def run(items, depth, want_latency=False):
+        wall, kern = ctypes.c_double(), ctypes.c_double()
+        lat = (ctypes.c_double * len(items))() if want_latency else None
+        rc = hip.tcpxuEngineRunTimed(engine, items, len(items), depth, 20000, ctypes.byref(wall), ctypes.byref(kern), lat)
+        pkg.check(rc, "tcpxuEngineRunTimed")
+        return wall.value, kern.value, (np.asarray(lat[:]) if want_latency else None)
+
+    # ---- warmup, then exactly K timed steps inside one launch of the persistent kernel ---------------------
+    if args.warmup > 0:
+        run(item_array(0, args.warmup), args.depth)
+    timed_items = item_array(args.warmup, args.steps)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    wall_us, kernel_us, _ = run(timed_items, args.depth)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    payload = float(sum(workloads[(args.warmup + s) % args.chunks].info.payload_bytes for s in range(args.steps)))
+    value_gbps = payload / (wall_us * 1e-6) / 1e9
+    achieved = 2.0 * payload / (kernel_us * 1e-6) / 1e9
+
+    # ---- parity spot check: the last chunk written must equal the oracle's bytes ---------------------------
+    oracle = graft.load_oracle()
+    last = (args.warmup + args.steps - 1) % args.chunks
+    expect = np.full(chunk_bytes, 0xA5, dtype=np.uint8)
+    graft.oracle_unpack(oracle, expect, pool, np.ascontiguousarray(workloads[last].descs))
+    got = dst_d[256 + last * chunk_bytes : 256 + (last + 1) * chunk_bytes].cpu().numpy()
+    parity_ok = bool(np.array_equal(got, expect))
+
+    result = {
+        "metric": "unpack payload GB/s + % HBM r+w roofline at 8 MiB chunk; p50 request us",
+        "value": round(value_gbps, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_us / 1000.0 / args.steps, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u8",
+        "data": "synthetic",
+        "config": {
+            "workload": "8 MiB chunk, 4 interleaved flows, ~2155 fragments (90% 4096 B, 10% U[64,4095]), byte-unaligned "
+            "sources in a 256 MiB pool, 2 x 4 MiB requests per chunk, %d distinct chunks cycled, ring depth %d"
+            % (args.chunks, args.depth),
+            "path": "persistent engine: mapped descriptor ring -> gfx950 unpack kernel -> mapped completion word",
+            "descriptors_per_step": round(descs_per_step, 1),
+            "slots_per_step": slots_per_step,
+            "device": name.value.decode(),
+            "compute_units": cus.value,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "unpack_engine_kernel",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "bytes_per_launch": 2.0 * payload,
+            "launch_us": round(kernel_us, 1),
+        },
+        "parity_ok": parity_ok,
+        "timed_region_s": round(t1 - t0, 4),
+    }
+
+    if not args.skip_extras:
+        # Request completion latency, one request in flight: publish -> host poller sees the completion word.
+        storm = pkg.Workload(3, seed=0xC0FFEE03)
+        sd = np.array(storm.descs, copy=True)
+        n_lat = 2000
+        lat_items = (pkg.StreamItem * n_lat)()
+        for i in range(n_lat):
+            r = storm.requests[i % len(storm.requests)]
+            lat_items[i].bounce_base = pool_d.data_ptr()  # offsets beyond 256 MiB are folded into this pool below
+            lat_items[i].dst_base = dst_base + int(r["dst_off"]) % (args.chunks * chunk_bytes - 65536)
+            lat_items[i].descs_host = sd.ctypes.data + 16 * int(r["first_desc"])
+            lat_items[i].n_descs = int(r["n_descs"])
+        sd["src_off"] %= info0.pool_bytes
+        sd["dst_off"] %= 65536
+        _, _, lat64k = run(lat_items, 1, want_latency=True)
+        lat4m_items = item_array(0, 200)
+        _, _, lat4m = run(lat4m_items, 1, want_latency=True)
+        result["latency_us"] = {
+            "definition": "host publish of a slot -> host poller observes the completion word, one request in flight",
+            "request_64KiB_16_descs": {"p50": round(percentile(lat64k, 50), 2), "p99": round(percentile(lat64k, 99), 2)},
+            "request_4MiB_1078_descs": {"p50": round(percentile(lat4m, 50), 2), "p99": round(percentile(lat4m, 99), 2)},
+        }
+        result["p50_request_us"] = result["latency_us"]["request_64KiB_16_descs"]["p50"]
+
+        # Launch-per-batch kernel on the same chunk and on the 256 MiB bulk workload, and a plain copy kernel.
+        us = ctypes.c_double()
+        d0 = torch.from_numpy(np.ascontiguousarray(workloads[0].descs).view(np.uint8)).to("cuda:0")
+        pkg.check(hip.tcpxuUnpackBatchTimed(dev, pool_d.data_ptr(), dst_base, d0.data_ptr(), workloads[0].info.n_descs, 20, 200, ctypes.byref(us)), "batch timed")
+        result["launch_per_batch_8MiB"] = {
+            "kernel": "unpack_batch_kernel",
+            "launch_us": round(us.value, 2),
+            "rw_GBps": round(2 * chunk_bytes / us.value / 1e3, 1),
+            "frac": round(2 * chunk_bytes / us.value / 1e3 / HBM_PEAK_GBPS, 4),
+        }
+        n_copy = min(256 << 20, (args.chunks * chunk_bytes) // 2 // 4096 * 4096)
+        pkg.check(hip.tcpxuCopyKernelTimed(dev, dst_base + n_copy, dst_base, n_copy, 5, 50, ctypes.byref(us)), "copy timed")
+        result["plain_copy_kernel"] = {"bytes": n_copy, "launch_us": round(us.value, 2), "rw_GBps": round(2 * n_copy / us.value / 1e3, 1)}
+        del d0
+
+    pkg.check(hip.tcpxuEngineDestroy(engine), "tcpxuEngineDestroy")
+
+    # ---- CPU baseline on this machine's host cores: rank 0, bounded sample ---------------------------------
+    threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16") or 16))
+    gbps_1, it1 = cpu_baseline(oracle, workloads[0], pool, 1, args.cpu_seconds)
+    gbps_t, itt = cpu_baseline(oracle, workloads[0], pool, threads, args.cpu_seconds)
+    result["cpu_baseline"] = {
+        "value": round(gbps_t, 2),
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": "the same 8 MiB chunk (descriptor list 0), pool and destination in host DRAM, memcpy per descriptor, "
+        "descriptor list range-partitioned over %d threads, median of %d iterations" % (threads, itt),
+        "single_thread": {"value": round(gbps_1, 2), "cores": 1, "iterations": it1},
+    }
+    print(json.dumps(result))
+    if not parity_ok:
+        sys.exit("bench.py: GPU result differs from the oracle")
+
+
+if __name__ == "__main__":
+    main()

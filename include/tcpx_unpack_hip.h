@@ -1,0 +1,171 @@
+/*
+ * tcpx_unpack_hip.h -- C-ABI of the HIP layer (libtcpxu_hip.so) of the MI355X receive-side unpack path.
+ *
+ * Everything the host-side plugin needs from the GPU goes through these entry points: plain pointers and
+ * sizes, no C++ types, no torch types.  Each entry point names the interface of the reference
+ * (google/nccl-plugin-gpudirecttcpx, paths relative to its root) that it stands in for.
+ *
+ * Result codes are the numeric values of ncclResult_t that the reference returns through its adapter
+ * (src/adapter/nccl/ret.h:22-31): 0 success, 1 unhandled device error, 2 system error, 3 internal error,
+ * 4 invalid argument, 5 invalid usage.
+ */
+#ifndef TCPX_UNPACK_HIP_H_
+#define TCPX_UNPACK_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TCPXU_SUCCESS 0
+#define TCPXU_DEVICE_ERROR 1
+#define TCPXU_SYSTEM_ERROR 2
+#define TCPXU_INTERNAL_ERROR 3
+#define TCPXU_INVALID_ARGUMENT 4
+#define TCPXU_INVALID_USAGE 5
+#define TCPXU_IN_PROGRESS 7 /* ncclInProgress: nothing wrong, try again */
+
+/* One unpack descriptor: copy `len` bytes from bounce_base + src_off to dst_base + dst_off.
+ * Same 16-byte layout as NCCL's `union loadMeta`, whose fields the reference fills at
+ * src/sock/tcpx.h:178-180 and whose 16-byte stride it relies on at src/net_tcpx.cc:1128-1130. */
+typedef struct tcpxuLoadMeta {
+  uint32_t src_off;
+  uint32_t len;
+  uint64_t dst_off;
+} tcpxuLoadMeta;
+
+/* Ring geometry the reference compiles against (NCCL's NCCL_NET_DEVICE_UNPACK_MAX_QUEUE_DEPTH and
+ * NET_UNPACK_MAX_SLICE_PAGES; used at src/devcomm/nccl/unpack_defs1.h:22-23). */
+#define TCPXU_QUEUE_DEPTH 16
+#define TCPXU_SLOT_PAGES 2048
+#define TCPXU_PAGE_SIZE 4096
+
+/* ---- device selection -------------------------------------------------------------------------------- */
+
+/* Number of visible GPUs.  Replaces gpu_n_dev (src/gpu/cuda_wrapper.cu:49-60). */
+int tcpxuDeviceCount(int* count);
+
+/* Human-readable name and compute-unit count of a GPU (for bench output). */
+int tcpxuDeviceInfo(int device, char* name, size_t name_len, int* compute_units);
+
+/* Last error message of the calling thread ("" if none). */
+const char* tcpxuLastError(void);
+
+/* ---- (1) bounce-page arena in HBM -------------------------------------------------------------------- */
+
+/* Allocates `bytes` of device memory as the bounce-page arena (4 KiB-aligned base) and returns its device
+ * address.  Replaces gpu_get_rxmem / GpumemImport, which import the receive-datapath-manager's NIC-bound page
+ * pool (src/gpu/cuda_wrapper.cu:214-224, src/gpu/rx_pool.cu:62-121): here the pool is a plain hipMalloc. */
+int tcpxuArenaCreate(int device, size_t bytes, void** arena_base);
+int tcpxuArenaDestroy(int device, void* arena_base);
+
+/* Plain device buffers and copies, so that a host driver needs no other GPU runtime. */
+int tcpxuDeviceAlloc(int device, size_t bytes, void** ptr);
+int tcpxuDeviceFree(int device, void* ptr);
+int tcpxuCopyToDevice(int device, void* dst_dev, const void* src_host, size_t bytes);
+int tcpxuCopyToHost(int device, void* dst_host, const void* src_dev, size_t bytes);
+int tcpxuFillDevice(int device, void* dst_dev, int byte_value, size_t bytes);
+int tcpxuDeviceSynchronize(int device);
+
+/* ---- (2) host-mapped unpack-metadata memory ---------------------------------------------------------- */
+
+/* Allocates `bytes` of pinned host memory that the GPU can read and write (hipHostMalloc, mapped and
+ * coherent) and returns both addresses.  Replaces the cuMemHostAlloc(DEVICEMAP|PORTABLE) +
+ * cuMemHostGetDevicePointer pair of __tcpxNetDeviceQueueNew (src/devcomm/nccl/unpack1.cu:41-43,54). */
+int tcpxuMappedAlloc(int device, size_t bytes, void** host_ptr, void** dev_ptr);
+int tcpxuMappedFree(int device, void* host_ptr);
+
+/* ---- (3) launch-per-batch unpack --------------------------------------------------------------------- */
+
+/* Scatter-gathers `n_descs` descriptors with one kernel launch on `stream` (a hipStream_t, NULL = the
+ * default stream): for each i, dst_base[dst_off_i .. +len_i) = bounce_base[src_off_i .. +len_i).
+ * `descs` must be readable by the GPU (device memory or the device alias of mapped host memory).
+ * Asynchronous; zero-length descriptors are skipped; destination ranges must not overlap each other.
+ * Stands in for the consumer the reference feeds, NCCL's ncclNetDeviceUnpack (not part of the reference
+ * tree; selected at CMakeLists.txt:77-89), for one slot's descriptor list (src/net_tcpx.cc:1128-1130,1354). */
+int tcpxuUnpackBatch(int device, const void* bounce_base, void* dst_base, const tcpxuLoadMeta* descs,
+                     uint64_t n_descs, void* stream);
+
+/* Same launch bracketed by HIP events on its stream, repeated `iters` times after `warmup` untimed ones;
+ * writes the mean duration of one launch in microseconds.  Measurement helper for benchmarks: the events
+ * sit on the stream the kernel is launched on. */
+int tcpxuUnpackBatchTimed(int device, const void* bounce_base, void* dst_base, const tcpxuLoadMeta* descs,
+                          uint64_t n_descs, int warmup, int iters, double* mean_us);
+
+/* Plain device-to-device copy kernel of `bytes` (multiple of 16), timed the same way: the achievable-copy
+ * yardstick printed beside the unpack figure, and the known-size kernel used to calibrate HBM counters. */
+int tcpxuCopyKernelTimed(int device, void* dst, const void* src, size_t bytes, int warmup, int iters,
+                         double* mean_us);
+
+/* ---- (4) persistent unpack engine -------------------------------------------------------------------- */
+
+/* One engine per GPU: a persistent kernel that polls a submission ring in mapped host memory, unpacks every
+ * submitted slot and writes a completion word back to mapped host memory -- no kernel launch per request.
+ * It takes the place of the NCCL collective kernel that runs ncclNetDeviceUnpack and of the head counter in
+ * `struct unpackNetDeviceHandle` (src/devcomm/nccl/unpack1.cu:53-63). */
+typedef struct tcpxuEngine tcpxuEngine;
+
+typedef struct tcpxuEngineConfig {
+  uint32_t ring_entries;    /* submission ring size, power of two, 0 = default (1024) */
+  uint32_t workgroups;      /* persistent grid size, 0 = fill the GPU */
+  uint32_t descs_per_ticket;/* descriptors one workgroup takes at a time, 0 = default */
+  uint32_t spin_limit;      /* 0 = poll until stopped; otherwise the kernel exits by itself after this many
+                               empty polls of the ring (a bounded wait, for tests of the timeout path) */
+} tcpxuEngineConfig;
+
+int tcpxuEngineCreate(int device, const tcpxuEngineConfig* config, tcpxuEngine** engine);
+/* Launches the persistent kernel.  The engine can be started and stopped repeatedly. */
+int tcpxuEngineStart(tcpxuEngine* engine);
+/* Asks the kernel to drain and exit, waits for it, and reports the duration of that launch in
+ * microseconds as measured by HIP events on the engine's stream (elapsed_us may be NULL). */
+int tcpxuEngineStop(tcpxuEngine* engine, double* elapsed_us);
+int tcpxuEngineDestroy(tcpxuEngine* engine);
+
+/* Publishes one slot: `n_descs` descriptors at `descs_dev` (device-visible address, normally the device
+ * alias of a slot of the mapped queue), gathered from `bounce_base` into `dst_base`.  When the GPU has
+ * written every byte it stores `done_value` (nonzero) to `*done_flag_dev` (device alias of a mapped 8-byte
+ * word that the host poller reads).  Returns TCPXU_IN_PROGRESS if the ring is full (caller retries).
+ * This is the publish of src/net_tcpx.cc:1354-1357 made explicit: count, then a release, then the tail. */
+int tcpxuEngineSubmit(tcpxuEngine* engine, const void* bounce_base, void* dst_base, const void* descs_dev,
+                      uint32_t n_descs, void* done_flag_dev, uint64_t done_value);
+
+/* Number of submissions the GPU has fully completed since creation (monotone; read from mapped memory). */
+int tcpxuEngineCompleted(tcpxuEngine* engine, uint64_t* completed);
+
+/* 1 if the persistent kernel is running, 0 if stopped or exited by its spin limit. */
+int tcpxuEngineRunning(tcpxuEngine* engine, int* running);
+
+/* ---- streaming driver (measurement helper) ------------------------------------------------------------ */
+
+/* One slot's worth of work for tcpxuEngineStream. */
+typedef struct tcpxuStreamItem {
+  const void* bounce_base;
+  void* dst_base;
+  const tcpxuLoadMeta* descs_host; /* descriptors in ordinary host memory */
+  uint32_t n_descs;                /* at most TCPXU_SLOT_PAGES */
+  uint32_t reserved;
+} tcpxuStreamItem;
+
+/* Drives a started engine the way the plugin's proxy loop does, from one host thread, with no Python in the
+ * loop: a mapped ring of `depth` slots (1..TCPXU_QUEUE_DEPTH) of TCPXU_SLOT_PAGES descriptors each; for every
+ * item, in order: wait until the slot's previous occupant has completed, copy the item's descriptors into the
+ * slot (the memcpy of src/net_tcpx.cc:1128-1130), publish it (src/net_tcpx.cc:1354-1357), and poll completion
+ * words in FIFO order (the tcpxTest / tcpxIrecvConsumed cadence).  Writes the wall time from the first publish
+ * to the last completion to *wall_us and, if latency_us is not NULL, each item's publish-to-completion-seen
+ * time in microseconds to latency_us[0..n_items).  Returns TCPXU_INTERNAL_ERROR if nothing completes for
+ * `stall_timeout_ms` milliseconds. */
+int tcpxuEngineStream(tcpxuEngine* engine, const tcpxuStreamItem* items, uint64_t n_items, uint32_t depth,
+                      uint32_t stall_timeout_ms, double* wall_us, double* latency_us);
+
+/* tcpxuEngineStart + tcpxuEngineStream + tcpxuEngineStop in one call on a stopped engine, so that the
+ * persistent kernel's launch covers exactly these items; *kernel_us is that launch's duration from HIP events
+ * on the engine's stream (the figure a kernel trace shows for it). */
+int tcpxuEngineRunTimed(tcpxuEngine* engine, const tcpxuStreamItem* items, uint64_t n_items, uint32_t depth,
+                        uint32_t stall_timeout_ms, double* wall_us, double* kernel_us, double* latency_us);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TCPX_UNPACK_HIP_H_ */

@@ -1,0 +1,294 @@
+"""MI355X-native receive-side unpack path of a GPUDirect-TCPX style net plugin: ctypes view of the C-ABI.
+
+This package holds no compute of its own.  It loads the in-tree shared libraries built from ``csrc/`` and
+exposes their C entry points (``include/tcpx_unpack_hip.h``, ``include/tcpx_synth.h``,
+``include/tcpx_plugin.h``) with argument types attached, so tests and the benchmark call exactly what a C or
+C++ host would call.  There is no CPU fallback: if a library is missing, loading raises.
+
+The directory name carries a hyphen, so it is imported through ``__graft_entry__.load_package()`` under the
+module name ``nccl_plugin_gpudirecttcpx_amd``.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_DIR = os.path.join(_HERE, "lib")
+REPO_ROOT = os.path.dirname(_HERE)
+
+SUCCESS, DEVICE_ERROR, SYSTEM_ERROR, INTERNAL_ERROR, INVALID_ARGUMENT, INVALID_USAGE = 0, 1, 2, 3, 4, 5
+IN_PROGRESS = 7
+
+QUEUE_DEPTH = 16
+SLOT_PAGES = 2048
+PAGE_SIZE = 4096
+
+c_u8p = ctypes.POINTER(ctypes.c_uint8)
+
+
+class LoadMeta(ctypes.Structure):
+    """``tcpxuLoadMeta`` / NCCL ``union loadMeta`` (reference fields: src/sock/tcpx.h:178-180)."""
+
+    _fields_ = [("src_off", ctypes.c_uint32), ("len", ctypes.c_uint32), ("dst_off", ctypes.c_uint64)]
+
+
+class SynthFrag(ctypes.Structure):
+    _fields_ = [
+        ("frag_offset", ctypes.c_uint32),
+        ("frag_size", ctypes.c_uint32),
+        ("frag_token", ctypes.c_uint32),
+        ("flow", ctypes.c_uint32),
+    ]
+
+
+class SynthRequest(ctypes.Structure):
+    _fields_ = [
+        ("first_desc", ctypes.c_uint64),
+        ("dst_off", ctypes.c_uint64),
+        ("n_descs", ctypes.c_uint32),
+        ("bytes", ctypes.c_uint32),
+        ("window", ctypes.c_uint32),
+        ("reserved", ctypes.c_uint32),
+    ]
+
+
+class SynthInfo(ctypes.Structure):
+    _fields_ = [
+        ("pool_bytes", ctypes.c_uint64),
+        ("payload_bytes", ctypes.c_uint64),
+        ("dst_bytes", ctypes.c_uint64),
+        ("n_descs", ctypes.c_uint64),
+        ("n_requests", ctypes.c_uint32),
+        ("n_flows", ctypes.c_uint32),
+        ("n_windows", ctypes.c_uint32),
+        ("dst_misalign", ctypes.c_uint32),
+    ]
+
+
+class EngineConfig(ctypes.Structure):
+    _fields_ = [
+        ("ring_entries", ctypes.c_uint32),
+        ("workgroups", ctypes.c_uint32),
+        ("descs_per_ticket", ctypes.c_uint32),
+        ("spin_limit", ctypes.c_uint32),
+    ]
+
+
+class StreamItem(ctypes.Structure):
+    _fields_ = [
+        ("bounce_base", ctypes.c_void_p),
+        ("dst_base", ctypes.c_void_p),
+        ("descs_host", ctypes.c_void_p),
+        ("n_descs", ctypes.c_uint32),
+        ("reserved", ctypes.c_uint32),
+    ]
+
+
+class MissingLibrary(RuntimeError):
+    pass
+
+
+def _load(name):
+    path = os.path.join(LIB_DIR, name)
+    if not os.path.exists(path):
+        raise MissingLibrary(
+            "%s is not built: run `python -c 'import __graft_entry__ as g; g.build()'` in %s" % (path, REPO_ROOT)
+        )
+    return ctypes.CDLL(path, mode=ctypes.RTLD_GLOBAL)
+
+
+_HIP_PROTOTYPES = {
+    # name: (restype, argtypes)
+    "tcpxuLastError": (ctypes.c_char_p, []),
+    "tcpxuDeviceCount": (ctypes.c_int, [ctypes.POINTER(ctypes.c_int)]),
+    "tcpxuDeviceInfo": (ctypes.c_int, [ctypes.c_int, ctypes.c_char_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_int)]),
+    "tcpxuArenaCreate": (ctypes.c_int, [ctypes.c_int, ctypes.c_size_t, ctypes.POINTER(ctypes.c_void_p)]),
+    "tcpxuArenaDestroy": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p]),
+    "tcpxuDeviceAlloc": (ctypes.c_int, [ctypes.c_int, ctypes.c_size_t, ctypes.POINTER(ctypes.c_void_p)]),
+    "tcpxuDeviceFree": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p]),
+    "tcpxuCopyToDevice": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]),
+    "tcpxuCopyToHost": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]),
+    "tcpxuFillDevice": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t]),
+    "tcpxuDeviceSynchronize": (ctypes.c_int, [ctypes.c_int]),
+    "tcpxuMappedAlloc": (
+        ctypes.c_int,
+        [ctypes.c_int, ctypes.c_size_t, ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_void_p)],
+    ),
+    "tcpxuMappedFree": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p]),
+    "tcpxuUnpackBatch": (
+        ctypes.c_int,
+        [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p],
+    ),
+    "tcpxuUnpackBatchTimed": (
+        ctypes.c_int,
+        [
+            ctypes.c_int,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.c_uint64,
+            ctypes.c_int,
+            ctypes.c_int,
+            ctypes.POINTER(ctypes.c_double),
+        ],
+    ),
+    "tcpxuCopyKernelTimed": (
+        ctypes.c_int,
+        [
+            ctypes.c_int,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.c_size_t,
+            ctypes.c_int,
+            ctypes.c_int,
+            ctypes.POINTER(ctypes.c_double),
+        ],
+    ),
+    "tcpxuEngineCreate": (
+        ctypes.c_int,
+        [ctypes.c_int, ctypes.POINTER(EngineConfig), ctypes.POINTER(ctypes.c_void_p)],
+    ),
+    "tcpxuEngineStart": (ctypes.c_int, [ctypes.c_void_p]),
+    "tcpxuEngineStop": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_double)]),
+    "tcpxuEngineDestroy": (ctypes.c_int, [ctypes.c_void_p]),
+    "tcpxuEngineSubmit": (
+        ctypes.c_int,
+        [
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.c_uint32,
+            ctypes.c_void_p,
+            ctypes.c_uint64,
+        ],
+    ),
+    "tcpxuEngineCompleted": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint64)]),
+    "tcpxuEngineRunning": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]),
+    "tcpxuEngineStream": (
+        ctypes.c_int,
+        [
+            ctypes.c_void_p,
+            ctypes.POINTER(StreamItem),
+            ctypes.c_uint64,
+            ctypes.c_uint32,
+            ctypes.c_uint32,
+            ctypes.POINTER(ctypes.c_double),
+            ctypes.POINTER(ctypes.c_double),
+        ],
+    ),
+    "tcpxuEngineRunTimed": (
+        ctypes.c_int,
+        [
+            ctypes.c_void_p,
+            ctypes.POINTER(StreamItem),
+            ctypes.c_uint64,
+            ctypes.c_uint32,
+            ctypes.c_uint32,
+            ctypes.POINTER(ctypes.c_double),
+            ctypes.POINTER(ctypes.c_double),
+            ctypes.POINTER(ctypes.c_double),
+        ],
+    ),
+}
+
+_SYNTH_PROTOTYPES = {
+    "tcpxSynthCreate": (
+        ctypes.c_int,
+        [ctypes.c_int, ctypes.c_uint64, ctypes.c_uint32, ctypes.POINTER(ctypes.c_void_p)],
+    ),
+    "tcpxSynthDestroy": (None, [ctypes.c_void_p]),
+    "tcpxSynthGetInfo": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(SynthInfo)]),
+    "tcpxSynthDescs": (ctypes.POINTER(LoadMeta), [ctypes.c_void_p]),
+    "tcpxSynthFrags": (ctypes.POINTER(SynthFrag), [ctypes.c_void_p]),
+    "tcpxSynthRequests": (ctypes.POINTER(SynthRequest), [ctypes.c_void_p]),
+    "tcpxSynthFillWindow": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_uint32, ctypes.c_void_p]),
+}
+
+
+def _bind(lib, prototypes):
+    for name, (restype, argtypes) in prototypes.items():
+        fn = getattr(lib, name)  # AttributeError if the library does not export it
+        fn.restype = restype
+        fn.argtypes = argtypes
+    return lib
+
+
+_cache = {}
+
+
+def hip_layer():
+    """``libtcpxu_hip.so`` with prototypes attached.  Loading does not need a GPU; calling does."""
+    if "hip" not in _cache:
+        _cache["hip"] = _bind(_load("libtcpxu_hip.so"), _HIP_PROTOTYPES)
+    return _cache["hip"]
+
+
+def synth_lib():
+    if "synth" not in _cache:
+        _cache["synth"] = _bind(_load("libtcpx_synth.so"), _SYNTH_PROTOTYPES)
+    return _cache["synth"]
+
+
+class HipError(RuntimeError):
+    def __init__(self, fn, rc, msg):
+        super().__init__("%s failed with result %d: %s" % (fn, rc, msg))
+        self.rc = rc
+
+
+def check(rc, fn="call"):
+    if rc != SUCCESS:
+        raise HipError(fn, rc, hip_layer().tcpxuLastError().decode(errors="replace"))
+
+
+class Workload:
+    """A generated workload (numpy views into memory owned by the C object)."""
+
+    def __init__(self, config, seed=0xC0FFEE00, shrink=0):
+        import numpy as np
+
+        self._lib = synth_lib()
+        handle = ctypes.c_void_p()
+        rc = self._lib.tcpxSynthCreate(config, seed, shrink, ctypes.byref(handle))
+        if rc != 0:
+            raise ValueError("tcpxSynthCreate(config=%r, shrink=%r) -> %d" % (config, shrink, rc))
+        self._h = handle
+        self.config, self.seed, self.shrink = config, seed, shrink
+        self.info = SynthInfo()
+        self._lib.tcpxSynthGetInfo(self._h, ctypes.byref(self.info))
+        n = self.info.n_descs
+        self.desc_dtype = np.dtype([("src_off", "<u4"), ("len", "<u4"), ("dst_off", "<u8")])
+        self.frag_dtype = np.dtype([("frag_offset", "<u4"), ("frag_size", "<u4"), ("frag_token", "<u4"), ("flow", "<u4")])
+        self.req_dtype = np.dtype(
+            [("first_desc", "<u8"), ("dst_off", "<u8"), ("n_descs", "<u4"), ("bytes", "<u4"), ("window", "<u4"), ("reserved", "<u4")]
+        )
+        self.descs = self._view(self._lib.tcpxSynthDescs(self._h), n, self.desc_dtype)
+        self.frags = self._view(self._lib.tcpxSynthFrags(self._h), n, self.frag_dtype)
+        self.requests = self._view(self._lib.tcpxSynthRequests(self._h), self.info.n_requests, self.req_dtype)
+
+    @staticmethod
+    def _view(ptr, n, dtype):
+        import numpy as np
+
+        if n == 0:
+            return np.zeros(0, dtype=dtype)
+        buf = (ctypes.c_uint8 * (n * dtype.itemsize)).from_address(ctypes.addressof(ptr.contents))
+        return np.frombuffer(buf, dtype=dtype)
+
+    def fill_window(self, window, pool):
+        """Writes pool generation `window` into the numpy uint8 array `pool` (length pool_bytes)."""
+        assert pool.nbytes == self.info.pool_bytes and pool.flags["C_CONTIGUOUS"]
+        rc = self._lib.tcpxSynthFillWindow(self._h, window, pool.ctypes.data_as(ctypes.c_void_p))
+        if rc != 0:
+            raise ValueError("tcpxSynthFillWindow -> %d" % rc)
+
+    def close(self):
+        if self._h:
+            self.descs = self.frags = self.requests = None
+            self._lib.tcpxSynthDestroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

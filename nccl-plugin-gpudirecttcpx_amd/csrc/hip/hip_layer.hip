@@ -1,0 +1,375 @@
+// HIP layer of the receive-side unpack path: device selection, the bounce-page arena, mapped queue memory and
+// the launch-per-batch unpack kernel, all behind the C-ABI of include/tcpx_unpack_hip.h.
+// The persistent engine lives in engine.hip.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "hip_common.h"
+#include "tcpx_unpack_hip.h"
+#include "unpack_device.h"
+
+namespace tcpxu {
+
+thread_local char g_last_error[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof g_last_error, fmt, ap);
+  va_end(ap);
+}
+
+namespace {
+
+constexpr uint32_t kMaxDescsPerWg = 64;
+
+// Launch-per-batch unpack.  A workgroup takes `descs_per_wg` consecutive descriptors, stages them in LDS with
+// one 16-byte load per thread, then its four wavefronts take fragments in turn.
+__global__ __launch_bounds__(kWgThreads) void unpack_batch_kernel(const uint8_t* __restrict__ bounce,
+                                                                   uint8_t* __restrict__ dst,
+                                                                   const tcpxuLoadMeta* __restrict__ descs,
+                                                                   uint64_t n_descs, uint32_t descs_per_wg,
+                                                                   uint64_t n_batches) {
+  __shared__ tcpxuLoadMeta staged[kMaxDescsPerWg];
+  const uint32_t tid = threadIdx.x;
+  const uint32_t lane = tid & (kWaveLanes - 1);
+  const uint32_t wave = tid / kWaveLanes;
+
+  for (uint64_t wg = blockIdx.x;; wg += gridDim.x) {
+    const uint64_t per_xcd = (n_batches + 7) / 8;
+    if (wg >= per_xcd * 8) break;
+    const uint64_t batch = xcd_contiguous_index(wg, n_batches);
+    if (batch < n_batches) {  // block-uniform
+      const uint64_t first = batch * descs_per_wg;
+      const uint32_t cnt = static_cast<uint32_t>(std::min<uint64_t>(descs_per_wg, n_descs - first));
+      if (tid < cnt) {
+        const u32x4 raw = *reinterpret_cast<const u32x4*>(descs + first + tid);
+        *reinterpret_cast<u32x4*>(&staged[tid]) = raw;
+      }
+      __syncthreads();
+      for (uint32_t j = wave; j < cnt; j += kWavesPerWg) {
+        const tcpxuLoadMeta d = staged[j];
+        const uint32_t len = __builtin_amdgcn_readfirstlane(d.len);
+        const uint32_t so = __builtin_amdgcn_readfirstlane(d.src_off);
+        const uint32_t dlo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(d.dst_off));
+        const uint32_t dhi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(d.dst_off >> 32));
+        const uint64_t doff = (static_cast<uint64_t>(dhi) << 32) | dlo;
+        wave_copy_fragment(bounce + so, dst + doff, len, lane);
+      }
+      __syncthreads();
+    }
+  }
+}
+
+// Plain streaming copy, 64 bytes per thread per step: the yardstick for what a copy kernel reaches here.
+__global__ __launch_bounds__(kWgThreads) void copy_kernel(uint8_t* __restrict__ dst, const uint8_t* __restrict__ src,
+                                                          uint64_t n_vec) {
+  const uint64_t stride = static_cast<uint64_t>(gridDim.x) * kWgThreads;
+  for (uint64_t base = static_cast<uint64_t>(blockIdx.x) * kWgThreads * kVecPerLane; base < n_vec;
+       base += stride * kVecPerLane) {
+    u32x4 r[kVecPerLane];
+#pragma unroll
+    for (int k = 0; k < kVecPerLane; ++k) {
+      const uint64_t v = base + static_cast<uint64_t>(k) * kWgThreads + threadIdx.x;
+      if (v < n_vec) r[k] = load_vec(src + (v << 4));
+    }
+#pragma unroll
+    for (int k = 0; k < kVecPerLane; ++k) {
+      const uint64_t v = base + static_cast<uint64_t>(k) * kWgThreads + threadIdx.x;
+      if (v < n_vec) store_vec(dst + (v << 4), r[k]);
+    }
+  }
+}
+
+struct DeviceProps {
+  bool valid = false;
+  int compute_units = 0;
+  char name[256] = "";
+};
+DeviceProps g_props[kMaxDevices];
+
+int env_int(const char* name, int fallback) {
+  const char* v = getenv(name);
+  if (!v || !*v) return fallback;
+  return atoi(v);
+}
+
+}  // namespace
+
+int use_device(int device) {
+  if (device < 0 || device >= kMaxDevices) {
+    set_error("device index %d out of range", device);
+    return TCPXU_INVALID_ARGUMENT;
+  }
+  TCPXU_HIP(hipSetDevice(device));
+  if (!g_props[device].valid) {
+    hipDeviceProp_t p;
+    TCPXU_HIP(hipGetDeviceProperties(&p, device));
+    g_props[device].compute_units = p.multiProcessorCount;
+    snprintf(g_props[device].name, sizeof g_props[device].name, "%s (%s)", p.name, p.gcnArchName);
+    g_props[device].valid = true;
+  }
+  return TCPXU_SUCCESS;
+}
+
+int device_compute_units(int device) { return g_props[device].compute_units; }
+
+// Grid geometry of the launch-per-batch kernel: enough descriptors per workgroup to amortise the staging
+// barrier, few enough that a small slot still spreads over the whole GPU.
+void batch_geometry(int device, uint64_t n_descs, uint32_t* descs_per_wg, uint64_t* n_batches, uint32_t* grid) {
+  const uint64_t cus = static_cast<uint64_t>(std::max(1, g_props[device].compute_units));
+  uint32_t dpw = static_cast<uint32_t>(env_int("TCPXU_DESCS_PER_WG", 0));
+  if (dpw == 0) {
+    // Aim for about 8 workgroups per compute unit; between one and four fragments per wavefront.
+    const uint64_t want_wgs = cus * 8;
+    const uint64_t d = (n_descs + want_wgs - 1) / want_wgs;
+    dpw = d <= 4 ? 4 : d <= 8 ? 8 : 16;
+  }
+  dpw = std::min(std::max(dpw, 1u), kMaxDescsPerWg);
+  const uint64_t batches = (n_descs + dpw - 1) / dpw;
+  const uint64_t per_xcd = (batches + 7) / 8;
+  const uint64_t max_grid = cus * 16;
+  *descs_per_wg = dpw;
+  *n_batches = batches;
+  *grid = static_cast<uint32_t>(std::min<uint64_t>(per_xcd * 8, std::max<uint64_t>(max_grid, 8)));
+}
+
+}  // namespace tcpxu
+
+using namespace tcpxu;
+
+extern "C" {
+
+const char* tcpxuLastError(void) { return g_last_error; }
+
+int tcpxuDeviceCount(int* count) {
+  if (!count) return TCPXU_INVALID_ARGUMENT;
+  *count = 0;
+  TCPXU_HIP(hipGetDeviceCount(count));
+  return TCPXU_SUCCESS;
+}
+
+int tcpxuDeviceInfo(int device, char* name, size_t name_len, int* compute_units) {
+  TCPXU_TRY(use_device(device));
+  if (name && name_len) snprintf(name, name_len, "%s", g_props[device].name);
+  if (compute_units) *compute_units = g_props[device].compute_units;
+  return TCPXU_SUCCESS;
+}
+
+int tcpxuArenaCreate(int device, size_t bytes, void** arena_base) {
+  if (!arena_base || bytes == 0 || bytes % TCPXU_PAGE_SIZE != 0) {
+    set_error("arena size %zu must be a positive multiple of %d", bytes, TCPXU_PAGE_SIZE);
+    return TCPXU_INVALID_ARGUMENT;
+  }
+  if (bytes > (1ull << 32)) {
+    set_error("arena size %zu exceeds the 4 GiB reach of a 32-bit src_off", bytes);
+    return TCPXU_INVALID_ARGUMENT;
+  }
+  TCPXU_TRY(use_device(device));
+  TCPXU_HIP(hipMalloc(arena_base, bytes));
+  if (reinterpret_cast<uintptr_t>(*arena_base) % TCPXU_PAGE_SIZE != 0) {
+    (void)hipFree(*arena_base);
+    *arena_base = nullptr;
+    set_error("arena base is not page aligned");
+    return TCPXU_INTERNAL_ERROR;
+  }
+  return TCPXU_SUCCESS;
+}
+
+int tcpxuArenaDestroy(int device, void* arena_base) {
+  TCPXU_TRY(use_device(device));
+  TCPXU_HIP(hipFree(arena_base));
+  return TCPXU_SUCCESS;
+}
+
+int tcpxuDeviceAlloc(int device, size_t bytes, void** ptr) {
+  if (!ptr || bytes == 0) return TCPXU_INVALID_ARGUMENT;
+  TCPXU_TRY(use_device(device));
+  TCPXU_HIP(hipMalloc(ptr, bytes));
+  return TCPXU_SUCCESS;
+}
+
+int tcpxuDeviceFree(int device, void* ptr) {
+  TCPXU_TRY(use_device(device));
+  TCPXU_HIP(hipFree(ptr));
+  return TCPXU_SUCCESS;
+}
+
+int tcpxuCopyToDevice(int device, void* dst_dev, const void* src_host, size_t bytes) {
+  TCPXU_TRY(use_device(device));
+  TCPXU_HIP(hipMemcpy(dst_dev, src_host, bytes, hipMemcpyHostToDevice));
+  return TCPXU_SUCCESS;
+}
+
+int tcpxuCopyToHost(int device, void* dst_host, const void* src_dev, size_t bytes) {
+  TCPXU_TRY(use_device(device));
+  TCPXU_HIP(hipMemcpy(dst_host, src_dev, bytes, hipMemcpyDeviceToHost));
+  return TCPXU_SUCCESS;
+}
+
+int tcpxuFillDevice(int device, void* dst_dev, int byte_value, size_t bytes) {
+  TCPXU_TRY(use_device(device));
+  TCPXU_HIP(hipMemset(dst_dev, byte_value, bytes));
+  TCPXU_HIP(hipDeviceSynchronize());
+  return TCPXU_SUCCESS;
+}
+
+int tcpxuDeviceSynchronize(int device) {
+  TCPXU_TRY(use_device(device));
+  TCPXU_HIP(hipDeviceSynchronize());
+  return TCPXU_SUCCESS;
+}
+
+int tcpxuMappedAlloc(int device, size_t bytes, void** host_ptr, void** dev_ptr) {
+  if (!host_ptr || !dev_ptr || bytes == 0) return TCPXU_INVALID_ARGUMENT;
+  TCPXU_TRY(use_device(device));
+  TCPXU_HIP(hipHostMalloc(host_ptr, bytes, hipHostMallocMapped | hipHostMallocCoherent | hipHostMallocPortable));
+  memset(*host_ptr, 0, bytes);
+  TCPXU_HIP(hipHostGetDevicePointer(dev_ptr, *host_ptr, 0));
+  return TCPXU_SUCCESS;
+}
+
+int tcpxuMappedFree(int device, void* host_ptr) {
+  TCPXU_TRY(use_device(device));
+  TCPXU_HIP(hipHostFree(host_ptr));
+  return TCPXU_SUCCESS;
+}
+
+static int launch_batch(int device, const void* bounce_base, void* dst_base, const tcpxuLoadMeta* descs,
+                        uint64_t n_descs, hipStream_t stream) {
+  if (n_descs == 0) return TCPXU_SUCCESS;
+  if (!bounce_base || !dst_base || !descs) {
+    set_error("null pointer passed to unpack");
+    return TCPXU_INVALID_ARGUMENT;
+  }
+  if (reinterpret_cast<uintptr_t>(descs) % 16 != 0) {
+    set_error("descriptor array must be 16-byte aligned");
+    return TCPXU_INVALID_ARGUMENT;
+  }
+  uint32_t dpw, grid;
+  uint64_t batches;
+  batch_geometry(device, n_descs, &dpw, &batches, &grid);
+  hipLaunchKernelGGL(unpack_batch_kernel, dim3(grid), dim3(kWgThreads), 0, stream,
+                     static_cast<const uint8_t*>(bounce_base), static_cast<uint8_t*>(dst_base), descs, n_descs, dpw,
+                     batches);
+  TCPXU_HIP(hipGetLastError());
+  return TCPXU_SUCCESS;
+}
+
+int tcpxuUnpackBatch(int device, const void* bounce_base, void* dst_base, const tcpxuLoadMeta* descs,
+                     uint64_t n_descs, void* stream) {
+  TCPXU_TRY(use_device(device));
+  return launch_batch(device, bounce_base, dst_base, descs, n_descs, static_cast<hipStream_t>(stream));
+}
+
+// Mean of per-launch durations: every launch sits between its own pair of events on the launch stream, so
+// gaps between launches are not counted.
+static int time_launches(hipStream_t stream, int warmup, int iters, double* mean_us, int (*launch)(void*, hipStream_t),
+                         void* ctx) {
+  std::vector<hipEvent_t> ev(static_cast<size_t>(iters) * 2, nullptr);
+  int rc = TCPXU_SUCCESS;
+  for (int i = 0; i < warmup && rc == TCPXU_SUCCESS; ++i) rc = launch(ctx, stream);
+  for (auto& e : ev) {
+    if (rc == TCPXU_SUCCESS && hipEventCreate(&e) != hipSuccess) {
+      set_error("hipEventCreate failed");
+      rc = TCPXU_DEVICE_ERROR;
+    }
+  }
+  if (rc == TCPXU_SUCCESS && hipStreamSynchronize(stream) != hipSuccess) rc = TCPXU_DEVICE_ERROR;
+  for (int i = 0; i < iters && rc == TCPXU_SUCCESS; ++i) {
+    if (hipEventRecord(ev[2 * i], stream) != hipSuccess) rc = TCPXU_DEVICE_ERROR;
+    if (rc == TCPXU_SUCCESS) rc = launch(ctx, stream);
+    if (rc == TCPXU_SUCCESS && hipEventRecord(ev[2 * i + 1], stream) != hipSuccess) rc = TCPXU_DEVICE_ERROR;
+  }
+  if (rc == TCPXU_SUCCESS) {
+    hipError_t e = hipStreamSynchronize(stream);
+    if (e != hipSuccess) {
+      set_error("stream synchronize failed: %s", hipGetErrorString(e));
+      rc = TCPXU_DEVICE_ERROR;
+    }
+  }
+  if (rc == TCPXU_SUCCESS) {
+    double total_ms = 0.0;
+    for (int i = 0; i < iters; ++i) {
+      float ms = 0.f;
+      if (hipEventElapsedTime(&ms, ev[2 * i], ev[2 * i + 1]) != hipSuccess) rc = TCPXU_DEVICE_ERROR;
+      total_ms += ms;
+    }
+    *mean_us = total_ms * 1000.0 / iters;
+  }
+  for (auto e : ev)
+    if (e) (void)hipEventDestroy(e);
+  return rc;
+}
+
+struct BatchLaunch {
+  int device;
+  const void* bounce;
+  void* dst;
+  const tcpxuLoadMeta* descs;
+  uint64_t n;
+};
+
+int tcpxuUnpackBatchTimed(int device, const void* bounce_base, void* dst_base, const tcpxuLoadMeta* descs,
+                          uint64_t n_descs, int warmup, int iters, double* mean_us) {
+  if (!mean_us || iters <= 0 || warmup < 0 || n_descs == 0) return TCPXU_INVALID_ARGUMENT;
+  TCPXU_TRY(use_device(device));
+  hipStream_t stream;
+  TCPXU_HIP(hipStreamCreate(&stream));
+  BatchLaunch b{device, bounce_base, dst_base, descs, n_descs};
+  int rc = time_launches(
+      stream, warmup, iters, mean_us,
+      [](void* c, hipStream_t s) {
+        auto* b = static_cast<BatchLaunch*>(c);
+        return launch_batch(b->device, b->bounce, b->dst, b->descs, b->n, s);
+      },
+      &b);
+  (void)hipStreamDestroy(stream);
+  return rc;
+}
+
+struct CopyLaunch {
+  uint8_t* dst;
+  const uint8_t* src;
+  uint64_t n_vec;
+  uint32_t grid;
+};
+
+int tcpxuCopyKernelTimed(int device, void* dst, const void* src, size_t bytes, int warmup, int iters,
+                         double* mean_us) {
+  if (!mean_us || iters <= 0 || warmup < 0 || !dst || !src || bytes == 0 || bytes % 16 != 0 ||
+      reinterpret_cast<uintptr_t>(dst) % 16 != 0 || reinterpret_cast<uintptr_t>(src) % 16 != 0) {
+    set_error("copy kernel needs 16-byte aligned buffers and a size that is a multiple of 16");
+    return TCPXU_INVALID_ARGUMENT;
+  }
+  TCPXU_TRY(use_device(device));
+  const uint64_t n_vec = bytes / 16;
+  const uint64_t per_wg = static_cast<uint64_t>(kWgThreads) * kVecPerLane;
+  const uint64_t cus = static_cast<uint64_t>(std::max(1, device_compute_units(device)));
+  const uint32_t grid = static_cast<uint32_t>(std::min<uint64_t>((n_vec + per_wg - 1) / per_wg, cus * 16));
+  hipStream_t stream;
+  TCPXU_HIP(hipStreamCreate(&stream));
+  CopyLaunch c{static_cast<uint8_t*>(dst), static_cast<const uint8_t*>(src), n_vec, grid};
+  int rc = time_launches(
+      stream, warmup, iters, mean_us,
+      [](void* p, hipStream_t s) {
+        auto* c = static_cast<CopyLaunch*>(p);
+        hipLaunchKernelGGL(copy_kernel, dim3(c->grid), dim3(kWgThreads), 0, s, c->dst, c->src, c->n_vec);
+        if (hipGetLastError() != hipSuccess) {
+          set_error("copy kernel launch failed");
+          return TCPXU_DEVICE_ERROR;
+        }
+        return TCPXU_SUCCESS;
+      },
+      &c);
+  (void)hipStreamDestroy(stream);
+  return rc;
+}
+
+}  // extern "C"

@@ -1,0 +1,225 @@
+"""GPU parity of the persistent unpack engine against the CPU oracle, byte-exact, through the C-ABI.
+
+Descriptors and completion words live in hipHostMalloc-mapped memory; the destination is read back while the
+engine kernel is still running wherever the test says so, which is what a real consumer does.
+Every wait in this file has a deadline, so a stuck engine fails a test instead of hanging the run.
+"""
+import ctypes
+import time
+
+import numpy as np
+import pytest
+
+from conftest import GUARD, SENTINEL, GpuBuffers, first_difference, make_descs, oracle_expected
+
+pytestmark = pytest.mark.gpu
+
+
+class Mapped:
+    """A block of mapped host memory: [0, 8*n_flags) completion words, then descriptors."""
+
+    def __init__(self, pkg, hip, descs, n_flags):
+        self.pkg, self.hip = pkg, hip
+        self.flag_bytes = (8 * n_flags + 63) // 64 * 64
+        self.host, self.dev = ctypes.c_void_p(), ctypes.c_void_p()
+        nbytes = self.flag_bytes + max(descs.nbytes, 16)
+        pkg.check(hip.tcpxuMappedAlloc(0, nbytes, ctypes.byref(self.host), ctypes.byref(self.dev)), "tcpxuMappedAlloc")
+        if descs.nbytes:
+            ctypes.memmove(self.host.value + self.flag_bytes, descs.ctypes.data, descs.nbytes)
+        self.flags = (ctypes.c_uint64 * n_flags).from_address(self.host.value)
+
+    def desc_dev(self, index):
+        return self.dev.value + self.flag_bytes + 16 * index
+
+    def flag_dev(self, i):
+        return self.dev.value + 8 * i
+
+    def wait(self, i, value, seconds=20.0):
+        deadline = time.time() + seconds
+        while self.flags[i] != value:
+            if time.time() > deadline:
+                raise TimeoutError("completion word %d did not reach %d (is %d)" % (i, value, self.flags[i]))
+
+    def free(self):
+        self.pkg.check(self.hip.tcpxuMappedFree(0, self.host), "tcpxuMappedFree")
+
+
+class Engine:
+    def __init__(self, pkg, hip, **cfg):
+        self.pkg, self.hip = pkg, hip
+        self.h = ctypes.c_void_p()
+        c = pkg.EngineConfig(
+            cfg.get("ring_entries", 0), cfg.get("workgroups", 0), cfg.get("descs_per_ticket", 0), cfg.get("spin_limit", 0)
+        )
+        pkg.check(hip.tcpxuEngineCreate(0, ctypes.byref(c), ctypes.byref(self.h)), "tcpxuEngineCreate")
+        self.started = False
+
+    def start(self):
+        self.pkg.check(self.hip.tcpxuEngineStart(self.h), "tcpxuEngineStart")
+        self.started = True
+
+    def stop(self):
+        us = ctypes.c_double()
+        self.started = False
+        self.pkg.check(self.hip.tcpxuEngineStop(self.h, ctypes.byref(us)), "tcpxuEngineStop")
+        return us.value
+
+    def submit(self, bounce, dst, descs_dev, n, flag_dev, value, seconds=20.0):
+        deadline = time.time() + seconds
+        while True:
+            rc = self.hip.tcpxuEngineSubmit(self.h, bounce, dst, descs_dev, n, flag_dev, value)
+            if rc != self.pkg.IN_PROGRESS:
+                self.pkg.check(rc, "tcpxuEngineSubmit")
+                return
+            if time.time() > deadline:
+                raise TimeoutError("submission ring stayed full")
+
+    def completed(self):
+        c = ctypes.c_uint64()
+        self.pkg.check(self.hip.tcpxuEngineCompleted(self.h, ctypes.byref(c)), "tcpxuEngineCompleted")
+        return c.value
+
+    def running(self):
+        r = ctypes.c_int()
+        self.pkg.check(self.hip.tcpxuEngineRunning(self.h, ctypes.byref(r)), "tcpxuEngineRunning")
+        return bool(r.value)
+
+    def destroy(self):
+        if self.started:
+            self.stop()
+        self.pkg.check(self.hip.tcpxuEngineDestroy(self.h), "tcpxuEngineDestroy")
+
+
+def run_requests(pkg, hip, oracle, wl, read_back_while_running, **cfg):
+    """One submission per request of the workload; returns nothing, asserts byte equality with the oracle."""
+    info = wl.info
+    pool = np.empty(info.pool_bytes, dtype=np.uint8)
+    wl.fill_window(0, pool)
+    expect = oracle_expected(oracle, pool, wl.descs, info.dst_bytes, info.dst_misalign)
+    g = GpuBuffers(pool, wl.descs, info.dst_bytes, info.dst_misalign)
+    m = Mapped(pkg, hip, np.ascontiguousarray(wl.descs), len(wl.requests))
+    e = Engine(pkg, hip, **cfg)
+    print("engine case: config=%d shrink=%d requests=%d cfg=%r" % (wl.config, wl.shrink, len(wl.requests), cfg), flush=True)
+    e.start()
+    try:
+        for i, r in enumerate(wl.requests):
+            e.submit(g.pool.data_ptr(), g.dst_base, m.desc_dev(int(r["first_desc"])), int(r["n_descs"]), m.flag_dev(i), i + 1)
+        for i in range(len(wl.requests)):
+            m.wait(i, i + 1)
+        if read_back_while_running:
+            got = g.result()
+    finally:
+        e.stop()
+    if not read_back_while_running:
+        got = g.result()
+    assert e.completed() == len(wl.requests)
+    e.destroy()
+    m.free()
+    assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
+
+
+def test_engine_smallest(pkg, hip, oracle):
+    """One submission, read back after the engine has stopped."""
+    wl = pkg.Workload(1, seed=11, shrink=4)
+    run_requests(pkg, hip, oracle, wl, read_back_while_running=False)
+
+
+@pytest.mark.parametrize("config", [1, 2, 3, 4, 5])
+def test_engine_workloads_reduced(pkg, hip, oracle, config):
+    wl = pkg.Workload(config, seed=0xC0FFEE00 + config, shrink=3)
+    run_requests(pkg, hip, oracle, wl, read_back_while_running=True)
+
+
+@pytest.mark.parametrize("config", [2, 4])
+def test_engine_workloads_full_size(pkg, hip, oracle, config):
+    wl = pkg.Workload(config, seed=0xC0FFEE00 + config, shrink=0)
+    run_requests(pkg, hip, oracle, wl, read_back_while_running=True)
+
+
+@pytest.mark.parametrize("per_ticket", [1, 4, 16, 64])
+def test_engine_ticket_sizes(pkg, hip, oracle, per_ticket):
+    wl = pkg.Workload(5, seed=5, shrink=3)
+    run_requests(pkg, hip, oracle, wl, read_back_while_running=True, descs_per_ticket=per_ticket)
+
+
+def test_engine_small_ring_backpressure(pkg, hip, oracle):
+    """More submissions than ring entries: submit reports 'in progress' and later succeeds."""
+    wl = pkg.Workload(3, seed=6, shrink=3)  # 256 requests
+    run_requests(pkg, hip, oracle, wl, read_back_while_running=True, ring_entries=8)
+
+
+def test_engine_restart_and_empty_submission(pkg, hip, oracle):
+    pool = np.random.default_rng(7).integers(0, 256, size=1 << 20, dtype=np.uint8)
+    rows = [((i * 4096 + 5) % (1 << 20 - 1), 4000 + i % 90, i * 4096 + 9) for i in range(100)]
+    descs = make_descs(rows)
+    expect = oracle_expected(oracle, pool, descs, 100 * 4096 + 4096)
+    g = GpuBuffers(pool, descs, 100 * 4096 + 4096)
+    m = Mapped(pkg, hip, descs, 4)
+    e = Engine(pkg, hip)
+    for round_ in range(3):
+        g.reset()
+        for f in range(4):
+            m.flags[f] = 0
+        e.start()
+        assert e.running()
+        e.submit(g.pool.data_ptr(), g.dst_base, m.desc_dev(0), 50, m.flag_dev(0), 100 + round_)
+        e.submit(None, None, None, 0, m.flag_dev(1), 200 + round_)  # zero descriptors: completes at once
+        e.submit(g.pool.data_ptr(), g.dst_base, m.desc_dev(50), 50, m.flag_dev(2), 300 + round_)
+        m.wait(0, 100 + round_)
+        m.wait(1, 200 + round_)
+        m.wait(2, 300 + round_)
+        us = e.stop()
+        assert not e.running()
+        assert us > 0
+        assert e.completed() == 3 * (round_ + 1)
+        got = g.result()
+        assert first_difference(got, expect) is None, repr(first_difference(got, expect))
+    e.destroy()
+    m.free()
+
+
+def test_engine_submissions_queued_while_stopped(pkg, hip, oracle):
+    """Submissions made before the kernel is launched are picked up when it starts."""
+    pool = np.random.default_rng(8).integers(0, 256, size=1 << 18, dtype=np.uint8)
+    descs = make_descs([(i * 1000, 999, i * 1000) for i in range(200)])
+    expect = oracle_expected(oracle, pool, descs, 200 * 1000)
+    g = GpuBuffers(pool, descs, 200 * 1000)
+    m = Mapped(pkg, hip, descs, 2)
+    e = Engine(pkg, hip)
+    e.submit(g.pool.data_ptr(), g.dst_base, m.desc_dev(0), 120, m.flag_dev(0), 1)
+    e.submit(g.pool.data_ptr(), g.dst_base, m.desc_dev(120), 80, m.flag_dev(1), 2)
+    e.start()
+    m.wait(0, 1)
+    m.wait(1, 2)
+    e.stop()
+    got = g.result()
+    e.destroy()
+    m.free()
+    assert first_difference(got, expect) is None
+
+
+def test_engine_spin_limit_exits_by_itself(pkg, hip):
+    """Bounded wait: with a spin limit the kernel leaves on its own when nothing is submitted."""
+    e = Engine(pkg, hip, spin_limit=2000)
+    e.start()
+    deadline = time.time() + 20
+    while e.running():
+        assert time.time() < deadline, "engine with a spin limit is still running"
+        time.sleep(0.01)
+    e.stop()  # reaps the finished launch
+    e.destroy()
+
+
+def test_engine_argument_errors(pkg, hip):
+    e = Engine(pkg, hip)
+    flag = ctypes.c_void_p(0x1000)
+    assert hip.tcpxuEngineSubmit(e.h, None, None, None, 0, None, 1) == pkg.INVALID_ARGUMENT
+    assert hip.tcpxuEngineSubmit(e.h, None, None, None, 0, flag, 0) == pkg.INVALID_ARGUMENT
+    assert hip.tcpxuEngineSubmit(e.h, None, None, None, 4, flag, 1) == pkg.INVALID_ARGUMENT
+    assert hip.tcpxuEngineStop(e.h, None) == pkg.INVALID_USAGE
+    bad = pkg.EngineConfig(1000, 0, 0, 0)
+    h = ctypes.c_void_p()
+    assert hip.tcpxuEngineCreate(0, ctypes.byref(bad), ctypes.byref(h)) == pkg.INVALID_ARGUMENT
+    bad = pkg.EngineConfig(0, 0, 65, 0)
+    assert hip.tcpxuEngineCreate(0, ctypes.byref(bad), ctypes.byref(h)) == pkg.INVALID_ARGUMENT
+    e.destroy()

@@ -1,0 +1,162 @@
+"""GPU parity of the launch-per-batch unpack kernel (tcpxuUnpackBatch) against the CPU oracle, byte-exact.
+
+Tolerance: none -- this path is integer/byte work, every byte of the destination (guard bands included) must be
+identical to the oracle's.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+
+from conftest import GUARD, SENTINEL, GpuBuffers, first_difference, make_descs, oracle_expected
+
+pytestmark = pytest.mark.gpu
+
+
+def run_batch(pkg, hip, oracle, pool, descs, dst_bytes, misalign=0):
+    expect = oracle_expected(oracle, pool, descs, dst_bytes, misalign)
+    g = GpuBuffers(pool, descs, dst_bytes, misalign)
+    print("case: n=%d dst_bytes=%d misalign=%d" % (len(descs), dst_bytes, misalign), flush=True)
+    pkg.check(hip.tcpxuUnpackBatch(0, g.pool.data_ptr(), g.dst_base, g.descs.data_ptr(), g.n, None), "tcpxuUnpackBatch")
+    pkg.check(hip.tcpxuDeviceSynchronize(0), "sync")
+    got = g.result()
+    assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
+
+
+def seeded_pool(nbytes, seed):
+    return np.random.default_rng(seed).integers(0, 256, size=nbytes, dtype=np.uint8)
+
+
+@pytest.mark.parametrize("config", [1, 2, 3, 4, 5])
+def test_workloads_reduced(pkg, hip, oracle, config):
+    wl = pkg.Workload(config, seed=0xC0FFEE00 + config, shrink=4)
+    pool = np.empty(wl.info.pool_bytes, dtype=np.uint8)
+    wl.fill_window(0, pool)
+    # window 0 payload everywhere: reuse of pages across windows is exercised in test_windows_refill
+    run_batch(pkg, hip, oracle, pool, wl.descs, wl.info.dst_bytes, wl.info.dst_misalign)
+
+
+@pytest.mark.parametrize("config", [1, 2, 3, 4])
+def test_workloads_full_size(pkg, hip, oracle, config):
+    wl = pkg.Workload(config, seed=0xC0FFEE00 + config, shrink=0)
+    pool = np.empty(wl.info.pool_bytes, dtype=np.uint8)
+    wl.fill_window(0, pool)
+    run_batch(pkg, hip, oracle, pool, wl.descs, wl.info.dst_bytes, wl.info.dst_misalign)
+
+
+def test_windows_refill_full_size(pkg, hip, oracle):
+    """Adversarial workload at full size: pages are refilled between requests, as recycled pages would be."""
+    import torch
+
+    wl = pkg.Workload(5, seed=0xC0FFEE05, shrink=0)
+    info = wl.info
+    pool = np.empty(info.pool_bytes, dtype=np.uint8)
+    expect = np.full(GUARD + info.dst_misalign + info.dst_bytes + GUARD, SENTINEL, dtype=np.uint8)
+    base = GUARD + info.dst_misalign
+    g = None
+    for r in wl.requests:
+        w = int(r["window"])
+        wl.fill_window(w, pool)
+        d = np.ascontiguousarray(wl.descs[int(r["first_desc"]) : int(r["first_desc"]) + int(r["n_descs"])])
+        import __graft_entry__ as graft
+
+        graft.oracle_unpack(oracle, expect[base : base + info.dst_bytes], pool, d)
+        if g is None:
+            g = GpuBuffers(pool, wl.descs, info.dst_bytes, info.dst_misalign)
+        else:
+            g.pool.copy_(torch.from_numpy(pool))
+            torch.cuda.synchronize()
+        print("window %d: %d descriptors" % (w, len(d)), flush=True)
+        pkg.check(
+            hip.tcpxuUnpackBatch(0, g.pool.data_ptr(), g.dst_base, g.descs.data_ptr() + 16 * int(r["first_desc"]), len(d), None),
+            "tcpxuUnpackBatch",
+        )
+        pkg.check(hip.tcpxuDeviceSynchronize(0), "sync")
+    got = g.result()
+    assert first_difference(got, expect) is None, repr(first_difference(got, expect))
+
+
+def test_every_alignment_and_short_length(pkg, hip, oracle):
+    """All 16x16 (src, dst) alignments times lengths around the vector and round boundaries."""
+    pool = seeded_pool(1 << 20, 1)
+    lengths = [1, 2, 3, 15, 16, 17, 31, 32, 33, 63, 64, 65, 255, 256, 1023, 1024, 1025, 4079, 4080, 4081, 4095, 4096]
+    rows, dst = [], 0
+    rng = np.random.default_rng(2)
+    for sa in range(16):
+        for da in range(16):
+            for ln in lengths:
+                page = int(rng.integers(0, (1 << 20) // 4096))
+                in_page = sa if sa + ln <= 4096 else 0
+                dst = (dst + 15) // 16 * 16 + da
+                rows.append((page * 4096 + in_page, ln, dst))
+                dst += ln + 1  # one sentinel byte between neighbours must survive
+    run_batch(pkg, hip, oracle, pool, make_descs(rows), dst + 16)
+
+
+def test_empty_and_zero_length(pkg, hip, oracle):
+    pool = seeded_pool(1 << 16, 3)
+    run_batch(pkg, hip, oracle, pool, make_descs([]), 4096)
+    run_batch(pkg, hip, oracle, pool, make_descs([(0, 0, 0), (5, 0, 100), (4096, 0, 4095)]), 4096)
+    run_batch(pkg, hip, oracle, pool, make_descs([(0, 0, 0), (7, 100, 3), (9, 0, 50), (4096, 1, 200)]), 4096)
+
+
+def test_single_bytes_and_ragged_tail(pkg, hip, oracle):
+    pool = seeded_pool(1 << 16, 4)
+    rows = [(i * 37 % 60000, 1, i * 3) for i in range(1000)]
+    run_batch(pkg, hip, oracle, pool, make_descs(rows), 3 * 1000 + 8)
+    # descriptor count that is not a multiple of any batch size
+    rows = [((i * 4096) % 61440, 4096 - (i % 7), i * 4096) for i in range(1021)]
+    run_batch(pkg, hip, oracle, pool, make_descs(rows), 1021 * 4096)
+
+
+def test_long_descriptor_beyond_one_page(pkg, hip, oracle):
+    """The wire contract caps a fragment at 4 KiB, but `len` is 32 bits: longer copies must still be exact."""
+    pool = seeded_pool(1 << 20, 5)
+    rows = [(3, 70001, 5), (100000, 8192, 80000), (200001, 4097, 90001)]
+    run_batch(pkg, hip, oracle, pool, make_descs(rows), 100000)
+
+
+def test_descriptors_in_mapped_host_memory(pkg, hip, oracle):
+    """The kernel reads descriptors through the device alias of hipHostMalloc-mapped memory."""
+    wl = pkg.Workload(2, seed=77, shrink=3)
+    pool = np.empty(wl.info.pool_bytes, dtype=np.uint8)
+    wl.fill_window(0, pool)
+    expect = oracle_expected(oracle, pool, wl.descs, wl.info.dst_bytes)
+    g = GpuBuffers(pool, wl.descs, wl.info.dst_bytes)
+    host_p, dev_p = ctypes.c_void_p(), ctypes.c_void_p()
+    pkg.check(hip.tcpxuMappedAlloc(0, wl.descs.nbytes, ctypes.byref(host_p), ctypes.byref(dev_p)), "tcpxuMappedAlloc")
+    ctypes.memmove(host_p.value, wl.descs.ctypes.data, wl.descs.nbytes)
+    pkg.check(hip.tcpxuUnpackBatch(0, g.pool.data_ptr(), g.dst_base, dev_p.value, g.n, None), "tcpxuUnpackBatch")
+    pkg.check(hip.tcpxuDeviceSynchronize(0), "sync")
+    got = g.result()
+    pkg.check(hip.tcpxuMappedFree(0, host_p), "tcpxuMappedFree")
+    assert first_difference(got, expect) is None, repr(first_difference(got, expect))
+
+
+def test_linearity_two_halves_equal_whole(pkg, hip, oracle):
+    """Size-independent property: unpacking a list in two launches equals unpacking it in one."""
+    wl = pkg.Workload(4, seed=9, shrink=2)
+    pool = np.empty(wl.info.pool_bytes, dtype=np.uint8)
+    wl.fill_window(0, pool)
+    g = GpuBuffers(pool, wl.descs, wl.info.dst_bytes)
+    pkg.check(hip.tcpxuUnpackBatch(0, g.pool.data_ptr(), g.dst_base, g.descs.data_ptr(), g.n, None), "whole")
+    pkg.check(hip.tcpxuDeviceSynchronize(0), "sync")
+    whole = g.result()
+    g.reset()
+    half = g.n // 2 + 3
+    pkg.check(hip.tcpxuUnpackBatch(0, g.pool.data_ptr(), g.dst_base, g.descs.data_ptr() + 16 * half, g.n - half, None), "b")
+    pkg.check(hip.tcpxuUnpackBatch(0, g.pool.data_ptr(), g.dst_base, g.descs.data_ptr(), half, None), "a")
+    pkg.check(hip.tcpxuDeviceSynchronize(0), "sync")
+    assert np.array_equal(whole, g.result())
+    assert np.array_equal(whole, oracle_expected(oracle, pool, wl.descs, wl.info.dst_bytes))
+
+
+def test_argument_errors(pkg, hip):
+    assert hip.tcpxuUnpackBatch(0, None, None, None, 5, None) == pkg.INVALID_ARGUMENT
+    p = ctypes.c_void_p()
+    assert hip.tcpxuArenaCreate(0, 4097, ctypes.byref(p)) == pkg.INVALID_ARGUMENT
+    assert hip.tcpxuArenaCreate(0, (1 << 32) + 4096, ctypes.byref(p)) == pkg.INVALID_ARGUMENT
+    assert hip.tcpxuArenaCreate(99, 4096, ctypes.byref(p)) == pkg.INVALID_ARGUMENT
+    pkg.check(hip.tcpxuArenaCreate(0, 1 << 20, ctypes.byref(p)), "arena")
+    assert p.value % 4096 == 0
+    pkg.check(hip.tcpxuArenaDestroy(0, p), "arena destroy")
