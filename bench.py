@@ -152,7 +152,7 @@ def main():
         "dtype": "u8",
         "data": "synthetic",
         "config": {
-            "workload": "8 MiB chunk, 4 interleaved flows, ~2155 fragments (90% 4096 B, 10% U[64,4095]), byte-unaligned "
+            "workload": "8 MiB chunk, 4 interleaved flows, ~2155 fragments (90%% 4096 B, 10%% U[64,4095]), byte-unaligned "
             "sources in a 256 MiB pool, 2 x 4 MiB requests per chunk, %d distinct chunks cycled, ring depth %d"
             % (args.chunks, args.depth),
             "path": "persistent engine: mapped descriptor ring -> gfx950 unpack kernel -> mapped completion word",
