@@ -108,7 +108,7 @@ int tcpxuCopyKernelTimed(int device, void* dst, const void* src, size_t bytes, i
 typedef struct tcpxuEngine tcpxuEngine;
 
 typedef struct tcpxuEngineConfig {
-  uint32_t ring_entries;    /* submission ring size, power of two, 0 = default (1024) */
+  uint32_t ring_entries;    /* submission ring size, power of two >= 16, 0 = default (1024) */
   uint32_t workgroups;      /* persistent grid size, 0 = fill the GPU */
   uint32_t descs_per_ticket;/* descriptors one workgroup takes at a time, 0 = default */
   uint32_t spin_limit;      /* 0 = poll until stopped; otherwise the kernel exits by itself after this many

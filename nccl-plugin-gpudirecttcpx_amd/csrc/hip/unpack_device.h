@@ -95,6 +95,97 @@ __device__ __forceinline__ void wave_copy_fragment(const uint8_t* __restrict__ s
   if (edge) store_byte(dst + edge_off, edge_byte);
 }
 
+// ---- coherent variant, for the persistent engine ------------------------------------------------------------------
+// A kernel that never ends gets no cache invalidate at launch and no write-back at exit, so its payload accesses
+// carry the coherence themselves: loads and stores are issued at system scope (sc0 sc1).  A load then never
+// returns a line that an XCD's L2 kept from an earlier use of a recycled bounce page, and a store is written
+// through, so that once the wavefront's store counter has drained (s_waitcnt vmcnt(0)) the bytes are where the
+// host, a DMA engine or another kernel will read them -- no L2 write-back instruction is ever needed.
+// The loads of one round and the wait for them form a single asm block: the compiler does not track counters
+// for memory instructions it cannot see.
+__device__ __forceinline__ void store_vec_sys(uint8_t* p, u32x4 v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void store_byte_sys(uint8_t* p, uint32_t v) {
+  asm volatile("global_store_byte %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+}
+
+// Same contract as wave_copy_fragment.  One round moves up to 4 KiB: every lane issues the edge-byte load and
+// one or four vector loads back to back (lanes past the end re-read the fragment's last vector, which is in
+// range), waits once, then stores under its predicates.
+__device__ __forceinline__ void wave_copy_fragment_coherent(const uint8_t* __restrict__ src,
+                                                            uint8_t* __restrict__ dst, uint32_t len,
+                                                            uint32_t lane) {
+  if (len == 0) return;
+  uint32_t head = static_cast<uint32_t>(-reinterpret_cast<uintptr_t>(dst)) & 15u;
+  if (head > len) head = len;
+  const uint32_t body = len - head;
+  const uint32_t nvec = body >> 4;
+  const uint32_t tail = body & 15u;
+
+  uint32_t edge_off = 0;
+  bool edge = false;
+  if (lane < head) {
+    edge = true;
+    edge_off = lane;
+  } else if (lane >= 16u && lane - 16u < tail) {
+    edge = true;
+    edge_off = head + (nvec << 4) + (lane - 16u);
+  }
+  const uint8_t* edge_src = src + edge_off;  // offset 0 for lanes without an edge byte: inside the fragment
+  uint32_t edge_byte = 0;
+
+  if (nvec == 0) {
+    asm volatile(
+        "global_load_ubyte %0, %1, off sc0 sc1\n"
+        "s_waitcnt vmcnt(0)"
+        : "=&v"(edge_byte)
+        : "v"(edge_src)
+        : "memory");
+    if (edge) store_byte_sys(dst + edge_off, edge_byte);
+    return;
+  }
+
+  const uint8_t* sb = src + head;
+  uint8_t* db = dst + head;
+  const uint32_t last = nvec - 1;
+  for (uint32_t base = 0; base < nvec; base += kVecPerRound) {
+    const uint32_t v0 = base + lane;
+    const uint32_t v1 = v0 + kWaveLanes, v2 = v0 + 2 * kWaveLanes, v3 = v0 + 3 * kWaveLanes;
+    const uint8_t* p0 = sb + (static_cast<size_t>(v0 < last ? v0 : last) << 4);
+    u32x4 r0, r1, r2, r3;
+    if (nvec - base <= kWaveLanes) {  // wave-uniform
+      asm volatile(
+          "global_load_ubyte %1, %3, off sc0 sc1\n"
+          "global_load_dwordx4 %0, %2, off sc0 sc1\n"
+          "s_waitcnt vmcnt(0)"
+          : "=&v"(r0), "=&v"(edge_byte)
+          : "v"(p0), "v"(edge_src)
+          : "memory");
+      if (v0 < nvec) store_vec_sys(db + (static_cast<size_t>(v0) << 4), r0);
+    } else {
+      const uint8_t* p1 = sb + (static_cast<size_t>(v1 < last ? v1 : last) << 4);
+      const uint8_t* p2 = sb + (static_cast<size_t>(v2 < last ? v2 : last) << 4);
+      const uint8_t* p3 = sb + (static_cast<size_t>(v3 < last ? v3 : last) << 4);
+      asm volatile(
+          "global_load_ubyte %4, %9, off sc0 sc1\n"
+          "global_load_dwordx4 %0, %5, off sc0 sc1\n"
+          "global_load_dwordx4 %1, %6, off sc0 sc1\n"
+          "global_load_dwordx4 %2, %7, off sc0 sc1\n"
+          "global_load_dwordx4 %3, %8, off sc0 sc1\n"
+          "s_waitcnt vmcnt(0)"
+          : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3), "=&v"(edge_byte)
+          : "v"(p0), "v"(p1), "v"(p2), "v"(p3), "v"(edge_src)
+          : "memory");
+      if (v0 < nvec) store_vec_sys(db + (static_cast<size_t>(v0) << 4), r0);
+      if (v1 < nvec) store_vec_sys(db + (static_cast<size_t>(v1) << 4), r1);
+      if (v2 < nvec) store_vec_sys(db + (static_cast<size_t>(v2) << 4), r2);
+      if (v3 < nvec) store_vec_sys(db + (static_cast<size_t>(v3) << 4), r3);
+    }
+  }
+  if (edge) store_byte_sys(dst + edge_off, edge_byte);
+}
+
 // The 8 XCDs of an MI355X receive workgroups round-robin by workgroup id and each has its own L2.  This maps a
 // workgroup id to a work-item index such that every XCD walks one contiguous eighth of the index space:
 // neighbouring descriptor batches (neighbouring destination lines) then meet in the same L2.

@@ -145,7 +145,7 @@ def test_engine_ticket_sizes(pkg, hip, oracle, per_ticket):
 def test_engine_small_ring_backpressure(pkg, hip, oracle):
     """More submissions than ring entries: submit reports 'in progress' and later succeeds."""
     wl = pkg.Workload(3, seed=6, shrink=3)  # 256 requests
-    run_requests(pkg, hip, oracle, wl, read_back_while_running=True, ring_entries=8)
+    run_requests(pkg, hip, oracle, wl, read_back_while_running=True, ring_entries=16)
 
 
 def test_engine_restart_and_empty_submission(pkg, hip, oracle):
