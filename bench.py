@@ -110,6 +110,9 @@ def main():
     cfg = pkg.EngineConfig(0, 0, 0, 0)
     pkg.check(hip.tcpxuEngineCreate(dev, ctypes.byref(cfg), ctypes.byref(engine)), "tcpxuEngineCreate")
 
+    eff = pkg.EngineConfig()
+    pkg.check(hip.tcpxuEngineGetConfig(engine, ctypes.byref(eff)), "tcpxuEngineGetConfig")
+
     def run(items, depth, want_latency=False):
         wall, kern = ctypes.c_double(), ctypes.c_double()
         lat = (ctypes.c_double * len(items))() if want_latency else None
@@ -160,6 +163,8 @@ def main():
             "slots_per_step": slots_per_step,
             "device": name.value.decode(),
             "compute_units": cus.value,
+            "engine_workgroups": eff.workgroups,
+            "descs_per_ticket": eff.descs_per_ticket,
         },
         "roofline": {
             "bound": "hbm",

@@ -134,6 +134,9 @@ int tcpxuEngineSubmit(tcpxuEngine* engine, const void* bounce_base, void* dst_ba
 /* Number of submissions the GPU has fully completed since creation (monotone; read from mapped memory). */
 int tcpxuEngineCompleted(tcpxuEngine* engine, uint64_t* completed);
 
+/* The configuration in effect (defaults resolved: actual grid size, ring size, ticket size). */
+int tcpxuEngineGetConfig(tcpxuEngine* engine, tcpxuEngineConfig* config);
+
 /* 1 if the persistent kernel is running, 0 if stopped or exited by its spin limit. */
 int tcpxuEngineRunning(tcpxuEngine* engine, int* running);
 

@@ -36,6 +36,7 @@
 #include <mutex>
 #include <new>
 #include <thread>
+#include <unordered_map>
 #include <vector>
 
 #include "hip_common.h"
@@ -107,25 +108,12 @@ __device__ __forceinline__ uint64_t bcast64(uint64_t v, uint32_t src_lane) {
   return (static_cast<uint64_t>(bcast(static_cast<uint32_t>(v >> 32), src_lane)) << 32) |
          bcast(static_cast<uint32_t>(v), src_lane);
 }
-// Payload word i of the record held by lanes [first_lane, first_lane + 16).
-__device__ __forceinline__ uint32_t payload32(uint32_t word, uint32_t first_lane, int i) {
-  return bcast(word, first_lane + payload_slot(i));
-}
-__device__ __forceinline__ uint64_t payload64(uint32_t word, uint32_t first_lane, int i) {
-  return (static_cast<uint64_t>(payload32(word, first_lane, i + 1)) << 32) | payload32(word, first_lane, i);
-}
-
-__device__ __forceinline__ void write_record(Record* rec, const uint32_t (&p)[kPayloadWords], uint32_t stamp) {
-  uint8_t* base = reinterpret_cast<uint8_t*>(rec);
-#pragma unroll
-  for (int sct = 0; sct < 4; ++sct) {
-    u32x4 v = {p[3 * sct], p[3 * sct + 1], p[3 * sct + 2], stamp};
-    store_vec_sys(base + 16 * sct, v);
-  }
-}
-
 // ---- leader -------------------------------------------------------------------------------------------------------
 // Runs on wavefront 0 of workgroup 0.  All control flow is wave-uniform.
+__device__ __forceinline__ uint32_t lane_value(uint32_t v, uint32_t src_lane) {
+  return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), static_cast<int>(src_lane)));
+}
+
 __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uint32_t* job_target,
                             uint32_t ring_mask, uint32_t per_ticket, uint32_t spin_limit) {
   const uint32_t lane = threadIdx.x;
@@ -134,59 +122,69 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
   uint64_t mirrored = ~0ull;
   uint64_t idle = 0;
   uint32_t reason = 0;
+  // Fixed per-lane roles in the auxiliary load (second load of every poll), so that both loads of a poll are
+  // issued back to back by all lanes and waited for once:
+  //   lanes 0-3  jobs_done of the job slots of entries s..s+3      lanes 4-7  job_target of the same slots
+  //   lane 8     low word of tickets_done                          lane 9     low word of the host stop word
+  //   other lanes repeat lane 9.
+  const uint32_t* const tickets_done_lo = reinterpret_cast<const uint32_t*>(&st->tickets_done);
+  const uint32_t* const host_stop_lo = reinterpret_cast<const uint32_t*>(&ctl->stop);
 
   for (;;) {
-    // One round trip fetches entries s .. s+3 (lane 16k+i reads word i of entry s+k) and, alongside, what is
-    // needed to act on them: for each entry its job slot's counters, plus tickets_done and the host stop word.
+    // One round trip fetches entries s .. s+3: lane 16k+i reads word i of entry s+k.
     const uint32_t k_of_lane = lane >> 4;
-    const Record* e = &ctl->ring[(s + k_of_lane) & ring_mask];
-    const uint32_t word = sys_load(&e->w[lane & 15]);
-    uint64_t aux = 0;
-    if (lane < kPollEntries) aux = sys_load(&jobs_done[(s + lane) & ring_mask]);
-    else if (lane < 2 * kPollEntries) aux = sys_load(&job_target[(s + lane - kPollEntries) & ring_mask]);
-    else if (lane == 8) aux = sys_load(&st->tickets_done);
-    else if (lane == 9) aux = sys_load(&ctl->stop);
+    const uint32_t word = sys_load(&ctl->ring[(s + k_of_lane) & ring_mask].w[lane & 15]);
+    const uint32_t* aux_addr = host_stop_lo;
+    if (lane < kPollEntries) aux_addr = &jobs_done[(s + lane) & ring_mask];
+    else if (lane < 2 * kPollEntries) aux_addr = &job_target[(s + lane - kPollEntries) & ring_mask];
+    else if (lane == 8) aux_addr = tickets_done_lo;
+    const uint32_t aux = sys_load(aux_addr);
+
     const uint32_t expect = static_cast<uint32_t>(s + k_of_lane + 1);
     const bool stamp_ok = ((lane & 3) == 3) ? (word == expect) : true;
     const uint64_t ok_mask = __ballot(stamp_ok);
-    const uint64_t tickets_done = bcast64(aux, 8);
+    const uint32_t tickets_done = lane_value(aux, 8);
 
     uint32_t consumed = 0;
+#pragma unroll 1
     for (uint32_t k = 0; k < kPollEntries; ++k) {
       if (((ok_mask >> (16 * k)) & 0xFFFFull) != 0xFFFFull) break;
-      const uint32_t first_lane = 16 * k;
-      const uint32_t n = payload32(word, first_lane, 10);
+      const uint32_t fl = 16 * k;  // first lane of entry k
+      const uint32_t n = lane_value(word, fl + payload_slot(10));
+      const uint32_t flag_lo = lane_value(word, fl + payload_slot(6)), flag_hi = lane_value(word, fl + payload_slot(7));
+      const uint32_t val_lo = lane_value(word, fl + payload_slot(8)), val_hi = lane_value(word, fl + payload_slot(9));
       if (n == 0) {
-        // Lane broadcasts need the whole wavefront: read the fields before narrowing to one lane.
-        const uint64_t done_flag = payload64(word, first_lane, 6);
-        const uint64_t done_value = payload64(word, first_lane, 8);
         if (lane == 0) {
-          sys_store(reinterpret_cast<uint64_t*>(done_flag), done_value);
+          sys_store(reinterpret_cast<uint64_t*>((static_cast<uint64_t>(flag_hi) << 32) | flag_lo),
+                    (static_cast<uint64_t>(val_hi) << 32) | val_lo);
           __hip_atomic_fetch_add(&st->jobs_completed, 1ull, __ATOMIC_RELAXED, SYS);
         }
       } else {
         const uint32_t nt = (n + per_ticket - 1) / per_ticket;
         const uint32_t slot = static_cast<uint32_t>(s + k) & ring_mask;
-        const uint32_t done_now = bcast(static_cast<uint32_t>(aux), k);
-        const uint32_t target_prev = bcast(static_cast<uint32_t>(aux), kPollEntries + k);
+        const uint32_t done_now = lane_value(aux, k);
+        const uint32_t target_prev = lane_value(aux, kPollEntries + k);
         // The job slot is free once every ticket ever issued for it has been counted; the ticket ring has room
-        // while fewer than its size are outstanding.  Otherwise leave this entry for a later poll.
+        // while fewer than its size are outstanding (32-bit wrapping arithmetic).  Otherwise leave this entry
+        // for a later poll.
         if (done_now != target_prev) break;
-        if (tickets_out + nt - tickets_done > kTicketRing) break;
+        if (static_cast<uint32_t>(tickets_out) + nt - tickets_done > kTicketRing) break;
         const uint32_t target = target_prev + nt;
         if (lane == 0) sys_store(&job_target[slot], target);
-        uint32_t p[kPayloadWords];
-#pragma unroll
-        for (int i = 0; i < 10; ++i) p[i] = payload32(word, first_lane, i);
-        p[11] = target;
-        const uint64_t descs = (static_cast<uint64_t>(p[5]) << 32) | p[4];
+        const uint32_t bounce_lo = lane_value(word, fl + payload_slot(0)), bounce_hi = lane_value(word, fl + payload_slot(1));
+        const uint32_t dst_lo = lane_value(word, fl + payload_slot(2)), dst_hi = lane_value(word, fl + payload_slot(3));
+        const uint64_t descs =
+            (static_cast<uint64_t>(lane_value(word, fl + payload_slot(5))) << 32) | lane_value(word, fl + payload_slot(4));
         for (uint32_t i = lane; i < nt; i += kWaveLanes) {
           const uint64_t d = descs + static_cast<uint64_t>(i) * per_ticket * sizeof(tcpxuLoadMeta);
-          p[4] = static_cast<uint32_t>(d);
-          p[5] = static_cast<uint32_t>(d >> 32);
-          p[10] = std::min(per_ticket, n - i * per_ticket) | (slot << 8);
+          const uint32_t count = std::min(per_ticket, n - i * per_ticket);
           const uint64_t t = tickets_out + i;
-          write_record(&st->tickets[t & (kTicketRing - 1)], p, static_cast<uint32_t>(t + 1));
+          const uint32_t stamp = static_cast<uint32_t>(t + 1);
+          uint8_t* rec = reinterpret_cast<uint8_t*>(&st->tickets[t & (kTicketRing - 1)]);
+          store_vec_sys(rec, u32x4{bounce_lo, bounce_hi, dst_lo, stamp});
+          store_vec_sys(rec + 16, u32x4{dst_hi, static_cast<uint32_t>(d), static_cast<uint32_t>(d >> 32), stamp});
+          store_vec_sys(rec + 32, u32x4{flag_lo, flag_hi, val_lo, stamp});
+          store_vec_sys(rec + 48, u32x4{val_hi, count | (slot << 8), target, stamp});
         }
         tickets_out += nt;
       }
@@ -200,7 +198,8 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
     }
 
     // Nothing could be consumed this round.
-    if (bcast64(aux, 9) != 0 && ((ok_mask & 0xFFFFull) != 0xFFFFull)) {
+    const bool nothing_there = (ok_mask & 0xFFFFull) != 0xFFFFull;
+    if (lane_value(aux, 9) != 0 && nothing_there) {
       // Stop requested and entry s not there.  The host wrote its last tail before the stop word, so a tail
       // read now bounds what is still to come.
       uint64_t tail_now = 0;
@@ -218,7 +217,6 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
         mirrored = c;
       }
     }
-    const bool nothing_there = (ok_mask & 0xFFFFull) != 0xFFFFull;
     if (spin_limit != 0 && nothing_there && ++idle > spin_limit) {
       reason = 2;
       break;
@@ -238,118 +236,212 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
 }
 
 // ---- worker -------------------------------------------------------------------------------------------------------
-__device__ void worker_loop(DevState* st, uint32_t* jobs_done) {
-  __shared__ uint32_t s_payload[kPayloadWords];
-  __shared__ tcpxuLoadMeta s_desc[kMaxDescsPerTicket];
-  __shared__ uint32_t s_go;
+// A worker workgroup is kCopyWaves copy wavefronts and one fetcher wavefront.  The fetcher stays one ticket ahead:
+// while the copy wavefronts move ticket i, it claims a number, polls that ticket's slot and pulls the ticket's
+// descriptors over PCIe into the other LDS stage.  Copy wavefronts therefore never wait for PCIe: between two
+// tickets they only meet the fetcher at one barrier.  The copy wavefront that finishes a ticket last counts it.
+constexpr uint32_t kCopyWaves = 8;
+constexpr uint32_t kEngineThreads = (kCopyWaves + 1) * kWaveLanes;
 
-  const uint32_t tid = threadIdx.x;
-  const uint32_t lane = tid & (kWaveLanes - 1);
-  const uint32_t wave = tid / kWaveLanes;
-  const uint32_t* stop_word = &st->stop[blockIdx.x % kStopReplicas].value;
-  uint64_t my_ticket = 0;  // valid in wavefront 0
-  if (wave == 0) {
-    uint64_t t = 0;
-    if (lane == 0) t = __hip_atomic_fetch_add(&st->ticket_head, 1ull, __ATOMIC_RELAXED, SYS);
-    my_ticket = bcast64(t, 0);
+struct Stage {
+  uint32_t payload[kPayloadWords];
+  uint32_t go;
+  uint32_t pad[3];
+  tcpxuLoadMeta desc[kMaxDescsPerTicket];
+};
+
+// Fetcher: look once at the slot of ticket number `ticket` (one 64-byte read, with this workgroup's stop word in
+// the same round trip).  Returns 1 and stages the ticket if it is there.  Wave-uniform.
+__device__ uint32_t try_fetch_ticket(DevState* st, const uint32_t* stop_word, uint64_t ticket, Stage* stage,
+                                     uint32_t lane, bool* stop_up) {
+  const Record* rec = &st->tickets[ticket & (kTicketRing - 1)];
+  const uint32_t expect = static_cast<uint32_t>(ticket + 1);
+  uint32_t word = 0;
+  if (lane < 16) word = sys_load(&rec->w[lane]);
+  else if (lane == 16) word = sys_load(stop_word);
+  *stop_up = bcast(word, 16) != 0;
+  const bool stamp_ok = (lane < 16 && (lane & 3) == 3) ? (word == expect) : true;
+  if (!__all(stamp_ok)) return 0;
+  // Lane broadcasts need the whole wavefront: gather first, then let 12 lanes store.
+  const uint32_t pl = lane < kPayloadWords ? lane : 0u;
+  const uint32_t gathered = bcast(word, (pl / 3) * 4 + (pl % 3));
+  if (lane < kPayloadWords) stage->payload[lane] = gathered;
+  if (lane == 0) stage->go = 1;
+  const uint64_t descs_addr =
+      (static_cast<uint64_t>(bcast(word, payload_slot(5))) << 32) | bcast(word, payload_slot(4));
+  const uint32_t n = bcast(word, payload_slot(10)) & 0xFFu;
+  if (lane < n) {
+    // One 16-byte descriptor per lane straight from the mapped slot (system scope: never a cached copy).
+    const u32x4 d = load_vec_sys(reinterpret_cast<const uint8_t*>(descs_addr) + 16 * lane);
+    *reinterpret_cast<u32x4*>(&stage->desc[lane]) = d;
   }
+  return 1;
+}
 
-  for (;;) {
-    if (wave == 0) {
-      // Poll my ticket's slot (one 64-byte read) together with this workgroup's stop word.
-      const Record* rec = &st->tickets[my_ticket & (kTicketRing - 1)];
-      const uint32_t expect = static_cast<uint32_t>(my_ticket + 1);
-      uint32_t go = 0;
-      uint32_t word = 0;
-      bool stop_seen = false;
-      uint32_t backoff = 1;
-      for (;;) {
-        uint32_t v = 0;
-        if (lane < 16) v = sys_load(&rec->w[lane]);
-        else if (lane == 16) v = sys_load(stop_word);
-        const bool stamp_ok = (lane < 16 && (lane & 3) == 3) ? (v == expect) : true;
-        if (__all(stamp_ok)) {
-          go = 1;
-          word = v;
-          break;
-        }
-        if (stop_seen) break;  // the stop word was already up on the previous look: my ticket will never come
-        stop_seen = bcast(v, 16) != 0;
-        if (!stop_seen) {
-          for (uint32_t i = 0; i < backoff; ++i) __builtin_amdgcn_s_sleep(4);
-          if (backoff < 16) backoff <<= 1;
-        }
-      }
-      // Lane broadcasts need the whole wavefront: gather first, then let 12 lanes store.
-      const uint32_t pl = lane < kPayloadWords ? lane : 0u;
-      const uint32_t gathered = bcast(word, (pl / 3) * 4 + (pl % 3));
-      if (go && lane < kPayloadWords) s_payload[lane] = gathered;
-      if (lane == 0) s_go = go;
+// Counts a finished ticket (all of its payload is in memory); the last ticket of a submission publishes the
+// completion word.
+__device__ void retire_ticket(DevState* st, uint32_t* jobs_done, const Stage* stage, uint32_t lane) {
+  if (lane == 0) {
+    const uint32_t job = stage->payload[10] >> 8;
+    const uint32_t target = stage->payload[11];
+    const uint32_t count = __hip_atomic_fetch_add(&jobs_done[job], 1u, __ATOMIC_RELAXED, SYS) + 1u;
+    __hip_atomic_fetch_add(&st->tickets_done, 1ull, __ATOMIC_RELAXED, SYS);
+    if (count == target) {
+      // Every other ticket's payload was in memory before it was counted, and so is this one's.
+      const uint64_t done_flag = (static_cast<uint64_t>(stage->payload[7]) << 32) | stage->payload[6];
+      const uint64_t done_value = (static_cast<uint64_t>(stage->payload[9]) << 32) | stage->payload[8];
+      sys_store(reinterpret_cast<uint64_t*>(done_flag), done_value);
+      __hip_atomic_fetch_add(&st->jobs_completed, 1ull, __ATOMIC_RELAXED, SYS);
     }
-    __syncthreads();
-    if (s_go == 0) break;  // workgroup-uniform
-    const uint64_t bounce_addr = (static_cast<uint64_t>(s_payload[1]) << 32) | s_payload[0];
-    const uint64_t dst_addr = (static_cast<uint64_t>(s_payload[3]) << 32) | s_payload[2];
-    const uint64_t descs_addr = (static_cast<uint64_t>(s_payload[5]) << 32) | s_payload[4];
-    const uint32_t n = s_payload[10] & 0xFFu;
-    if (tid < n) {
-      // 16-byte descriptor as two system-scope 8-byte loads straight from the mapped slot.
-      const uint64_t* p = reinterpret_cast<const uint64_t*>(descs_addr) + 2 * tid;
-      const uint64_t lo = sys_load(p);
-      const uint64_t hi = sys_load(p + 1);
-      s_desc[tid].src_off = static_cast<uint32_t>(lo);
-      s_desc[tid].len = static_cast<uint32_t>(lo >> 32);
-      s_desc[tid].dst_off = hi;
-    }
-    // Claim the next ticket number now: the atomic's round trip overlaps this ticket's copy.
-    uint64_t next_ticket = 0;
-    if (tid == 0) next_ticket = __hip_atomic_fetch_add(&st->ticket_head, 1ull, __ATOMIC_RELAXED, SYS);
-    __syncthreads();
-
-    const uint8_t* bounce = reinterpret_cast<const uint8_t*>(bounce_addr);
-    uint8_t* dst = reinterpret_cast<uint8_t*>(dst_addr);
-    for (uint32_t j = wave; j < n; j += kWavesPerWg) {
-      const tcpxuLoadMeta d = s_desc[j];
-      const uint32_t len = __builtin_amdgcn_readfirstlane(d.len);
-      const uint32_t so = __builtin_amdgcn_readfirstlane(d.src_off);
-      const uint32_t dlo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(d.dst_off));
-      const uint32_t dhi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(d.dst_off >> 32));
-      wave_copy_fragment_coherent(bounce + so, dst + ((static_cast<uint64_t>(dhi) << 32) | dlo), len, lane);
-    }
-    // Each wavefront waits until its own write-through payload stores are acknowledged; after the barrier the
-    // whole ticket is in memory and may be counted.
-    drain_memory_ops();
-    __syncthreads();
-
-    if (wave == 0) {
-      if (lane == 0) {
-        const uint32_t job = s_payload[10] >> 8;
-        const uint32_t target = s_payload[11];
-        const uint32_t count = __hip_atomic_fetch_add(&jobs_done[job], 1u, __ATOMIC_RELAXED, SYS) + 1u;
-        __hip_atomic_fetch_add(&st->tickets_done, 1ull, __ATOMIC_RELAXED, SYS);
-        if (count == target) {
-          // Last ticket of the submission: every other ticket's payload was in memory before it was counted.
-          const uint64_t done_flag = (static_cast<uint64_t>(s_payload[7]) << 32) | s_payload[6];
-          const uint64_t done_value = (static_cast<uint64_t>(s_payload[9]) << 32) | s_payload[8];
-          sys_store(reinterpret_cast<uint64_t*>(done_flag), done_value);
-          __hip_atomic_fetch_add(&st->jobs_completed, 1ull, __ATOMIC_RELAXED, SYS);
-        }
-      }
-      my_ticket = bcast64(next_ticket, 0);
-    }
-    // s_payload / s_desc are rewritten only after the next barrier pair; wavefront 0 rewrites s_payload before
-    // the first barrier of the next iteration, so everybody must be past their reads of it: they are, since
-    // the reads above happen before the second barrier of this iteration.
   }
 }
 
-__global__ __launch_bounds__(kWgThreads) void unpack_engine_kernel(HostCtl* ctl, DevState* st, uint32_t* jobs_done,
+// Copy wavefront `wave` of kCopyWaves: fragments wave, wave + kCopyWaves, ... of the staged ticket, with the
+// loads of the next round issued before the stores of the current one.  Two register sets alternate so that no
+// register is copied while a load into it is in flight.
+__device__ void copy_ticket(const Stage* stage, uint32_t wave, uint32_t lane) {
+  // Everything that describes a fragment is wave-uniform; saying so keeps it in scalar registers and leaves
+  // the vector registers to the payload in flight.
+  auto uniform = [](uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(v)); };
+  const uint8_t* bounce = reinterpret_cast<const uint8_t*>((static_cast<uint64_t>(uniform(stage->payload[1])) << 32) |
+                                                           uniform(stage->payload[0]));
+  uint8_t* dst =
+      reinterpret_cast<uint8_t*>((static_cast<uint64_t>(uniform(stage->payload[3])) << 32) | uniform(stage->payload[2]));
+  const uint32_t n = uniform(stage->payload[10]) & 0xFFu;
+  wave = uniform(wave);
+  uint32_t j = wave;
+  FragmentRounds fr;
+  // Next round of this wavefront's work, or false when there is none.  `prev` is the round before it.
+  auto produce = [&](CopyRound& out, const CopyRound& prev) -> bool {
+    if (fr.more()) {
+      out = fr.next_round(prev);
+      return true;
+    }
+    while (j < n) {
+      const tcpxuLoadMeta d = stage->desc[j];
+      j += kCopyWaves;
+      const uint32_t len = __builtin_amdgcn_readfirstlane(d.len);
+      if (len == 0) continue;
+      const uint32_t so = __builtin_amdgcn_readfirstlane(d.src_off);
+      const uint32_t dlo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(d.dst_off));
+      const uint32_t dhi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(d.dst_off >> 32));
+      const uint8_t* fsrc = bounce + so;
+      uint8_t* fdst = dst + ((static_cast<uint64_t>(dhi) << 32) | dlo);
+      if (fragment_is_tiny(fdst, len)) {
+        copy_tiny_fragment(fsrc, fdst, len, lane);
+        continue;
+      }
+      out = fr.first_round(fsrc, fdst, len, lane);
+      return true;
+    }
+    return false;
+  };
+  CopyRound ra, rb;
+  CopyRegs xa, xb;
+  if (!produce(ra, ra)) return;
+  round_load(ra, xa, lane);
+  for (;;) {
+    if (!produce(rb, ra)) {
+      round_store(ra, xa, lane);
+      break;
+    }
+    round_load(rb, xb, lane);
+    round_store(ra, xa, lane);
+    if (!produce(ra, rb)) {
+      round_store(rb, xb, lane);
+      break;
+    }
+    round_load(ra, xa, lane);
+    round_store(rb, xb, lane);
+  }
+}
+
+__device__ void worker_loop(DevState* st, uint32_t* jobs_done, uint32_t flags) {
+  __shared__ Stage stages[2];
+  __shared__ uint32_t s_waves_done;  // copy wavefronts that have finished (and drained) a ticket, running total
+  const uint32_t tid = threadIdx.x;
+  const uint32_t lane = tid & (kWaveLanes - 1);
+  const uint32_t wave = tid / kWaveLanes;
+  if (tid == 0) s_waves_done = 0;
+  __syncthreads();
+
+  if (wave == kCopyWaves) {
+    // ---- fetcher ----
+    // Each pass stages this workgroup's next ticket (or the exit marker) into the free LDS stage, then meets the
+    // copy wavefronts at the barrier.
+    //
+    // When to claim the next ticket number.  Numbers are served in order, so a number claimed by a workgroup
+    // that is still busy keeps its ticket waiting even if other workgroups are idle.  A fetcher therefore claims
+    // ahead of time ("eager") only while tickets are queueing up -- its previous ticket was already there at the
+    // first look -- and otherwise claims when its copy wavefronts have finished.
+    const uint32_t* stop_word = &st->stop[blockIdx.x % kStopReplicas].value;
+    uint32_t staged = 0;
+    bool eager = false;
+    const bool allow_eager = (flags & 1u) != 0;
+    const uint32_t backoff_cap = (flags >> 8) & 0xFFu;
+    for (;;) {
+      Stage* next = &stages[staged & 1];
+      if (!eager) {
+        // Wait for the copy of ticket staged-1 to finish (LDS only: no memory traffic while waiting).
+        while (__hip_atomic_load(&s_waves_done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != staged * kCopyWaves)
+          __builtin_amdgcn_s_sleep(1);
+      }
+      uint64_t t = 0;
+      if (lane == 0) t = __hip_atomic_fetch_add(&st->ticket_head, 1ull, __ATOMIC_RELAXED, SYS);
+      const uint64_t ticket = bcast64(t, 0);
+      bool give_up = false, stop_before = false, first_look = true;
+      uint32_t backoff = 1;
+      for (;;) {
+        bool stop_up = false;
+        if (try_fetch_ticket(st, stop_word, ticket, next, lane, &stop_up)) {
+          eager = first_look && allow_eager;
+          break;
+        }
+        if (stop_before) {
+          // The stop word was already up at the previous look and the ticket is still not there: the leader
+          // publishes every ticket before any stop word, so it never will be.
+          give_up = true;
+          if (lane == 0) next->go = 0;
+          break;
+        }
+        stop_before = stop_up;
+        first_look = false;
+        if (!stop_before) {
+          // Idle: look again soon at first, then back off so that a thousand idle workgroups do not load the
+          // memory system that busy ones are using.
+          for (uint32_t i = 0; i < backoff; ++i) __builtin_amdgcn_s_sleep(4);
+          if (backoff < backoff_cap) backoff <<= 1;
+        }
+      }
+      __syncthreads();  // hands `next` to the copy wavefronts, which are waiting here after their ticket
+      if (give_up) break;
+      ++staged;
+    }
+  } else {
+    // ---- copy wavefronts ----
+    for (uint32_t i = 0;; ++i) {
+      __syncthreads();  // stage i&1 is ready
+      const Stage* stage = &stages[i & 1];
+      if (stage->go == 0) break;
+      copy_ticket(stage, wave, lane);
+      drain_memory_ops();  // this wavefront's write-through stores are acknowledged
+      uint32_t arrived = 0;
+      if (lane == 0)
+        arrived = __hip_atomic_fetch_add(&s_waves_done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) + 1u;
+      // The wavefront that finishes last counts the ticket: every wavefront's payload is in memory by then.
+      if (bcast(arrived, 0) == (i + 1) * kCopyWaves) retire_ticket(st, jobs_done, stage, lane);
+    }
+  }
+}
+
+__global__ __launch_bounds__(kEngineThreads) void unpack_engine_kernel(HostCtl* ctl, DevState* st, uint32_t* jobs_done,
                                                                    uint32_t* job_target, uint32_t ring_mask,
-                                                                   uint32_t per_ticket, uint32_t spin_limit) {
+                                                                   uint32_t per_ticket, uint32_t spin_limit,
+                                                                   uint32_t flags) {
   if (blockIdx.x == 0) {
     if (threadIdx.x < kWaveLanes) leader_loop(ctl, st, jobs_done, job_target, ring_mask, per_ticket, spin_limit);
   } else {
-    worker_loop(st, jobs_done);
+    worker_loop(st, jobs_done, flags);
   }
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -377,6 +469,7 @@ struct tcpxuEngine {
   uint32_t workgroups = 0;
   uint32_t per_ticket = 0;
   uint32_t spin_limit = 0;
+  uint32_t flags = 0;  // bit 0: fetchers may claim ahead; bits 8-15: idle poll backoff cap
   hipStream_t stream = nullptr;
   hipEvent_t ev_start = nullptr, ev_stop = nullptr;
   HostCtl* ctl = nullptr;      // host address of the mapped control block
@@ -409,7 +502,7 @@ int tcpxuEngineCreate(int device, const tcpxuEngineConfig* config, tcpxuEngine**
   }
   if (cfg.descs_per_ticket == 0) {
     const char* v = getenv("TCPXU_DESCS_PER_TICKET");
-    cfg.descs_per_ticket = (v && *v) ? static_cast<uint32_t>(atoi(v)) : 8;
+    cfg.descs_per_ticket = (v && *v) ? static_cast<uint32_t>(atoi(v)) : 16;
   }
   if (cfg.descs_per_ticket == 0 || cfg.descs_per_ticket > kMaxDescsPerTicket) {
     set_error("descs_per_ticket %u must be in [1,%u]", cfg.descs_per_ticket, kMaxDescsPerTicket);
@@ -418,14 +511,16 @@ int tcpxuEngineCreate(int device, const tcpxuEngineConfig* config, tcpxuEngine**
   TCPXU_TRY(use_device(device));
   const uint32_t cus = static_cast<uint32_t>(std::max(1, device_compute_units(device)));
   if (cfg.workgroups == 0) {
-    const char* v = getenv("TCPXU_ENGINE_WGS_PER_CU");
-    const uint32_t per_cu = (v && *v) ? static_cast<uint32_t>(atoi(v)) : 6;
-    // Leave wavefront slots free on every compute unit so that other kernels (copies, the caller's own work)
-    // can still be scheduled while the engine runs.
+    // Fill the compute units, but leave a few wavefront slots free on each so that other kernels (copies, the
+    // caller's own work) can still be scheduled while the engine runs: a CU has 32 slots.
     int max_active = 0;
-    TCPXU_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&max_active, unpack_engine_kernel, kWgThreads, 0));
-    const uint32_t cap = max_active > 1 ? static_cast<uint32_t>(max_active) - 1 : 1;
-    cfg.workgroups = cus * std::min(std::max(per_cu, 1u), cap) + 1;
+    TCPXU_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&max_active, unpack_engine_kernel, kEngineThreads, 0));
+    const uint32_t waves_per_wg = kEngineThreads / kWaveLanes;
+    uint32_t per_cu = static_cast<uint32_t>(std::max(max_active, 1));
+    while (per_cu > 1 && per_cu * waves_per_wg > 28) --per_cu;
+    const char* v = getenv("TCPXU_ENGINE_WGS_PER_CU");
+    if (v && *v) per_cu = std::min(std::max(static_cast<uint32_t>(atoi(v)), 1u), static_cast<uint32_t>(std::max(max_active, 1)));
+    cfg.workgroups = cus * per_cu + 1;
   }
   if (cfg.workgroups < 2) {
     set_error("an engine needs the leader workgroup and at least one worker");
@@ -439,6 +534,13 @@ int tcpxuEngineCreate(int device, const tcpxuEngineConfig* config, tcpxuEngine**
   e->workgroups = cfg.workgroups;
   e->per_ticket = cfg.descs_per_ticket;
   e->spin_limit = cfg.spin_limit;
+  {
+    const char* ve = getenv("TCPXU_ENGINE_EAGER");
+    const char* vb = getenv("TCPXU_ENGINE_BACKOFF_CAP");
+    const uint32_t eager = (ve && *ve) ? static_cast<uint32_t>(atoi(ve)) & 1u : 0u;
+    const uint32_t cap = (vb && *vb) ? static_cast<uint32_t>(atoi(vb)) & 0xFFu : 8u;
+    e->flags = eager | (cap << 8);
+  }
   int rc = TCPXU_SUCCESS;
   do {
     void *h = nullptr, *d = nullptr;
@@ -482,8 +584,8 @@ int tcpxuEngineStart(tcpxuEngine* e) {
   e->ctl->exited = 0;
   std::atomic_thread_fence(std::memory_order_seq_cst);
   TCPXU_HIP(hipEventRecord(e->ev_start, e->stream));
-  hipLaunchKernelGGL(unpack_engine_kernel, dim3(e->workgroups), dim3(kWgThreads), 0, e->stream, e->ctl_dev, e->st,
-                     e->jobs_done, e->job_target, e->ring_entries - 1, e->per_ticket, e->spin_limit);
+  hipLaunchKernelGGL(unpack_engine_kernel, dim3(e->workgroups), dim3(kEngineThreads), 0, e->stream, e->ctl_dev, e->st,
+                     e->jobs_done, e->job_target, e->ring_entries - 1, e->per_ticket, e->spin_limit, e->flags);
   TCPXU_HIP(hipGetLastError());
   TCPXU_HIP(hipEventRecord(e->ev_stop, e->stream));
   e->launched = true;
@@ -583,6 +685,15 @@ int tcpxuEngineCompleted(tcpxuEngine* e, uint64_t* completed) {
   return TCPXU_SUCCESS;
 }
 
+int tcpxuEngineGetConfig(tcpxuEngine* e, tcpxuEngineConfig* config) {
+  if (!e || !config) return TCPXU_INVALID_ARGUMENT;
+  config->ring_entries = e->ring_entries;
+  config->workgroups = e->workgroups;
+  config->descs_per_ticket = e->per_ticket;
+  config->spin_limit = e->spin_limit;
+  return TCPXU_SUCCESS;
+}
+
 int tcpxuEngineRunning(tcpxuEngine* e, int* running) {
   if (!e || !running) return TCPXU_INVALID_ARGUMENT;
   std::lock_guard<std::mutex> lock(e->mu);
@@ -612,6 +723,20 @@ int tcpxuEngineStream(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_i
   uint8_t* hb = static_cast<uint8_t*>(e->stream_host);
   uint8_t* db = static_cast<uint8_t*>(e->stream_dev);
   memset(hb, 0, flags_bytes);
+  // Probe switch for tuning: after the ring's first lap, reuse the descriptors already in each slot.
+  const bool skip_copy = getenv("TCPXU_STREAM_SKIP_COPY") != nullptr;
+  // Probe switch for tuning: descriptors pre-staged in device memory instead of the mapped slots.
+  const bool descs_in_hbm = getenv("TCPXU_STREAM_DESCS_IN_HBM") != nullptr;
+  std::unordered_map<const void*, void*> hbm_copies;
+  if (descs_in_hbm) {
+    for (uint64_t i = 0; i < n_items; ++i) {
+      if (!items[i].n_descs || hbm_copies.count(items[i].descs_host)) continue;
+      void* d = nullptr;
+      TCPXU_HIP(hipMalloc(&d, sizeof(tcpxuLoadMeta) * items[i].n_descs));
+      TCPXU_HIP(hipMemcpy(d, items[i].descs_host, sizeof(tcpxuLoadMeta) * items[i].n_descs, hipMemcpyHostToDevice));
+      hbm_copies[items[i].descs_host] = d;  // leaked on purpose: probe only
+    }
+  }
   using clock = std::chrono::steady_clock;
   std::vector<clock::time_point> published(depth);
   int rc = TCPXU_SUCCESS;
@@ -638,9 +763,12 @@ int tcpxuEngineStream(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_i
       const uint32_t slot = static_cast<uint32_t>(next_submit % depth);
       const tcpxuStreamItem& it = items[next_submit];
       uint8_t* slot_host = hb + flags_bytes + slot_bytes * slot;
-      if (it.n_descs) memcpy(slot_host, it.descs_host, sizeof(tcpxuLoadMeta) * it.n_descs);
+      if (it.n_descs && !descs_in_hbm && !(skip_copy && next_submit >= depth))
+        memcpy(slot_host, it.descs_host, sizeof(tcpxuLoadMeta) * it.n_descs);
       published[slot] = clock::now();
-      rc = tcpxuEngineSubmit(e, it.bounce_base, it.dst_base, db + flags_bytes + slot_bytes * slot, it.n_descs,
+      const void* descs_dev = db + flags_bytes + slot_bytes * slot;
+      if (descs_in_hbm && it.n_descs) descs_dev = hbm_copies[it.descs_host];
+      rc = tcpxuEngineSubmit(e, it.bounce_base, it.dst_base, descs_dev, it.n_descs,
                              db + flag_stride * slot, next_submit + 1);
       if (rc == kTcpxuInProgress) {
         rc = TCPXU_SUCCESS;

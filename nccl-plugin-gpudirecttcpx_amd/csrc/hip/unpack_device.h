@@ -99,92 +99,111 @@ __device__ __forceinline__ void wave_copy_fragment(const uint8_t* __restrict__ s
 // A kernel that never ends gets no cache invalidate at launch and no write-back at exit, so its payload accesses
 // carry the coherence themselves: loads and stores are issued at system scope (sc0 sc1).  A load then never
 // returns a line that an XCD's L2 kept from an earlier use of a recycled bounce page, and a store is written
-// through, so that once the wavefront's store counter has drained (s_waitcnt vmcnt(0)) the bytes are where the
+// through, so that once the wavefront's memory counter has drained (s_waitcnt vmcnt(0)) the bytes are where the
 // host, a DMA engine or another kernel will read them -- no L2 write-back instruction is ever needed.
-// The loads of one round and the wait for them form a single asm block: the compiler does not track counters
-// for memory instructions it cannot see.
+typedef TCPXU_GLOBAL u32x4* gvec_ptr;
+__device__ __forceinline__ u32x4 load_vec_sys(const uint8_t* p) {
+  return __builtin_amdgcn_global_load_b128((gvec_ptr)p, "");
+}
 __device__ __forceinline__ void store_vec_sys(uint8_t* p, u32x4 v) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+  __builtin_amdgcn_global_store_b128((gvec_ptr)p, v, "");
 }
-__device__ __forceinline__ void store_byte_sys(uint8_t* p, uint32_t v) {
-  asm volatile("global_store_byte %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+__device__ __forceinline__ uint32_t load_byte_sys(const uint8_t* p) {
+  return __hip_atomic_load((const TCPXU_GLOBAL uint8_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+__device__ __forceinline__ void store_byte_sys(uint8_t* p, uint8_t v) {
+  __hip_atomic_store((TCPXU_GLOBAL uint8_t*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
-// Same contract as wave_copy_fragment.  One round moves up to 4 KiB: every lane issues the edge-byte load and
-// one or four vector loads back to back (lanes past the end re-read the fragment's last vector, which is in
-// range), waits once, then stores under its predicates.
-__device__ __forceinline__ void wave_copy_fragment_coherent(const uint8_t* __restrict__ src,
-                                                            uint8_t* __restrict__ dst, uint32_t len,
-                                                            uint32_t lane) {
-  if (len == 0) return;
-  uint32_t head = static_cast<uint32_t>(-reinterpret_cast<uintptr_t>(dst)) & 15u;
-  if (head > len) head = len;
-  const uint32_t body = len - head;
-  const uint32_t nvec = body >> 4;
-  const uint32_t tail = body & 15u;
+// One round of a wavefront's copy work: up to 4 KiB of 16-byte vectors with a 16-byte aligned destination, plus
+// the edge bytes of the fragment it belongs to (a fragment's head and tail, carried by its first round).
+// Loading and storing are separate steps so that a wavefront can issue the loads of its next round before the
+// stores of the current one: the memory counter of gfx9 retires in issue order, so waiting for the older loads
+// leaves the younger ones in flight.
+//
+// Nothing in a round is predicated.  A lane whose vector index is past the round's end is clamped to the last
+// vector for the load AND for the store: it re-reads and re-writes that vector with the very same bytes, which
+// changes nothing.  A lane without an edge byte copies the fragment's byte 0 onto itself the same way.  Every
+// round therefore issues exactly kVecPerLane + 1 loads and as many stores on every path, which lets the
+// compiler compute exact wait counts and keep the younger round in flight.
+struct CopyRound {
+  // Wave-uniform (scalar registers):
+  const uint8_t* src_vec;   // source of vector 0 of this round (any alignment)
+  uint8_t* dst_vec;         // destination of vector 0 (16-byte aligned)
+  const uint8_t* src_frag;  // first byte of the fragment
+  uint8_t* dst_frag;
+  uint32_t nvec;            // vectors in this round, 1..kVecPerRound
+  // Per lane:
+  uint32_t edge_off;        // offset of this lane's edge byte in the fragment, 0 if it has none
+};
+struct CopyRegs {
+  u32x4 r[kVecPerLane];
+  uint32_t edge_byte;
+};
 
-  uint32_t edge_off = 0;
-  bool edge = false;
-  if (lane < head) {
-    edge = true;
-    edge_off = lane;
-  } else if (lane >= 16u && lane - 16u < tail) {
-    edge = true;
-    edge_off = head + (nvec << 4) + (lane - 16u);
-  }
-  const uint8_t* edge_src = src + edge_off;  // offset 0 for lanes without an edge byte: inside the fragment
-  uint32_t edge_byte = 0;
-
-  if (nvec == 0) {
-    asm volatile(
-        "global_load_ubyte %0, %1, off sc0 sc1\n"
-        "s_waitcnt vmcnt(0)"
-        : "=&v"(edge_byte)
-        : "v"(edge_src)
-        : "memory");
-    if (edge) store_byte_sys(dst + edge_off, edge_byte);
-    return;
-  }
-
-  const uint8_t* sb = src + head;
-  uint8_t* db = dst + head;
+// Byte offset of lane's k-th vector in a round of nvec vectors, clamped to the last one.
+__device__ __forceinline__ uint32_t round_vec_offset(uint32_t nvec, int k, uint32_t lane) {
+  const uint32_t v = static_cast<uint32_t>(k) * kWaveLanes + lane;
   const uint32_t last = nvec - 1;
-  for (uint32_t base = 0; base < nvec; base += kVecPerRound) {
-    const uint32_t v0 = base + lane;
-    const uint32_t v1 = v0 + kWaveLanes, v2 = v0 + 2 * kWaveLanes, v3 = v0 + 3 * kWaveLanes;
-    const uint8_t* p0 = sb + (static_cast<size_t>(v0 < last ? v0 : last) << 4);
-    u32x4 r0, r1, r2, r3;
-    if (nvec - base <= kWaveLanes) {  // wave-uniform
-      asm volatile(
-          "global_load_ubyte %1, %3, off sc0 sc1\n"
-          "global_load_dwordx4 %0, %2, off sc0 sc1\n"
-          "s_waitcnt vmcnt(0)"
-          : "=&v"(r0), "=&v"(edge_byte)
-          : "v"(p0), "v"(edge_src)
-          : "memory");
-      if (v0 < nvec) store_vec_sys(db + (static_cast<size_t>(v0) << 4), r0);
-    } else {
-      const uint8_t* p1 = sb + (static_cast<size_t>(v1 < last ? v1 : last) << 4);
-      const uint8_t* p2 = sb + (static_cast<size_t>(v2 < last ? v2 : last) << 4);
-      const uint8_t* p3 = sb + (static_cast<size_t>(v3 < last ? v3 : last) << 4);
-      asm volatile(
-          "global_load_ubyte %4, %9, off sc0 sc1\n"
-          "global_load_dwordx4 %0, %5, off sc0 sc1\n"
-          "global_load_dwordx4 %1, %6, off sc0 sc1\n"
-          "global_load_dwordx4 %2, %7, off sc0 sc1\n"
-          "global_load_dwordx4 %3, %8, off sc0 sc1\n"
-          "s_waitcnt vmcnt(0)"
-          : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3), "=&v"(edge_byte)
-          : "v"(p0), "v"(p1), "v"(p2), "v"(p3), "v"(edge_src)
-          : "memory");
-      if (v0 < nvec) store_vec_sys(db + (static_cast<size_t>(v0) << 4), r0);
-      if (v1 < nvec) store_vec_sys(db + (static_cast<size_t>(v1) << 4), r1);
-      if (v2 < nvec) store_vec_sys(db + (static_cast<size_t>(v2) << 4), r2);
-      if (v3 < nvec) store_vec_sys(db + (static_cast<size_t>(v3) << 4), r3);
-    }
-  }
-  if (edge) store_byte_sys(dst + edge_off, edge_byte);
+  return (v < last ? v : last) << 4;
 }
+
+__device__ __forceinline__ void round_load(const CopyRound& c, CopyRegs& x, uint32_t lane) {
+  x.edge_byte = load_byte_sys(c.src_frag + c.edge_off);
+#pragma unroll
+  for (int k = 0; k < kVecPerLane; ++k) x.r[k] = load_vec_sys(c.src_vec + round_vec_offset(c.nvec, k, lane));
+}
+
+__device__ __forceinline__ void round_store(const CopyRound& c, const CopyRegs& x, uint32_t lane) {
+#pragma unroll
+  for (int k = 0; k < kVecPerLane; ++k) store_vec_sys(c.dst_vec + round_vec_offset(c.nvec, k, lane), x.r[k]);
+  store_byte_sys(c.dst_frag + c.edge_off, static_cast<uint8_t>(x.edge_byte));
+}
+
+// A fragment too short to contain one destination-aligned vector (at most 30 bytes) is copied byte per lane,
+// outside the round pipeline.
+__device__ __forceinline__ bool fragment_is_tiny(const uint8_t* dst, uint32_t len) {
+  const uint32_t head = static_cast<uint32_t>(-reinterpret_cast<uintptr_t>(dst)) & 15u;
+  return len < head + 16u;
+}
+__device__ __forceinline__ void copy_tiny_fragment(const uint8_t* src, uint8_t* dst, uint32_t len, uint32_t lane) {
+  if (lane < len) store_byte_sys(dst + lane, static_cast<uint8_t>(load_byte_sys(src + lane)));
+}
+
+// Splits a fragment that is not tiny (src, dst, len wave-uniform) into rounds of 1..kVecPerRound vectors.  Fragments of the wire format (at most
+// 4 KiB) have exactly one round; later rounds of a longer fragment repeat the edge copy with the same bytes.
+struct FragmentRounds {
+  uint32_t nvec_left = 0;  // vectors not yet handed out
+
+  __device__ __forceinline__ CopyRound first_round(const uint8_t* src, uint8_t* dst, uint32_t len, uint32_t lane) {
+    uint32_t head = static_cast<uint32_t>(-reinterpret_cast<uintptr_t>(dst)) & 15u;
+    if (head > len) head = len;
+    const uint32_t body = len - head;
+    const uint32_t tail = body & 15u;
+    const uint32_t nvec = body >> 4;
+    CopyRound c;
+    c.src_frag = src;
+    c.dst_frag = dst;
+    c.src_vec = src + head;
+    c.dst_vec = dst + head;
+    // Lanes [0,head) carry the head, lanes [16,16+tail) the tail (both < 16 bytes); every other lane gets 0.
+    c.edge_off = 0;
+    if (lane < head) c.edge_off = lane;
+    else if (lane >= 16u && lane - 16u < tail) c.edge_off = head + (nvec << 4) + (lane - 16u);
+    c.nvec = nvec < kVecPerRound ? nvec : kVecPerRound;
+    nvec_left = nvec - c.nvec;
+    return c;
+  }
+  __device__ __forceinline__ bool more() const { return nvec_left != 0; }
+  __device__ __forceinline__ CopyRound next_round(const CopyRound& prev) {
+    CopyRound c = prev;
+    c.src_vec = prev.src_vec + (static_cast<size_t>(prev.nvec) << 4);
+    c.dst_vec = prev.dst_vec + (static_cast<size_t>(prev.nvec) << 4);
+    c.nvec = nvec_left < kVecPerRound ? nvec_left : kVecPerRound;
+    nvec_left -= c.nvec;
+    return c;
+  }
+};
 
 // The 8 XCDs of an MI355X receive workgroups round-robin by workgroup id and each has its own L2.  This maps a
 // workgroup id to a work-item index such that every XCD walks one contiguous eighth of the index space:
