@@ -12,7 +12,7 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_DIR = os.path.join(_HERE, "lib")
+LIB_DIR = os.environ.get("TCPX_AMD_LIB_DIR") or os.path.join(_HERE, "lib")  # override: an alternative build
 REPO_ROOT = os.path.dirname(_HERE)
 
 SUCCESS, DEVICE_ERROR, SYSTEM_ERROR, INTERNAL_ERROR, INVALID_ARGUMENT, INVALID_USAGE = 0, 1, 2, 3, 4, 5

@@ -43,6 +43,11 @@
 #include "tcpx_unpack_hip.h"
 #include "unpack_device.h"
 
+// One round in flight per wavefront: measured faster than two (half the registers, more wavefronts resident).
+#ifndef TCPXU_ENGINE_TWO_ROUNDS
+#define TCPXU_ENGINE_TWO_ROUNDS false
+#endif
+
 namespace tcpxu {
 namespace {
 
@@ -240,7 +245,10 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
 // while the copy wavefronts move ticket i, it claims a number, polls that ticket's slot and pulls the ticket's
 // descriptors over PCIe into the other LDS stage.  Copy wavefronts therefore never wait for PCIe: between two
 // tickets they only meet the fetcher at one barrier.  The copy wavefront that finishes a ticket last counts it.
-constexpr uint32_t kCopyWaves = 8;
+#ifndef TCPXU_ENGINE_COPY_WAVES
+#define TCPXU_ENGINE_COPY_WAVES 8
+#endif
+constexpr uint32_t kCopyWaves = TCPXU_ENGINE_COPY_WAVES;
 constexpr uint32_t kEngineThreads = (kCopyWaves + 1) * kWaveLanes;
 
 struct Stage {
@@ -296,64 +304,15 @@ __device__ void retire_ticket(DevState* st, uint32_t* jobs_done, const Stage* st
   }
 }
 
-// Copy wavefront `wave` of kCopyWaves: fragments wave, wave + kCopyWaves, ... of the staged ticket, with the
-// loads of the next round issued before the stores of the current one.  Two register sets alternate so that no
-// register is copied while a load into it is in flight.
+// Copy wavefront `wave` of kCopyWaves: fragments wave, wave + kCopyWaves, ... of the staged ticket.
 __device__ void copy_ticket(const Stage* stage, uint32_t wave, uint32_t lane) {
-  // Everything that describes a fragment is wave-uniform; saying so keeps it in scalar registers and leaves
-  // the vector registers to the payload in flight.
   auto uniform = [](uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(v)); };
   const uint8_t* bounce = reinterpret_cast<const uint8_t*>((static_cast<uint64_t>(uniform(stage->payload[1])) << 32) |
                                                            uniform(stage->payload[0]));
   uint8_t* dst =
       reinterpret_cast<uint8_t*>((static_cast<uint64_t>(uniform(stage->payload[3])) << 32) | uniform(stage->payload[2]));
   const uint32_t n = uniform(stage->payload[10]) & 0xFFu;
-  wave = uniform(wave);
-  uint32_t j = wave;
-  FragmentRounds fr;
-  // Next round of this wavefront's work, or false when there is none.  `prev` is the round before it.
-  auto produce = [&](CopyRound& out, const CopyRound& prev) -> bool {
-    if (fr.more()) {
-      out = fr.next_round(prev);
-      return true;
-    }
-    while (j < n) {
-      const tcpxuLoadMeta d = stage->desc[j];
-      j += kCopyWaves;
-      const uint32_t len = __builtin_amdgcn_readfirstlane(d.len);
-      if (len == 0) continue;
-      const uint32_t so = __builtin_amdgcn_readfirstlane(d.src_off);
-      const uint32_t dlo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(d.dst_off));
-      const uint32_t dhi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(d.dst_off >> 32));
-      const uint8_t* fsrc = bounce + so;
-      uint8_t* fdst = dst + ((static_cast<uint64_t>(dhi) << 32) | dlo);
-      if (fragment_is_tiny(fdst, len)) {
-        copy_tiny_fragment(fsrc, fdst, len, lane);
-        continue;
-      }
-      out = fr.first_round(fsrc, fdst, len, lane);
-      return true;
-    }
-    return false;
-  };
-  CopyRound ra, rb;
-  CopyRegs xa, xb;
-  if (!produce(ra, ra)) return;
-  round_load(ra, xa, lane);
-  for (;;) {
-    if (!produce(rb, ra)) {
-      round_store(ra, xa, lane);
-      break;
-    }
-    round_load(rb, xb, lane);
-    round_store(ra, xa, lane);
-    if (!produce(ra, rb)) {
-      round_store(rb, xb, lane);
-      break;
-    }
-    round_load(ra, xa, lane);
-    round_store(rb, xb, lane);
-  }
+  wave_copy_descriptors<TCPXU_ENGINE_TWO_ROUNDS>(stage->desc, n, wave, kCopyWaves, bounce, dst, lane);
 }
 
 __device__ void worker_loop(DevState* st, uint32_t* jobs_done, uint32_t flags) {

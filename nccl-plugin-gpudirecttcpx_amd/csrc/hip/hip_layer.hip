@@ -14,6 +14,11 @@
 #include "tcpx_unpack_hip.h"
 #include "unpack_device.h"
 
+// One round in flight per wavefront: measured faster than two (half the registers, more wavefronts resident).
+#ifndef TCPXU_BATCH_TWO_ROUNDS
+#define TCPXU_BATCH_TWO_ROUNDS false
+#endif
+
 namespace tcpxu {
 
 thread_local char g_last_error[512] = "";
@@ -31,7 +36,6 @@ constexpr uint32_t kMaxDescsPerWg = 64;
 
 // Launch-per-batch unpack.  A workgroup takes `descs_per_wg` consecutive descriptors, stages them in LDS with
 // one 16-byte load per thread, then its four wavefronts take fragments in turn.
-template <bool kCoherent>
 __global__ __launch_bounds__(kWgThreads) void unpack_batch_kernel(const uint8_t* __restrict__ bounce,
                                                                    uint8_t* __restrict__ dst,
                                                                    const tcpxuLoadMeta* __restrict__ descs,
@@ -54,40 +58,13 @@ __global__ __launch_bounds__(kWgThreads) void unpack_batch_kernel(const uint8_t*
         *reinterpret_cast<u32x4*>(&staged[tid]) = raw;
       }
       __syncthreads();
-      for (uint32_t j = wave; j < cnt; j += kWavesPerWg) {
-        const tcpxuLoadMeta d = staged[j];
-        const uint32_t len = __builtin_amdgcn_readfirstlane(d.len);
-        const uint32_t so = __builtin_amdgcn_readfirstlane(d.src_off);
-        const uint32_t dlo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(d.dst_off));
-        const uint32_t dhi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(d.dst_off >> 32));
-        const uint64_t doff = (static_cast<uint64_t>(dhi) << 32) | dlo;
-        if constexpr (kCoherent) {
-          if (len != 0) {
-            if (fragment_is_tiny(dst + doff, len)) {
-              copy_tiny_fragment(bounce + so, dst + doff, len, lane);
-            } else {
-              FragmentRounds fr;
-              CopyRound c = fr.first_round(bounce + so, dst + doff, len, lane);
-              for (;;) {
-                CopyRegs x;
-                round_load(c, x, lane);
-                round_store(c, x, lane);
-                if (!fr.more()) break;
-                c = fr.next_round(c);
-              }
-            }
-          }
-        } else {
-          wave_copy_fragment(bounce + so, dst + doff, len, lane);
-        }
-      }
+      wave_copy_descriptors<TCPXU_BATCH_TWO_ROUNDS>(staged, cnt, wave, kWavesPerWg, bounce, dst, lane);
       __syncthreads();
     }
   }
 }
 
-// Plain streaming copy, 64 bytes per thread per step: the yardstick for what a copy kernel reaches here.
-template <bool kCoherent>
+// Plain copy, 64 bytes per thread per step: the yardstick for what a copy kernel reaches here.
 __global__ __launch_bounds__(kWgThreads) void copy_kernel(uint8_t* __restrict__ dst, const uint8_t* __restrict__ src,
                                                           uint64_t n_vec) {
   const uint64_t stride = static_cast<uint64_t>(gridDim.x) * kWgThreads;
@@ -97,15 +74,12 @@ __global__ __launch_bounds__(kWgThreads) void copy_kernel(uint8_t* __restrict__ 
 #pragma unroll
     for (int k = 0; k < kVecPerLane; ++k) {
       const uint64_t v = base + static_cast<uint64_t>(k) * kWgThreads + threadIdx.x;
-      if (v < n_vec) r[k] = kCoherent ? load_vec_sys(src + (v << 4)) : load_vec(src + (v << 4));
+      if (v < n_vec) r[k] = load_vec_sys(src + (v << 4));
     }
 #pragma unroll
     for (int k = 0; k < kVecPerLane; ++k) {
       const uint64_t v = base + static_cast<uint64_t>(k) * kWgThreads + threadIdx.x;
-      if (v < n_vec) {
-        if (kCoherent) store_vec_sys(dst + (v << 4), r[k]);
-        else store_vec(dst + (v << 4), r[k]);
-      }
+      if (v < n_vec) store_vec_sys(dst + (v << 4), r[k]);
     }
   }
 }
@@ -278,16 +252,9 @@ static int launch_batch(int device, const void* bounce_base, void* dst_base, con
   uint32_t dpw, grid;
   uint64_t batches;
   batch_geometry(device, n_descs, &dpw, &batches, &grid);
-  // Probe switch: the system-scope access variant that the persistent engine uses, in a plain launch.
-  static const bool coherent = getenv("TCPXU_BATCH_COHERENT") != nullptr;
-  if (coherent)
-    hipLaunchKernelGGL(unpack_batch_kernel<true>, dim3(grid), dim3(kWgThreads), 0, stream,
-                       static_cast<const uint8_t*>(bounce_base), static_cast<uint8_t*>(dst_base), descs, n_descs,
-                       dpw, batches);
-  else
-    hipLaunchKernelGGL(unpack_batch_kernel<false>, dim3(grid), dim3(kWgThreads), 0, stream,
-                       static_cast<const uint8_t*>(bounce_base), static_cast<uint8_t*>(dst_base), descs, n_descs,
-                       dpw, batches);
+  hipLaunchKernelGGL(unpack_batch_kernel, dim3(grid), dim3(kWgThreads), 0, stream,
+                     static_cast<const uint8_t*>(bounce_base), static_cast<uint8_t*>(dst_base), descs, n_descs, dpw,
+                     batches);
   TCPXU_HIP(hipGetLastError());
   return TCPXU_SUCCESS;
 }
@@ -390,11 +357,7 @@ int tcpxuCopyKernelTimed(int device, void* dst, const void* src, size_t bytes, i
       stream, warmup, iters, mean_us,
       [](void* p, hipStream_t s) {
         auto* c = static_cast<CopyLaunch*>(p);
-        static const bool coherent = getenv("TCPXU_BATCH_COHERENT") != nullptr;
-        if (coherent)
-          hipLaunchKernelGGL(copy_kernel<true>, dim3(c->grid), dim3(kWgThreads), 0, s, c->dst, c->src, c->n_vec);
-        else
-          hipLaunchKernelGGL(copy_kernel<false>, dim3(c->grid), dim3(kWgThreads), 0, s, c->dst, c->src, c->n_vec);
+        hipLaunchKernelGGL(copy_kernel, dim3(c->grid), dim3(kWgThreads), 0, s, c->dst, c->src, c->n_vec);
         if (hipGetLastError() != hipSuccess) {
           set_error("copy kernel launch failed");
           return TCPXU_DEVICE_ERROR;

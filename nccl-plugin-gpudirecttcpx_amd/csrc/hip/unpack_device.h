@@ -1,10 +1,12 @@
-// Device-side building blocks of the gfx950 unpack kernels: how one 64-lane wavefront moves one fragment.
+// Device-side building blocks of the gfx950 unpack kernels: how one 64-lane wavefront moves fragments.
 //
 // A fragment is `len` bytes (at most one 4 KiB bounce page in practice) with arbitrary byte alignment on both
-// sides.  The copy is organised around the DESTINATION: a byte-wise head brings the destination to a 16-byte
-// boundary, the body is written with aligned 16-byte vector stores, a byte-wise tail finishes.  Source vectors
-// are fetched with 16-byte loads at whatever alignment results (gfx950 global loads accept any alignment), so
-// no realignment in registers is needed.  This is a pure bandwidth copy: no MFMA, no LDS for payload.
+// sides.  The copy is organised around the DESTINATION: the body is written with aligned 16-byte vector stores
+// that cover whole 128-byte lines wherever a neighbouring fragment continues the line, and byte-wise heads and
+// tails remain only at the ends of a run of fragments.  Source vectors are fetched with 16-byte loads at
+// whatever alignment results (gfx950 global loads accept any alignment), so no realignment in registers is
+// needed except for the one vector that straddles two fragments.  This is a pure bandwidth copy: no MFMA, no
+// LDS for payload.
 #ifndef TCPXU_UNPACK_DEVICE_H_
 #define TCPXU_UNPACK_DEVICE_H_
 
@@ -27,80 +29,17 @@ typedef u32x4 u32x4_any __attribute__((aligned(1)));  // 16-byte vector at any b
 
 // Payload always lives in global memory (the arena and the caller's receive buffer), so every payload access
 // is cast to the global address space: the compiler then emits global_* instead of flat_* instructions even
-// where the address arrives as an integer.  Payload is read once and written once, so both sides carry the
-// non-temporal hint.
+// where the address arrives as an integer.
 #define TCPXU_GLOBAL __attribute__((address_space(1)))
-__device__ __forceinline__ u32x4 load_vec(const uint8_t* p) {
-  return __builtin_nontemporal_load((const TCPXU_GLOBAL u32x4_any*)p);
-}
-__device__ __forceinline__ void store_vec(uint8_t* p, u32x4 v) {
-  __builtin_nontemporal_store(v, (TCPXU_GLOBAL u32x4*)p);
-}
-__device__ __forceinline__ uint8_t load_byte(const uint8_t* p) { return *(const TCPXU_GLOBAL uint8_t*)p; }
-__device__ __forceinline__ void store_byte(uint8_t* p, uint8_t v) { *(TCPXU_GLOBAL uint8_t*)p = v; }
 
-// Copies src[0,len) to dst[0,len) with the 64 lanes of the calling wavefront.  `len`, `src` and `dst` must be
-// wave-uniform.  Writes exactly [dst, dst+len): bytes on either side are never touched.
-__device__ __forceinline__ void wave_copy_fragment(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
-                                                   uint32_t len, uint32_t lane) {
-  if (len == 0) return;
-  uint32_t head = static_cast<uint32_t>(-reinterpret_cast<uintptr_t>(dst)) & 15u;
-  if (head > len) head = len;
-  const uint32_t body = len - head;
-  const uint32_t nvec = body >> 4;
-  const uint32_t tail = body & 15u;
-
-  // Edge bytes: lanes [0,head) carry the head, lanes [16,16+tail) the tail (both < 16 bytes).
-  uint32_t edge_off = 0;
-  bool edge = false;
-  if (lane < head) {
-    edge = true;
-    edge_off = lane;
-  } else if (lane >= 16u && lane - 16u < tail) {
-    edge = true;
-    edge_off = head + (nvec << 4) + (lane - 16u);
-  }
-  uint8_t edge_byte = 0;
-  if (edge) edge_byte = load_byte(src + edge_off);
-
-  const uint8_t* sb = src + head;
-  uint8_t* db = dst + head;
-  uint32_t base = 0;
-  // Full rounds: every lane moves four vectors, all four loads in flight before the first store.
-  for (; base + kVecPerRound <= nvec; base += kVecPerRound) {
-    u32x4 r[kVecPerLane];
-#pragma unroll
-    for (int k = 0; k < kVecPerLane; ++k)
-      r[k] = load_vec(sb + (static_cast<size_t>(base + static_cast<uint32_t>(k) * kWaveLanes + lane) << 4));
-#pragma unroll
-    for (int k = 0; k < kVecPerLane; ++k)
-      store_vec(db + (static_cast<size_t>(base + static_cast<uint32_t>(k) * kWaveLanes + lane) << 4), r[k]);
-  }
-  // Last, partial round.  Loads are unconditional (lanes past the end re-read the last vector, which is inside
-  // the fragment) so that all of them are issued back to back; only the stores are predicated.
-  if (base < nvec) {
-    u32x4 r[kVecPerLane];
-    const uint32_t last = nvec - 1;
-#pragma unroll
-    for (int k = 0; k < kVecPerLane; ++k) {
-      const uint32_t v = base + static_cast<uint32_t>(k) * kWaveLanes + lane;
-      r[k] = load_vec(sb + (static_cast<size_t>(v < last ? v : last) << 4));
-    }
-#pragma unroll
-    for (int k = 0; k < kVecPerLane; ++k) {
-      const uint32_t v = base + static_cast<uint32_t>(k) * kWaveLanes + lane;
-      if (v < nvec) store_vec(db + (static_cast<size_t>(v) << 4), r[k]);
-    }
-  }
-  if (edge) store_byte(dst + edge_off, edge_byte);
-}
-
-// ---- coherent variant, for the persistent engine ------------------------------------------------------------------
-// A kernel that never ends gets no cache invalidate at launch and no write-back at exit, so its payload accesses
-// carry the coherence themselves: loads and stores are issued at system scope (sc0 sc1).  A load then never
-// returns a line that an XCD's L2 kept from an earlier use of a recycled bounce page, and a store is written
-// through, so that once the wavefront's memory counter has drained (s_waitcnt vmcnt(0)) the bytes are where the
-// host, a DMA engine or another kernel will read them -- no L2 write-back instruction is ever needed.
+// ---- the copy path ------------------------------------------------------------------------------------------------
+// Scope of the payload accesses.  A kernel that never ends gets no cache invalidate at launch and no write-back
+// at exit, so its payload accesses carry the coherence themselves: loads and stores are issued at system scope
+// (sc0 sc1).  A load then never returns a line that an XCD's L2 kept from an earlier use of a recycled bounce
+// page, and a store is written through, so that once the wavefront's memory counter has drained
+// (s_waitcnt vmcnt(0)) the bytes are where the host, a DMA engine or another kernel will read them -- no L2
+// write-back instruction is ever needed.  Plain launches use the same accesses: measured here they stream at
+// least as fast as cached non-temporal ones.
 typedef TCPXU_GLOBAL u32x4* gvec_ptr;
 __device__ __forceinline__ u32x4 load_vec_sys(const uint8_t* p) {
   return __builtin_amdgcn_global_load_b128((gvec_ptr)p, "");
@@ -115,29 +54,65 @@ __device__ __forceinline__ void store_byte_sys(uint8_t* p, uint8_t v) {
   __hip_atomic_store((TCPXU_GLOBAL uint8_t*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
-// One round of a wavefront's copy work: up to 4 KiB of 16-byte vectors with a 16-byte aligned destination, plus
-// the edge bytes of the fragment it belongs to (a fragment's head and tail, carried by its first round).
+// Destination lines.  HBM with ECC punishes a 128-byte line that arrives as two partial writes, and with
+// write-through stores no cache merges them.  Consecutive fragments of a message land back to back in the
+// destination at arbitrary byte offsets, so almost every fragment boundary falls inside a line.  Rule: a line
+// belongs to the fragment that holds its first byte.  The wavefront that copies fragment A also writes the rest
+// of A's last line, taking those bytes from the source of the next fragment B, and the wavefront that copies B
+// starts at B's first full line.  Every line inside a run of fragments is then written whole, by one wavefront.
+// Both owners decide with the same inputs whether the rule applies to a boundary:
+constexpr uint32_t kLineBytes = 128;
+constexpr uint32_t kShareMinLen = 256;  // shorter fragments keep their own partial lines
+__device__ __forceinline__ bool shares_line(uint64_t dst_a, uint32_t len_a, uint64_t dst_b, uint32_t len_b) {
+  return dst_a + len_a == dst_b && len_a >= kShareMinLen && len_b >= kShareMinLen &&
+         ((dst_a + len_a) & (kLineBytes - 1)) != 0;
+}
+
+// 16 bytes starting at byte `shift` (0..16) of the 32 bytes a:b.
+__device__ __forceinline__ u32x4 extract16(u32x4 a, u32x4 b, uint32_t shift) {
+  const uint32_t q = shift >> 2, r = shift & 3u;
+  const uint32_t w[9] = {a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3], 0u};
+  uint32_t sel[5];
+#pragma unroll
+  for (int k = 0; k < 5; ++k)
+    sel[k] = q == 0 ? w[k] : q == 1 ? w[k + 1] : q == 2 ? w[k + 2] : q == 3 ? w[k + 3] : w[k + 4];
+  u32x4 out;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) out[d] = __builtin_amdgcn_alignbyte(sel[d + 1], sel[d], r);
+  return out;
+}
+
+// One round of a wavefront's copy work: up to 4 KiB of 16-byte vectors with a 16-byte aligned destination, the
+// edge bytes of the fragment (a head and a tail of fewer than 16 bytes where the fragment keeps its own partial
+// lines), and the shared last line (eight vectors, each assembled from up to two sources).
 // Loading and storing are separate steps so that a wavefront can issue the loads of its next round before the
 // stores of the current one: the memory counter of gfx9 retires in issue order, so waiting for the older loads
 // leaves the younger ones in flight.
 //
 // Nothing in a round is predicated.  A lane whose vector index is past the round's end is clamped to the last
 // vector for the load AND for the store: it re-reads and re-writes that vector with the very same bytes, which
-// changes nothing.  A lane without an edge byte copies the fragment's byte 0 onto itself the same way.  Every
-// round therefore issues exactly kVecPerLane + 1 loads and as many stores on every path, which lets the
-// compiler compute exact wait counts and keep the younger round in flight.
+// changes nothing.  A lane without an edge byte copies the fragment's byte 0 onto itself the same way, and a
+// round without a shared line repeats its vector 0 in its place.  Every round therefore issues exactly the
+// same loads and stores on every path, which lets the compiler compute exact wait counts and keep the younger
+// round in flight.
 struct CopyRound {
   // Wave-uniform (scalar registers):
   const uint8_t* src_vec;   // source of vector 0 of this round (any alignment)
   uint8_t* dst_vec;         // destination of vector 0 (16-byte aligned)
   const uint8_t* src_frag;  // first byte of the fragment
   uint8_t* dst_frag;
+  const uint8_t* src_next;  // first byte of the next fragment's source if the last line is shared, else src_frag
   uint32_t nvec;            // vectors in this round, 1..kVecPerRound
+  uint32_t frag_len;
+  uint32_t line_off;        // offset of the shared last line from dst_frag
+  bool share_next;          // this wavefront completes its last line out of the next fragment
   // Per lane:
   uint32_t edge_off;        // offset of this lane's edge byte in the fragment, 0 if it has none
 };
 struct CopyRegs {
   u32x4 r[kVecPerLane];
+  u32x4 line_a, line_b;
+  uint32_t tail_dword;
   uint32_t edge_byte;
 };
 
@@ -148,15 +123,90 @@ __device__ __forceinline__ uint32_t round_vec_offset(uint32_t nvec, int k, uint3
   return (v < last ? v : last) << 4;
 }
 
+// What a lane does for the shared last line: vector (lane & 7) of the line is bytes [shift, shift+16) of
+// A:B with A = 16 bytes at src_frag + off_a and B = 16 bytes at src_next + off_b.
+struct LineLane {
+  uint32_t off_a, off_b, shift, dst_off;
+};
+__device__ __forceinline__ LineLane line_lane(const CopyRound& c, uint32_t lane) {
+  LineLane l;
+  if (c.share_next) {  // wave-uniform
+    const uint32_t x = c.line_off + ((lane & 7u) << 4);  // this vector's offset from the fragment's start
+    const int32_t own = static_cast<int32_t>(c.frag_len) - static_cast<int32_t>(x);  // bytes still in this fragment
+    l.dst_off = x;
+    if (own >= 16) {  // entirely this fragment
+      l.off_a = x;
+      l.off_b = 0;
+      l.shift = 0;
+    } else if (own <= 0) {  // entirely the next fragment
+      l.off_a = c.frag_len - 16u;
+      l.off_b = static_cast<uint32_t>(-own);
+      l.shift = 16;
+    } else {  // the last `own` bytes of this fragment, then the first bytes of the next
+      l.off_a = c.frag_len - 16u;
+      l.off_b = 0;
+      l.shift = 16u - static_cast<uint32_t>(own);
+    }
+  } else {  // repeat vector 0 of the round
+    l.dst_off = static_cast<uint32_t>(c.dst_vec - c.dst_frag);
+    l.off_a = l.dst_off;
+    l.off_b = l.dst_off;
+    l.shift = 0;
+  }
+  return l;
+}
+
+// Source realignment.  A 16-byte load whose address is not a multiple of 4 is split by the memory pipeline and
+// runs at roughly two thirds of the rate of one that is (a multiple of 4 that is not a multiple of 16 costs
+// nothing).  Source and destination of a fragment are misaligned against each other by an arbitrary number of
+// bytes, and the destination decides where vectors start, so the source address of a vector is arbitrary.  The
+// round therefore loads from the 4-byte aligned address just below (`skew` = 0..3 bytes below, the same for
+// every vector of the round) and shifts the bytes into place in registers: a vector is bytes [skew, skew+16)
+// of its own four dwords plus one more dword, and that fifth dword is the first dword of the next vector --
+// which the neighbouring lane holds.  Only the round's last vector has no neighbour; its fifth dword comes
+// from one extra 4-byte load.
+__device__ __forceinline__ uint32_t load_dword_sys(const uint8_t* p) {
+  return __hip_atomic_load((const TCPXU_GLOBAL uint32_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 __device__ __forceinline__ void round_load(const CopyRound& c, CopyRegs& x, uint32_t lane) {
+  const LineLane l = line_lane(c, lane);
+  const uint32_t skew = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(c.src_vec)) & 3u;
+  const uint8_t* base4 = c.src_vec - skew;
   x.edge_byte = load_byte_sys(c.src_frag + c.edge_off);
 #pragma unroll
-  for (int k = 0; k < kVecPerLane; ++k) x.r[k] = load_vec_sys(c.src_vec + round_vec_offset(c.nvec, k, lane));
+  for (int k = 0; k < kVecPerLane; ++k) x.r[k] = load_vec_sys(base4 + round_vec_offset(c.nvec, k, lane));
+  // The dword after the last vector's four.  With skew 0 nothing of it is used, and it may lie outside the
+  // fragment (even outside the arena), so the last vector's own last dword is read instead.  With skew > 0 it
+  // starts inside the fragment, and an aligned dword never leaves the 4 KiB page it starts in.
+  x.tail_dword = load_dword_sys(base4 + ((c.nvec - 1) << 4) + (skew != 0 ? 16u : 12u));
+  x.line_a = load_vec_sys(c.src_frag + l.off_a);
+  x.line_b = load_vec_sys(c.src_next + l.off_b);
 }
 
 __device__ __forceinline__ void round_store(const CopyRound& c, const CopyRegs& x, uint32_t lane) {
+  const LineLane l = line_lane(c, lane);
+  const uint32_t skew = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(c.src_vec)) & 3u;
+  const uint32_t last = c.nvec - 1;
 #pragma unroll
-  for (int k = 0; k < kVecPerLane; ++k) store_vec_sys(c.dst_vec + round_vec_offset(c.nvec, k, lane), x.r[k]);
+  for (int k = 0; k < kVecPerLane; ++k) {
+    // First dword of the next vector: lane+1 of this register, or lane 0 of the next register for lane 63.
+    uint32_t next0 = static_cast<uint32_t>(
+        __builtin_amdgcn_ds_bpermute(static_cast<int>(((lane + 1u) & 63u) << 2), static_cast<int>(x.r[k][0])));
+    if (k + 1 < kVecPerLane) {
+      const uint32_t wrap = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(x.r[k + 1 < kVecPerLane ? k + 1 : k][0]), 0));
+      if (lane == 63u) next0 = wrap;
+    }
+    const uint32_t v = static_cast<uint32_t>(k) * kWaveLanes + lane;
+    const uint32_t w4 = v < last ? next0 : x.tail_dword;  // the last vector and its clamped repeats use the tail
+    u32x4 out;
+    out[0] = __builtin_amdgcn_alignbyte(x.r[k][1], x.r[k][0], skew);
+    out[1] = __builtin_amdgcn_alignbyte(x.r[k][2], x.r[k][1], skew);
+    out[2] = __builtin_amdgcn_alignbyte(x.r[k][3], x.r[k][2], skew);
+    out[3] = __builtin_amdgcn_alignbyte(w4, x.r[k][3], skew);
+    store_vec_sys(c.dst_vec + round_vec_offset(c.nvec, k, lane), out);
+  }
+  store_vec_sys(c.dst_frag + l.dst_off, extract16(x.line_a, x.line_b, l.shift));
   store_byte_sys(c.dst_frag + c.edge_off, static_cast<uint8_t>(x.edge_byte));
 }
 
@@ -170,26 +220,45 @@ __device__ __forceinline__ void copy_tiny_fragment(const uint8_t* src, uint8_t* 
   if (lane < len) store_byte_sys(dst + lane, static_cast<uint8_t>(load_byte_sys(src + lane)));
 }
 
-// Splits a fragment that is not tiny (src, dst, len wave-uniform) into rounds of 1..kVecPerRound vectors.  Fragments of the wire format (at most
-// 4 KiB) have exactly one round; later rounds of a longer fragment repeat the edge copy with the same bytes.
+// Splits a fragment that is not tiny (all arguments wave-uniform) into rounds of 1..kVecPerRound vectors.
+// Fragments of the wire format (at most 4 KiB) have exactly one round; later rounds of a longer fragment repeat
+// the edge bytes and the shared line with the same bytes.
+//   share_prev  the fragment's first partial line is written by the owner of the previous fragment
+//   share_next  this owner completes the fragment's last line from src_next, the next fragment's source
 struct FragmentRounds {
   uint32_t nvec_left = 0;  // vectors not yet handed out
 
-  __device__ __forceinline__ CopyRound first_round(const uint8_t* src, uint8_t* dst, uint32_t len, uint32_t lane) {
-    uint32_t head = static_cast<uint32_t>(-reinterpret_cast<uintptr_t>(dst)) & 15u;
-    if (head > len) head = len;
-    const uint32_t body = len - head;
-    const uint32_t tail = body & 15u;
-    const uint32_t nvec = body >> 4;
+  __device__ __forceinline__ CopyRound first_round(const uint8_t* src, uint8_t* dst, uint32_t len, bool share_prev,
+                                                   bool share_next, const uint8_t* src_next, uint32_t lane) {
+    const uintptr_t d = reinterpret_cast<uintptr_t>(dst);
+    uint32_t head = 0, start_off;  // start_off: offset of vector 0 from dst
+    if (share_prev) {
+      start_off = static_cast<uint32_t>(-d) & (kLineBytes - 1);
+    } else {
+      head = static_cast<uint32_t>(-d) & 15u;
+      start_off = head;
+    }
+    uint32_t tail = 0, end_off;  // end_off: offset of the end of the last vector from dst
+    if (share_next) {
+      end_off = len - (static_cast<uint32_t>(d + len) & (kLineBytes - 1));
+    } else {
+      end_off = start_off + ((len - start_off) & ~15u);
+      tail = len - end_off;
+    }
+    const uint32_t nvec = (end_off - start_off) >> 4;
     CopyRound c;
     c.src_frag = src;
     c.dst_frag = dst;
-    c.src_vec = src + head;
-    c.dst_vec = dst + head;
+    c.src_vec = src + start_off;
+    c.dst_vec = dst + start_off;
+    c.src_next = share_next ? src_next : src;
+    c.frag_len = len;
+    c.line_off = end_off;
+    c.share_next = share_next;
     // Lanes [0,head) carry the head, lanes [16,16+tail) the tail (both < 16 bytes); every other lane gets 0.
     c.edge_off = 0;
     if (lane < head) c.edge_off = lane;
-    else if (lane >= 16u && lane - 16u < tail) c.edge_off = head + (nvec << 4) + (lane - 16u);
+    else if (lane >= 16u && lane - 16u < tail) c.edge_off = end_off + (lane - 16u);
     c.nvec = nvec < kVecPerRound ? nvec : kVecPerRound;
     nvec_left = nvec - c.nvec;
     return c;
@@ -204,6 +273,92 @@ struct FragmentRounds {
     return c;
   }
 };
+
+// Copies descriptors first, first + stride, ... < n of a descriptor list staged in LDS with the calling
+// wavefront; neighbours in the list decide which destination lines are shared.  The loads of the next round
+// are issued before the stores of the current one (kTwoRoundsInFlight); two register sets alternate so that no
+// register is copied while a load into it is in flight.  `bounce` and `dst` must be wave-uniform.
+template <bool kTwoRoundsInFlight>
+__device__ __forceinline__ void wave_copy_descriptors(const tcpxuLoadMeta* descs, uint32_t n, uint32_t first,
+                                                      uint32_t stride, const uint8_t* bounce, uint8_t* dst,
+                                                      uint32_t lane) {
+  // Everything that describes a fragment is wave-uniform; saying so keeps it in scalar registers and leaves
+  // the vector registers to the payload in flight.
+  auto uniform = [](uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(v)); };
+  auto uniform64 = [&](uint64_t v) {
+    return (static_cast<uint64_t>(uniform(static_cast<uint32_t>(v >> 32))) << 32) | uniform(static_cast<uint32_t>(v));
+  };
+  const uint64_t dst_addr = reinterpret_cast<uint64_t>(dst);
+  uint32_t j = uniform(first);
+  FragmentRounds fr;
+  // Next round of this wavefront's work, or false when there is none.  `prev` is the round before it.
+  auto produce = [&](CopyRound& out, const CopyRound& prev) -> bool {
+    if (fr.more()) {
+      out = fr.next_round(prev);
+      return true;
+    }
+    while (j < n) {
+      const uint32_t cur = j;
+      j += stride;
+      const tcpxuLoadMeta d = descs[cur];
+      const uint32_t len = uniform(d.len);
+      if (len == 0) continue;
+      const uint32_t so = uniform(d.src_off);
+      const uint64_t doff = uniform64(d.dst_off);
+      const uint8_t* fsrc = bounce + so;
+      uint8_t* fdst = dst + doff;
+      if (fragment_is_tiny(fdst, len)) {
+        copy_tiny_fragment(fsrc, fdst, len, lane);
+        continue;
+      }
+      bool share_prev = false, share_next = false;
+      const uint8_t* src_next = fsrc;
+      if (cur > 0) {
+        const tcpxuLoadMeta p = descs[cur - 1];
+        share_prev = shares_line(dst_addr + uniform64(p.dst_off), uniform(p.len), dst_addr + doff, len);
+      }
+      if (cur + 1 < n) {
+        const tcpxuLoadMeta q = descs[cur + 1];
+        share_next = shares_line(dst_addr + doff, len, dst_addr + uniform64(q.dst_off), uniform(q.len));
+        if (share_next) src_next = bounce + uniform(q.src_off);
+      }
+      out = fr.first_round(fsrc, fdst, len, share_prev, share_next, src_next, lane);
+      return true;
+    }
+    return false;
+  };
+  if constexpr (!kTwoRoundsInFlight) {
+    // One register set: more wavefronts fit on a compute unit, each with one round in flight.
+    CopyRound r;
+    CopyRegs x;
+    if (!produce(r, r)) return;
+    for (;;) {
+      round_load(r, x, lane);
+      round_store(r, x, lane);
+      CopyRound nxt;
+      if (!produce(nxt, r)) return;
+      r = nxt;
+    }
+  }
+  CopyRound ra, rb;
+  CopyRegs xa, xb;
+  if (!produce(ra, ra)) return;
+  round_load(ra, xa, lane);
+  for (;;) {
+    if (!produce(rb, ra)) {
+      round_store(ra, xa, lane);
+      break;
+    }
+    round_load(rb, xb, lane);
+    round_store(ra, xa, lane);
+    if (!produce(ra, rb)) {
+      round_store(rb, xb, lane);
+      break;
+    }
+    round_load(ra, xa, lane);
+    round_store(rb, xb, lane);
+  }
+}
 
 // The 8 XCDs of an MI355X receive workgroups round-robin by workgroup id and each has its own L2.  This maps a
 // workgroup id to a work-item index such that every XCD walks one contiguous eighth of the index space:
