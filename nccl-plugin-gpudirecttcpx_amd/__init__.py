@@ -214,6 +214,89 @@ def _bind(lib, prototypes):
     return lib
 
 
+class NetProperties(ctypes.Structure):
+    """ncclNetProperties_v7_t (include/nccl_net_v7.h)."""
+
+    _fields_ = [
+        ("name", ctypes.c_char_p),
+        ("pciPath", ctypes.c_char_p),
+        ("guid", ctypes.c_uint64),
+        ("ptrSupport", ctypes.c_int),
+        ("speed", ctypes.c_int),
+        ("port", ctypes.c_int),
+        ("latency", ctypes.c_float),
+        ("maxComms", ctypes.c_int),
+        ("maxRecvs", ctypes.c_int),
+        ("netDeviceType", ctypes.c_int),
+        ("netDeviceVersion", ctypes.c_int),
+    ]
+
+
+class NetDeviceHandle(ctypes.Structure):
+    """ncclNetDeviceHandle_v7_t."""
+
+    _fields_ = [
+        ("netDeviceType", ctypes.c_int),
+        ("netDeviceVersion", ctypes.c_int),
+        ("handle", ctypes.c_void_p),
+        ("size", ctypes.c_size_t),
+        ("needsProxyProgress", ctypes.c_int),
+    ]
+
+
+_V = ctypes.c_void_p
+_VP = ctypes.POINTER(ctypes.c_void_p)
+_IP = ctypes.POINTER(ctypes.c_int)
+NET_V7_MEMBERS = [
+    "name", "init", "devices", "getProperties", "listen", "connect", "accept", "regMr", "regMrDmaBuf", "deregMr",
+    "isend", "irecv", "iflush", "test", "closeSend", "closeRecv", "closeListen", "getDeviceMr", "irecvConsumed",
+]  # fmt: skip
+
+
+class NetV7(ctypes.Structure):
+    """ncclNet_v7_t as 19 pointer-sized members, in the reference's order (src/nccl_plugin.cc:22-42)."""
+
+    _fields_ = [(m, ctypes.c_void_p) for m in NET_V7_MEMBERS]
+
+
+_PLUGIN_PROTOTYPES = {
+    "tcpxInit": (ctypes.c_int, [_V]),
+    "tcpxFinalize": (ctypes.c_int, []),
+    "tcpxDevices": (ctypes.c_int, [_IP]),
+    "tcpxGetProperties": (ctypes.c_int, [ctypes.c_int, ctypes.POINTER(NetProperties)]),
+    "tcpxListen": (ctypes.c_int, [ctypes.c_int, _V, _VP]),
+    "tcpxConnect_v5": (ctypes.c_int, [ctypes.c_int, _V, _VP, _V]),
+    "tcpxAccept_v5": (ctypes.c_int, [_V, _VP, ctypes.POINTER(ctypes.POINTER(NetDeviceHandle))]),
+    "tcpxRegMr": (ctypes.c_int, [_V, _V, ctypes.c_int, ctypes.c_int, _VP]),
+    "tcpxDeregMr": (ctypes.c_int, [_V, _V]),
+    "tcpxIsend_v5": (ctypes.c_int, [_V, _V, ctypes.c_int, ctypes.c_int, _V, _VP]),
+    "tcpxIrecv_v5": (ctypes.c_int, [_V, ctypes.c_int, _VP, _IP, _IP, _VP, _VP]),
+    "tcpxIflush_v5": (ctypes.c_int, [_V, ctypes.c_int, _VP, _IP, _VP, _VP]),
+    "tcpxTest": (ctypes.c_int, [_V, _IP, _IP]),
+    "tcpxClose": (ctypes.c_int, [_V]),
+    "tcpxCloseListen": (ctypes.c_int, [_V]),
+    "tcpxGetDeviceMr": (ctypes.c_int, [_V, _V, _VP]),
+    "tcpxIrecvConsumed": (ctypes.c_int, [_V, ctypes.c_int, _V]),
+    "tcpxSynthArenaCreate": (ctypes.c_int, [ctypes.c_int, ctypes.c_size_t, _VP]),
+    "tcpxSynthCtrlSend": (
+        ctypes.c_int,
+        [_V, ctypes.c_uint16, ctypes.c_uint16, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32],
+    ),
+    "tcpxSynthDeliver": (ctypes.c_int, [_V, ctypes.c_uint32, _V, ctypes.c_uint32]),
+    "tcpxSynthSetRecvmsgLimit": (ctypes.c_int, [_V, ctypes.c_uint32]),
+    "tcpxSynthOutstandingPages": (ctypes.c_int, [_V, ctypes.POINTER(ctypes.c_uint64)]),
+    "tcpxDebugQueueState": (
+        ctypes.c_int,
+        [_V, ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint32 * 5)],
+    ),
+    "tcpxDebugSlot": (ctypes.c_int, [_V, ctypes.c_uint32, _VP, ctypes.POINTER(ctypes.c_uint64)]),
+    "tcpxSetDeviceOpsForTesting": (ctypes.c_int, [_V]),
+    "tcpxSetFailStopForTesting": (ctypes.c_int, [ctypes.c_int]),
+}
+
+NCCL_PTR_HOST, NCCL_PTR_CUDA = 1, 2
+CTRL_NORMAL, CTRL_INLINE = 0, 1
+
 _cache = {}
 
 
@@ -228,6 +311,15 @@ def synth_lib():
     if "synth" not in _cache:
         _cache["synth"] = _bind(_load("libtcpx_synth.so"), _SYNTH_PROTOTYPES)
     return _cache["synth"]
+
+
+def plugin_lib():
+    """``libnccl-net.so`` with prototypes attached, plus ``.table``: the exported ``ncclNetPlugin_v7``."""
+    if "plugin" not in _cache:
+        lib = _bind(_load("libnccl-net.so"), _PLUGIN_PROTOTYPES)
+        lib.table = NetV7.in_dll(lib, "ncclNetPlugin_v7")
+        _cache["plugin"] = lib
+    return _cache["plugin"]
 
 
 class HipError(RuntimeError):

@@ -1,0 +1,746 @@
+// ncclNet_v7 entry points of the receive-side unpack path and the progress engine behind them.
+//
+// Call pattern (NCCL's receive proxy, or a test driver in its place):
+//   irecv -> test* -> [consume the data] -> iflush? -> irecvConsumed
+// What differs from the reference by design: a request reports done=1 only after the GPU engine has written its
+// completion word, i.e. after the payload is in the receive buffer -- in the reference done=1 means "descriptor
+// count published" and NCCL's own kernel does the copy later.  Everything else (states, order checks, result
+// codes) follows src/net_tcpx.cc.
+#include <sched.h>
+
+#include <algorithm>
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+
+#include "plugin_internal.h"
+
+namespace tcpx {
+
+Global g;
+
+// ---- logging and flags --------------------------------------------------------------------------------------------
+void log_line(ncclDebugLogLevel level, unsigned long flags, const char* file, int line, const char* fmt, ...) {
+  char buf[1024];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  if (g.logger) {
+    g.logger(level, flags, file, line, "%s", buf);
+  } else if (level == NCCL_LOG_WARN) {
+    // Without NCCL's logger only warnings are printed (the reference's fallback prints everything,
+    // src/adapter/nccl/debug.cc:22-33; INFO is too chatty for a test run).
+    fprintf(stderr, "NET/GPUDirectTCPX-AMD WARN %s:%d %s\n", file, line, buf);
+  }
+}
+
+ncclResult_t fail_stop(const char* what) {
+  if (g.fail_stop) {
+    WARN("fail-stop: %s", what);
+    exit(1);
+  }
+  return ncclInternalError;
+}
+
+namespace {
+
+// NCCL_GPUDIRECTTCPX_<NAME>, kept only if it parses and lies in [lo, hi] (TCPX_GET_INT_FLAG,
+// src/net_tcpx.cc:440-452; TCPX_GET_ENV, src/adapter/param1.h:26-29).
+void int_flag(int* flag, const char* name, long lo, long hi) {
+  char env[128];
+  snprintf(env, sizeof env, "NCCL_GPUDIRECTTCPX_%s", name);
+  const char* v = getenv(env);
+  if (!v || !*v) return;
+  char* end = nullptr;
+  const long x = strtol(v, &end, 0);
+  if (end == v || x < lo || x > hi) {
+    WARN("%s=%s ignored: not an integer in [%ld, %ld]", env, v, lo, hi);
+    return;
+  }
+  *flag = static_cast<int>(x);
+}
+
+inline bool ctrl_done(const Request* r) { return r->next_flow >= 0; }  // CTRL_DONE, src/net_tcpx.cc:956
+// REQUEST_DONE, src/net_tcpx.cc:959-960
+inline bool request_done(const Request* r) {
+  return (r->size == 0 && ctrl_done(r)) || (r->size && r->size_pending == 0);
+}
+
+// ---- socket side: one task's progress (taskProgress, src/net_tcpx.cc:148-212) -------------------------------------
+ncclResult_t flow_progress(Comm* comm, int flow) {
+  FlowData* fd = &comm->flows[flow];
+  TaskRing* tasks = &fd->tasks;
+  if (tasks->has(kTaskActive)) {
+    Task* t = tasks->first(kTaskActive);
+    ncclResult_t res = ncclSuccess;
+    const ssize_t bytes = devmem_recv(&fd->sock, t->size, t->offset, t->pipe, static_cast<uint64_t>(t->request_offset), &res);
+    if (res != ncclSuccess) {
+      t->result = res;
+      return res;
+    }
+    if (bytes > 0) {
+      t->offset += static_cast<int>(bytes);
+      fd->bytes += static_cast<uint64_t>(bytes);
+    }
+    if (t->offset == t->size) tasks->advance(kTaskActive);  // ACTIVE -> COMPLETING
+  }
+  if (tasks->has(kTaskCompleting)) {
+    // The reference asks gpu_inline_test here, which always answers "done" (src/devcomm/nccl/inline.cu:55-60).
+    tasks->advance(kTaskCompleting);  // COMPLETING -> INACTIVE
+  }
+  return ncclSuccess;
+}
+
+void helper_main(Comm* comm) {  // persistentSocketThread, src/net_tcpx.cc:252-384 (receive part)
+  while (!comm->helper_stop.load(std::memory_order_acquire)) {
+    bool idle = true;
+    for (int f = 0; f < comm->num_flows; ++f) {
+      TaskRing* tasks = &comm->flows[f].tasks;
+      if (tasks->has(kTaskActive) || tasks->has(kTaskCompleting)) {
+        if (flow_progress(comm, f) != ncclSuccess) return;
+        idle = false;
+      }
+    }
+    if (idle) sched_yield();
+  }
+}
+
+// enqueueTask, src/net_tcpx.cc:1037-1097 (receive part)
+void enqueue_task(Comm* comm, Request* r) {
+  const int flow = r->next_flow;
+  r->next_flow = -1;  // RESET_CTRL
+  const int sz = r->next_size;
+  TaskRing* tasks = &comm->flows[flow].tasks;
+  Task* t = tasks->next_free();
+  t->op = r->op;
+  t->data = static_cast<char*>(r->data) + r->offset;
+  t->r = r;
+  t->result = ncclSuccess;
+  t->offset = 0;
+  t->request_offset = r->offset;
+  t->size = sz;
+  t->flow = flow;
+  t->pipe->cnt_cache = 0;
+  t->pipe->bytes_cnt = 0;
+  if (comm->passive) {
+    UnpackSlot* u = &r->slot;
+    u->flows[flow] = flow;
+    t->pipe->pgtoks = &u->pgtoks[static_cast<size_t>(flow) * kSlotPages];
+    t->pipe->pgtok_cnt = &u->pgtok_cnts[flow];
+    // Unlike the reference, the count is not zeroed here: a request may put several chunks on the same flow, and
+    // every chunk's pages must be given back when the request is consumed.  It is zeroed when the slot is taken.
+  }
+  tasks->enqueue();  // FREE -> ACTIVE
+  r->offset += sz;
+  if (r->size == r->offset) comm->rq.advance(kReqActive);  // REQUEST_INACTIVE -> finish_active
+}
+
+// tcpxCommProgress, src/net_tcpx.cc:1099-1308 (receive branch)
+ncclResult_t comm_progress(Comm* comm) {
+  if (comm->rq.empty()) return ncclSuccess;
+
+  if (!comm->use_helper) {
+    for (int f = 0; f < comm->num_flows; ++f) TCPXCHECK(flow_progress(comm, f));
+  }
+
+  // Reap finished tasks: their descriptors move into the request's slot (src/net_tcpx.cc:1119-1151).
+  bool any_flow_has_room = false;
+  for (int i = 0; i < comm->num_flows; ++i) {
+    int idx = comm->end_flow_idx - i;
+    if (idx < 0) idx += comm->num_flows;
+    TaskRing* tasks = &comm->flows[idx].tasks;
+    while (tasks->has(kTaskInactive)) {
+      Task* t = tasks->first(kTaskInactive);
+      if (t->result != ncclSuccess) return t->result;
+      t->r->size_pending -= t->size;
+      if (t->op == kOpRecv && t->size > 0) {
+        UnpackSlot* u = &t->r->slot;
+        if (u->cnt_cache + t->pipe->cnt_cache > static_cast<uint64_t>(kSlotPages)) {  // src/net_tcpx.cc:1350-1353
+          WARN("request too many pages %lu, failstop", static_cast<unsigned long>(u->cnt_cache + t->pipe->cnt_cache));
+          return fail_stop("request needs more descriptors than a slot holds");
+        }
+        memcpy(u->mem + u->cnt_cache, t->pipe->scatter_list.data(), sizeof(union loadMeta) * t->pipe->cnt_cache);
+        u->cnt_cache += t->pipe->cnt_cache;
+        t->pipe->cnt_cache = 0;
+      }
+      tasks->advance(kTaskInactive);  // INACTIVE -> FREE
+    }
+    if (tasks->has_free()) any_flow_has_room = true;
+  }
+
+  if (comm->rq.has(kReqPosted)) comm->rq.advance(kReqPosted);  // POSTED -> ACTIVE (src/net_tcpx.cc:1158-1180)
+
+  if (!comm->rq.has(kReqActive) || !any_flow_has_room) return ncclSuccess;
+  Request* ar = comm->rq.first(kReqActive);
+  if (ar->op != kOpRecv) return ncclSuccess;
+
+  do {  // src/net_tcpx.cc:1231-1304
+    if (!ctrl_done(ar)) {
+      CtrlMessage ctrl;
+      {
+        std::lock_guard<std::mutex> lock(comm->ctrl_mu);
+        if (comm->ctrl_rx.empty()) break;
+        ctrl = comm->ctrl_rx.front();
+        comm->ctrl_rx.pop_front();
+      }
+      if (ctrl.type != TCPX_CTRL_INLINE && ctrl.index >= comm->num_flows) {
+        WARN("control message names flow %u, comm has %d", ctrl.index, comm->num_flows);
+        return ncclInternalError;
+      }
+      ar->next_flow = ctrl.index;  // tcpxCtrlRecv, src/net_tcpx.cc:995-1014
+      ar->next_size = static_cast<int>(ctrl.size);
+      if (ar->size_pending < 0) ar->size_pending = ar->size = static_cast<int>(ctrl.total);
+
+      if (ctrl.type == TCPX_CTRL_INLINE) {  // src/net_tcpx.cc:1248-1276: an empty message still takes a slot
+        unpack_queue_next_free(comm->queue, &ar->slot);
+        if (!ar->slot.active) {
+          WARN("no more unpack queue slot, head %lu tail %lu", static_cast<unsigned long>(comm->queue->head),
+               static_cast<unsigned long>(comm->queue->tail));
+          // The control message is consumed and cannot be re-read: put it back so that a later poll retries.
+          std::lock_guard<std::mutex> lock(comm->ctrl_mu);
+          comm->ctrl_rx.push_front(ctrl);
+          ar->next_flow = -1;
+          break;
+        }
+        comm->queue->meta->nccl.cnt[ar->slot.idx] = 0;
+        comm->queue->record.flow_cnts[ar->slot.idx] = 0;
+        if (ar->size) {
+          WARN("payload through the control socket is not supported for device memory");
+          return ncclInternalError;
+        }
+        comm->rq.advance(kReqActive);  // -> TRANSMITTING
+        break;
+      }
+    }
+
+    if (ar->slot.cnt == nullptr) {  // first chunk of the request: take a slot (src/net_tcpx.cc:1279-1296)
+      unpack_queue_next_free(comm->queue, &ar->slot);
+      if (!ar->slot.active) {
+        WARN("no more unpack queue slot, head %lu tail %lu", static_cast<unsigned long>(comm->queue->head),
+             static_cast<unsigned long>(comm->queue->tail));
+        break;  // the pending control message stays in the request; retried at the next poll
+      }
+      *ar->slot.cnt = 0;
+      ar->slot.cnt_cache = 0;
+      *ar->slot.flow_cnt = static_cast<size_t>(comm->num_flows);
+      memset(ar->slot.pgtok_cnts, 0, kMaxFlows * sizeof(size_t));
+    }
+    TaskRing* tasks = &comm->flows[ar->next_flow].tasks;
+    if (!tasks->has_free()) break;  // "No free space for recv task": retried at the next poll
+    comm->end_flow_idx = ar->next_flow;
+    enqueue_task(comm, ar);
+  } while (ar->offset < ar->size);
+  return ncclSuccess;
+}
+
+// recyclePages, src/sock/tcpx.h:310-326
+ncclResult_t recycle_pages(Comm* comm, uint64_t q_idx) {
+  UnpackQueue* q = comm->queue;
+  q_idx %= kQueueDepth;
+  const size_t n_flows = q->record.flow_cnts[q_idx];
+  for (size_t i = 0; i < n_flows; ++i) {
+    const size_t n = q->record.pgtok_cnts[q_idx][i];
+    if (n > 0) {
+      const int flow = q->record.flows[q_idx][i];
+      if (comm->flows[flow].sock.dontneed(q->record.pgtoks[q_idx][i], n) != 0) {
+        WARN("page recycle failed on flow %d", flow);
+        return ncclInternalError;
+      }
+    }
+  }
+  return ncclSuccess;
+}
+
+ncclResult_t ensure_engine(DeviceState* ds) {
+  std::lock_guard<std::mutex> lock(ds->mu);
+  if (!ds->engine) {
+    tcpxuEngineConfig cfg{};
+    TCPXCHECK(device_result(g.ops->engine_create(ds->dev, &cfg, &ds->engine), "engine_create"));
+  }
+  if (!ds->engine_started) {
+    TCPXCHECK(device_result(g.ops->engine_start(ds->engine), "engine_start"));
+    ds->engine_started = true;
+  }
+  return ncclSuccess;
+}
+
+}  // namespace
+}  // namespace tcpx
+
+using namespace tcpx;
+
+extern "C" {
+
+ncclResult_t tcpxSetDeviceOpsForTesting(const tcpxDeviceOps* ops) {
+  std::lock_guard<std::mutex> lock(g.mu);
+  if (g.initialized) return ncclInvalidUsage;
+  g.ops = ops;
+  g.ops_injected = ops != nullptr;
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxSetFailStopForTesting(int enabled) {
+  g.fail_stop = enabled != 0;
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxInit(ncclDebugLogger_t logFunction) {
+  std::lock_guard<std::mutex> lock(g.mu);
+  g.logger = logFunction;
+  if (g.initialized) return ncclSuccess;
+  int_flag(&g.flows_per_comm, "AMD_FLOWS", 1, kMaxFlows);
+  int_flag(&g.use_helper_thread, "AMD_HELPER_THREAD", 0, 1);
+  if (!g.ops_injected) {
+    g.ops = default_device_ops();
+    if (!g.ops) {
+      WARN("the HIP layer is not available: this plugin has no other way to move data");
+      return ncclSystemError;
+    }
+  }
+  int n = 0;
+  TCPXCHECK(device_result(g.ops->device_count(&n), "device_count"));
+  if (n <= 0) {
+    WARN("no GPU visible");
+    return ncclSystemError;
+  }
+  g.n_devices = std::min(n, kMaxDevices);
+  for (int d = 0; d < g.n_devices; ++d) {
+    g.devices[d].dev = d;
+    snprintf(g.dev_names[d], sizeof g.dev_names[d], "tcpx-amd-synth%d", d);
+    snprintf(g.pci_paths[d], sizeof g.pci_paths[d], "/sys/class/net/tcpx-amd-synth%d/device", d);
+  }
+  g.initialized = true;
+  INFO(NCCL_INIT | NCCL_NET, "NET/GPUDirectTCPX-AMD initialised: %d device(s), %d flows per comm", g.n_devices,
+       g.flows_per_comm);
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxFinalize(void) {
+  std::lock_guard<std::mutex> lock(g.mu);
+  if (!g.initialized) return ncclSuccess;
+  ncclResult_t rc = ncclSuccess;
+  for (int d = 0; d < g.n_devices; ++d) {
+    DeviceState* ds = &g.devices[d];
+    std::lock_guard<std::mutex> dl(ds->mu);
+    if (ds->comms != 0) {
+      WARN("device %d still has %d open comm(s)", d, ds->comms);
+      rc = ncclInvalidUsage;
+      continue;
+    }
+    // Stop the persistent kernel first: nothing may be freed underneath it.
+    if (ds->engine) {
+      if (ds->engine_started && g.ops->engine_stop(ds->engine, nullptr) != TCPXU_SUCCESS) rc = ncclInternalError;
+      ds->engine_started = false;
+      if (g.ops->engine_destroy(ds->engine) != TCPXU_SUCCESS) rc = ncclInternalError;
+      ds->engine = nullptr;
+    }
+    for (QueueBlock& b : ds->free_blocks) {
+      g.ops->mapped_free(d, b.meta);
+      g.ops->device_free(d, b.dev_handle);
+    }
+    ds->free_blocks.clear();
+    if (ds->arena) g.ops->arena_destroy(d, ds->arena);
+    ds->arena = nullptr;
+    ds->arena_bytes = 0;
+    ds->page_refs.reset();
+    ds->n_pages = 0;
+    ds->pages_outstanding = 0;
+  }
+  if (rc == ncclSuccess) g.initialized = false;
+  return rc;
+}
+
+ncclResult_t tcpxDevices(int* ndev) {
+  std::lock_guard<std::mutex> lock(g.mu);
+  *ndev = g.n_devices;
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxGetProperties(int dev, ncclNetProperties_v7_t* props) {
+  if (dev < 0 || dev >= g.n_devices || !props) return ncclInternalError;
+  props->name = g.dev_names[dev];
+  props->pciPath = g.pci_paths[dev];
+  props->guid = static_cast<uint64_t>(dev);
+  props->ptrSupport = NCCL_PTR_HOST | NCCL_PTR_CUDA;
+  props->speed = 10000;  // the reference's fallback when sysfs has no speed (src/net_tcpx.cc:717-721)
+  props->port = 0;
+  props->maxComms = 65536;
+  props->latency = 0;
+  props->maxRecvs = 1;
+  props->netDeviceType = NCCL_NET_DEVICE_UNPACK;
+  props->netDeviceVersion = NCCL_NET_DEVICE_UNPACK_VERSION;
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxSynthArenaCreate(int dev, size_t bytes, void** base) {
+  if (!g.initialized || dev < 0 || dev >= g.n_devices || !base) return ncclInvalidArgument;
+  DeviceState* ds = &g.devices[dev];
+  std::lock_guard<std::mutex> lock(ds->mu);
+  if (ds->arena) {
+    WARN("device %d already has an arena", dev);
+    return ncclInvalidUsage;
+  }
+  TCPXCHECK(device_result(g.ops->arena_create(dev, bytes, &ds->arena), "arena_create"));
+  ds->arena_bytes = bytes;
+  ds->n_pages = bytes / SLICE_PAGE_SIZE;
+  ds->page_refs.reset(new std::atomic<int32_t>[ds->n_pages]);
+  for (size_t i = 0; i < ds->n_pages; ++i) ds->page_refs[i] = 0;
+  ds->pages_outstanding = 0;
+  *base = ds->arena;
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxListen(int dev, void* handle, void** listenComm) {
+  if (!g.initialized || dev < 0 || dev >= g.n_devices || !handle || !listenComm) return ncclInternalError;
+  static std::atomic<uint64_t> next_id{1};
+  ListenComm* l = static_cast<ListenComm*>(calloc(1, sizeof *l));
+  if (!l) return ncclSystemError;
+  l->dev = dev;
+  l->id = next_id.fetch_add(1);
+  memset(handle, 0, NCCL_NET_HANDLE_MAXSIZE);
+  memcpy(handle, l, sizeof *l);  // the connect handle: which listener, on which device
+  *listenComm = l;
+  return ncclSuccess;
+}
+
+static ncclResult_t new_comm(int dev, bool passive, Comm** out) {
+  Comm* c = new (std::nothrow) Comm;
+  if (!c) return ncclSystemError;
+  c->passive = passive;
+  c->dev = dev;
+  c->device = &g.devices[dev];
+  c->num_flows = g.flows_per_comm;
+  c->use_helper = g.use_helper_thread != 0;
+  for (int f = 0; f < kMaxFlows; ++f) c->flows[f].sock.device = c->device;
+  *out = c;
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxConnect_v5(int dev, void* handle, void** sendComm, ncclNetDeviceHandle_v7_t** sendDevHandle) {
+  if (!g.initialized || dev < 0 || dev >= g.n_devices || !handle || !sendComm) return ncclInternalError;
+  // The sending side is outside this build (no NIC, no sockets): the comm exists so that the call sequence of a
+  // real job can be replayed, but tcpxIsend_v5 on it reports an error.
+  Comm* c = nullptr;
+  TCPXCHECK(new_comm(dev, false, &c));
+  *sendComm = c;
+  (void)sendDevHandle;
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxAccept_v5(void* listenComm, void** recvComm, ncclNetDeviceHandle_v7_t** recvDevHandle) {
+  if (!g.initialized || !listenComm || !recvComm) return ncclInternalError;
+  ListenComm* l = static_cast<ListenComm*>(listenComm);
+  DeviceState* ds = &g.devices[l->dev];
+  if (!ds->arena) {
+    WARN("device %d has no bounce arena: call tcpxSynthArenaCreate first", l->dev);
+    return ncclInternalError;
+  }
+  Comm* c = nullptr;
+  TCPXCHECK(new_comm(l->dev, true, &c));
+  ncclResult_t rc = ensure_engine(ds);
+  if (rc == ncclSuccess) rc = unpack_queue_new(l->dev, true, &c->queue);  // tcpxGetDeviceHandle, src/net_tcpx.cc:1452-1471
+  if (rc != ncclSuccess) {
+    delete c;
+    return rc;
+  }
+  {
+    std::lock_guard<std::mutex> lock(ds->mu);
+    ds->comms++;
+  }
+  if (c->use_helper) c->helper = std::thread(helper_main, c);
+  if (recvDevHandle && *recvDevHandle) {
+    ncclNetDeviceHandle_v7_t* h = *recvDevHandle;
+    h->netDeviceType = NCCL_NET_DEVICE_UNPACK;
+    h->netDeviceVersion = NCCL_NET_DEVICE_UNPACK_VERSION;
+    h->handle = c->queue->dev_handle;
+    h->size = sizeof(struct unpackNetDeviceHandle);
+    h->needsProxyProgress = 1;
+  }
+  *recvComm = c;
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxRegMr(void* ocomm, void* data, int size, int type, void** mhandle) {
+  (void)size;
+  if (ocomm == nullptr) {
+    WARN("regMr called with NULL communicator.");
+    return ncclInternalError;
+  }
+  if (type != NCCL_PTR_HOST && type != NCCL_PTR_CUDA) {
+    WARN("unknown mem type %d", type);
+    return ncclInternalError;
+  }
+  MemHandle* m = static_cast<MemHandle*>(calloc(1, sizeof *m));
+  if (!m) return ncclSystemError;
+  m->ptr = data;
+  m->mem_type = type;
+  *mhandle = m;
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxDeregMr(void* ocomm, void* mhandle) {
+  (void)ocomm;
+  free(mhandle);  // NULL is fine (src/net_tcpx.cc:828)
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxGetDeviceMr(void* comm, void* mhandle, void** dptr_mhandle) {
+  (void)comm;
+  (void)mhandle;
+  (void)dptr_mhandle;
+  return ncclSuccess;
+}
+
+// tcpxGetRequest, src/net_tcpx.cc:862-896
+static ncclResult_t get_request(Comm* comm, int op, void* data, int size, MemHandle* mh, Request** req) {
+  if (mh == nullptr) {
+    WARN("mhandle is null");
+    return ncclInternalError;
+  }
+  if (!comm->rq.has_free()) {
+    WARN("unable to allocate requests");
+    return ncclInternalError;
+  }
+  Request* r = comm->rq.next_free();
+  r->op = op;
+  r->mem_type = mh->mem_type;
+  r->next_flow = -1;
+  r->next_size = 0;
+  r->data = data;
+  r->offset = 0;
+  r->size = size;
+  r->size_pending = op == kOpSend ? size : -1;
+  r->comm = comm;
+  r->slot = UnpackSlot{};  // cnt == nullptr: no slot yet
+  r->published = false;
+  r->done_value = 0;
+  *req = r;
+  comm->rq.enqueue();  // FREE -> POSTED
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxIsend_v5(void* sendComm, void* data, int size, int tag, void* mhandle, void** request) {
+  (void)sendComm, (void)data, (void)size, (void)tag, (void)mhandle;
+  if (request) *request = nullptr;
+  WARN("isend: the sending side is not part of this build (no NIC, no sockets)");
+  return ncclInternalError;
+}
+
+ncclResult_t tcpxIrecv_v5(void* recvComm, int n, void** data, int* sizes, int* tags, void** mhandles, void** request) {
+  (void)tags;
+  Comm* comm = static_cast<Comm*>(recvComm);
+  if (n != 1) return ncclInternalError;
+  if (!comm || !comm->passive) return ncclInternalError;
+  Request* r = nullptr;
+  TCPXCHECK(get_request(comm, kOpRecv, data[0], sizes[0], static_cast<MemHandle*>(mhandles[0]), &r));
+  *request = r;
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxIflush_v5(void* recvComm, int n, void** data, int* sizes, void** mhandles, void** request) {
+  (void)recvComm, (void)data, (void)mhandles;
+  // "Iflush unused for now" (src/net_tcpx.cc:946-954): the slot the caller passes still holds the receive
+  // request, whose size is echoed; no flush request is created and no work is done.
+  if (n != 1) return ncclInternalError;
+  if (request && request[0] && sizes) sizes[0] = static_cast<Request*>(request[0])->size;
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxTest(void* request, int* done, int* size) {
+  (void)size;  // never written, as in the reference
+  *done = 0;
+  Request* r = static_cast<Request*>(request);
+  if (r == nullptr) {
+    WARN("test called with NULL request");
+    return ncclInternalError;
+  }
+  Comm* comm = r->comm;
+  TCPXCHECK(comm_progress(comm));
+  if (!comm->rq.has(kReqTransmitting)) return ncclSuccess;
+  Request* ni = comm->rq.first(kReqTransmitting);
+  if (r != ni) {  // requests complete in the order they were posted (src/net_tcpx.cc:1322-1328)
+    WARN("test called with invalid request, r %p, ni %p", static_cast<void*>(r), static_cast<void*>(ni));
+    return ncclInternalError;
+  }
+  if (!request_done(r)) return ncclSuccess;
+  if (r->op == kOpRecv) {
+    if (r->size) {
+      UnpackQueue* q = comm->queue;
+      if (!r->published) {
+        if (r->slot.cnt_cache > static_cast<uint64_t>(kSlotPages)) {  // src/net_tcpx.cc:1350-1353
+          WARN("request too many pages %lu, failstop", static_cast<unsigned long>(r->slot.cnt_cache));
+          return fail_stop("request needs more descriptors than a slot holds");
+        }
+        // Publish: descriptor count, then a release, then the submission that makes the GPU look
+        // (src/net_tcpx.cc:1354-1357 is the count + fences; the doorbell is this build's).
+        *r->slot.cnt = r->slot.cnt_cache;
+        std::atomic_thread_fence(std::memory_order_release);
+        q->meta->done[r->slot.idx].value = 0;
+        r->done_value = ++comm->done_seq;
+        const int rc = g.ops->engine_submit(comm->device->engine, comm->device->arena, r->data,
+                                            q->meta_dev->nccl.mem[r->slot.idx], static_cast<uint32_t>(r->slot.cnt_cache),
+                                            &q->meta_dev->done[r->slot.idx].value, r->done_value);
+        if (rc == TCPXU_IN_PROGRESS) {  // submission ring full: try again at the next poll
+          --comm->done_seq;
+          return ncclSuccess;
+        }
+        TCPXCHECK(device_result(rc, "engine_submit"));
+        r->published = true;
+      }
+      const uint64_t seen =
+          reinterpret_cast<std::atomic<uint64_t>*>(&q->meta->done[r->slot.idx].value)->load(std::memory_order_acquire);
+      if (seen != r->done_value) return ncclSuccess;  // the GPU is still copying
+    } else {
+      *r->slot.cnt = 0;  // src/net_tcpx.cc:1361
+    }
+  }
+  comm->rq.advance(kReqTransmitting);  // -> INACTIVE
+  *done = 1;
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxIrecvConsumed(void* ocomm, int n, void* request) {
+  if (request == nullptr) {
+    WARN("irecvConsumed with null request");
+    return ncclInternalError;
+  }
+  if (n != 1) return ncclInternalError;
+  Comm* comm = static_cast<Comm*>(ocomm);
+  UnpackQueue* q = comm->queue;
+  Request* r = static_cast<Request*>(request);
+  if (r->op == kOpSend) {
+    WARN("irecvConsumed called for send request %p", request);
+    return ncclSuccess;
+  }
+  if (!r->size) {  // skip empty (src/net_tcpx.cc:1500-1504)
+    comm->rq.advance(kReqInactive);
+    q->head += 1;
+    return ncclSuccess;
+  }
+  if (!r->slot.active) {
+    WARN("irecvConsumed called with r %p ->size %d inactive unpack slot", request, r->size);
+    return ncclInternalError;
+  }
+  if (!comm->rq.has(kReqInactive)) {
+    WARN("irecvConsumed called with %p when no inactive request", request);
+    return ncclInternalError;
+  }
+  Request* ir = comm->rq.first(kReqInactive);
+  if (ir != r) {
+    WARN("irecvConsumed called with invalid request %p vs expected %p", request, static_cast<void*>(ir));
+    return ncclInternalError;
+  }
+  const uint64_t q_idx = ir->slot.idx;
+  if (q->head == q->tail) {
+    WARN("irecvConsumed shouldn't be called when head == tail == %lu", static_cast<unsigned long>(q->head));
+    return ncclInternalError;
+  }
+  if (q->head % kQueueDepth != q_idx) {
+    WARN("irecvConsumed unexpected q_idx %lu vs head %lu", static_cast<unsigned long>(q_idx),
+         static_cast<unsigned long>(q->head));
+    return ncclInternalError;
+  }
+  TCPXCHECK(recycle_pages(comm, q_idx));
+  comm->rq.advance(kReqInactive);  // INACTIVE -> FREE
+  q->head += 1;
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxClose(void* oComm) {
+  Comm* comm = static_cast<Comm*>(oComm);
+  if (!comm) return ncclSuccess;
+  if (comm->helper.joinable()) {
+    comm->helper_stop.store(true, std::memory_order_release);
+    comm->helper.join();
+  }
+  if (comm->queue) {
+    if (comm->queue->head != comm->queue->tail)  // src/net_tcpx.cc:1385-1390
+      WARN("head %lu tail %lu some pages not yet freed?", static_cast<unsigned long>(comm->queue->head),
+           static_cast<unsigned long>(comm->queue->tail));
+    unpack_queue_free(comm->queue);
+    std::lock_guard<std::mutex> lock(comm->device->mu);
+    comm->device->comms--;
+  }
+  delete comm;
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxCloseListen(void* oComm) {
+  free(oComm);
+  return ncclSuccess;
+}
+
+// ---- synthetic socket and inspection ------------------------------------------------------------------------------
+
+ncclResult_t tcpxSynthCtrlSend(void* recvComm, uint16_t type, uint16_t flow, uint32_t size, uint32_t offset,
+                               uint32_t total) {
+  Comm* comm = static_cast<Comm*>(recvComm);
+  if (!comm || !comm->passive || type > TCPX_CTRL_INLINE) return ncclInvalidArgument;
+  std::lock_guard<std::mutex> lock(comm->ctrl_mu);
+  comm->ctrl_rx.push_back(CtrlMessage{type, flow, size, offset, total});
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxSynthDeliver(void* recvComm, uint32_t flow, const tcpxSynthFrag* frags, uint32_t n_frags) {
+  Comm* comm = static_cast<Comm*>(recvComm);
+  if (!comm || !comm->passive || flow >= static_cast<uint32_t>(comm->num_flows) || (!frags && n_frags)) return ncclInvalidArgument;
+  const size_t arena = comm->device->arena_bytes;
+  for (uint32_t i = 0; i < n_frags; ++i) {
+    const tcpxSynthFrag& f = frags[i];
+    // The devmem contract: a fragment lies inside the arena and inside one 4 KiB page.
+    if (static_cast<size_t>(f.frag_offset) + f.frag_size > arena ||
+        (f.frag_offset % SLICE_PAGE_SIZE) + f.frag_size > SLICE_PAGE_SIZE) {
+      WARN("fragment %u (offset %u, size %u) breaks the devmem contract", i, f.frag_offset, f.frag_size);
+      return ncclInvalidArgument;
+    }
+  }
+  DevmemSocket* s = &comm->flows[flow].sock;
+  std::lock_guard<std::mutex> lock(s->mu);
+  s->rx.insert(s->rx.end(), frags, frags + n_frags);
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxSynthSetRecvmsgLimit(void* recvComm, uint32_t max_frags_per_recvmsg) {
+  Comm* comm = static_cast<Comm*>(recvComm);
+  if (!comm) return ncclInvalidArgument;
+  for (int f = 0; f < kMaxFlows; ++f) {
+    std::lock_guard<std::mutex> lock(comm->flows[f].sock.mu);
+    comm->flows[f].sock.max_frags_per_recvmsg = max_frags_per_recvmsg;
+  }
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxSynthOutstandingPages(void* recvComm, uint64_t* pages) {
+  Comm* comm = static_cast<Comm*>(recvComm);
+  if (!comm || !pages) return ncclInvalidArgument;
+  *pages = comm->device->pages_outstanding.load();
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxDebugQueueState(void* recvComm, uint64_t* head, uint64_t* tail, uint32_t request_idx[5]) {
+  Comm* comm = static_cast<Comm*>(recvComm);
+  if (!comm || !comm->queue) return ncclInvalidArgument;
+  if (head) *head = comm->queue->head;
+  if (tail) *tail = comm->queue->tail;
+  if (request_idx) {
+    // In the order of the reference's idx[]: [0] dequeue cursor, [1] left TRANSMITTING, [2] left ACTIVE,
+    // [3] left POSTED, [4] enqueue cursor.
+    request_idx[0] = comm->rq.left[kReqInactive];
+    request_idx[1] = comm->rq.left[kReqTransmitting];
+    request_idx[2] = comm->rq.left[kReqActive];
+    request_idx[3] = comm->rq.left[kReqPosted];
+    request_idx[4] = comm->rq.entered;
+  }
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxDebugSlot(void* recvComm, uint32_t slot_idx, const union loadMeta** descs, uint64_t* cnt) {
+  Comm* comm = static_cast<Comm*>(recvComm);
+  if (!comm || !comm->queue || slot_idx >= static_cast<uint32_t>(kQueueDepth)) return ncclInvalidArgument;
+  if (descs) *descs = comm->queue->meta->nccl.mem[slot_idx];
+  if (cnt) *cnt = comm->queue->meta->nccl.cnt[slot_idx];
+  return ncclSuccess;
+}
+
+}  // extern "C"

@@ -1,0 +1,313 @@
+// Internal types of the plugin library: the receive-side state that sits between the ncclNet_v7 calls and the
+// GPU engine.  Everything here is host code; the GPU is reached only through the tcpxDeviceOps table.
+//
+// Roles (reference file:line in parentheses)
+//   StageRing      fixed-capacity ring whose items move through an ordered list of stages
+//                  (tcpxItemQueue, src/work_queue.h:78-130)
+//   Request        one posted receive (tcpxRequest, src/work_queue.h:63-76) in a 16-deep RequestRing
+//                  (tcpxRequestQueue, src/work_queue.h:174-212; states src/work_queue_states.h:30-39)
+//   Task           one chunk of a request travelling on one data flow (tcpxTask, src/work_queue.h:38-59) in a
+//                  6-deep TaskRing shared with the socket thread (tcpxTaskQueue, src/work_queue.h:132-172)
+//   DataPipe       per-task staging of descriptors and page tokens (tcpxDataPipe, src/sock/datapipe.h:25-46)
+//   DevmemSocket   synthetic stand-in for one devmem-TCP data socket
+//   UnpackQueue    the slot ring in mapped memory (tcpxNetDeviceQueue, src/devcomm/unpack_defs1.h:39-74)
+//   Comm           per-connection state (tcpxComm, src/common.h:159-216)
+#ifndef TCPX_AMD_PLUGIN_INTERNAL_H_
+#define TCPX_AMD_PLUGIN_INTERNAL_H_
+
+#include <sys/socket.h>
+#include <sys/uio.h>
+
+#include <atomic>
+#include <cstdint>
+#include <cstdlib>
+#include <cstring>
+#include <deque>
+#include <memory>
+#include <mutex>
+#include <thread>
+#include <vector>
+
+#include "tcpx_plugin.h"
+
+namespace tcpx {
+
+constexpr int kMaxRequests = 16;  // MAX_REQUESTS, src/work_queue.h:20
+constexpr int kMaxTasks = 6;      // MAX_TASKS, src/work_queue.h:21
+constexpr int kMaxFlows = 8;      // MAX_SOCKETS, src/macro.h:36
+constexpr int kQueueDepth = NCCL_NET_DEVICE_UNPACK_MAX_QUEUE_DEPTH;
+constexpr int kSlotPages = NET_UNPACK_MAX_SLICE_PAGES;
+constexpr int kMaxDevices = 64;
+
+constexpr int kOpSend = 0;  // TCPX_SOCKET_SEND
+constexpr int kOpRecv = 1;  // TCPX_SOCKET_RECV
+
+// Linux devmem-TCP control-message types the reference parses (src/sock/tcpx.h:30-42).
+constexpr int kScmDevmemHeader = 98;
+constexpr int kScmDevmemOffset = 99;
+
+// ---- logging ------------------------------------------------------------------------------------------------------
+void log_line(ncclDebugLogLevel level, unsigned long flags, const char* file, int line, const char* fmt, ...)
+    __attribute__((format(printf, 5, 6)));
+#define WARN(...) ::tcpx::log_line(NCCL_LOG_WARN, NCCL_ALL, __FILE__, __LINE__, __VA_ARGS__)
+#define INFO(FLAGS, ...) ::tcpx::log_line(NCCL_LOG_INFO, (FLAGS), __FILE__, __LINE__, __VA_ARGS__)
+
+// Propagate errors up (TCPXCHECK, src/misc/checks1.h:53-61).
+#define TCPXCHECK(call)                                                    \
+  do {                                                                     \
+    ncclResult_t res_ = (call);                                            \
+    if (res_ != ncclSuccess) {                                             \
+      INFO(NCCL_ALL, "TCPXCHECK %s:%d -> %d", __FILE__, __LINE__, res_);   \
+      return res_;                                                         \
+    }                                                                      \
+  } while (0)
+
+// ---- StageRing ----------------------------------------------------------------------------------------------------
+// Items enter at stage 0 and leave each stage in FIFO order.  `entered` counts items ever enqueued, `left[k]` items
+// that have left stage k; an item leaving the last stage frees its slot.  Counters only grow, so
+//   entered >= left[0] >= left[1] >= ... >= left[Stages-1]   and   entered - left[Stages-1] <= Capacity.
+// With Counter = std::atomic<uint32_t> one thread may own `entered` and some stages while another owns the rest
+// (single producer, single consumer per counter).
+template <typename Item, int Capacity, int Stages, typename Counter>
+struct StageRing {
+  alignas(64) Counter entered;
+  alignas(64) Counter left[Stages];
+  alignas(64) Item items[Capacity];
+
+  StageRing() {
+    entered = 0;
+    for (int k = 0; k < Stages; ++k) left[k] = 0;
+  }
+  uint32_t in_flight() const { return static_cast<uint32_t>(entered) - static_cast<uint32_t>(left[Stages - 1]); }
+  bool empty() const { return in_flight() == 0; }
+  uint32_t num_free() const { return Capacity - in_flight(); }
+  bool has_free() const { return num_free() > 0; }
+  Item* next_free() { return &items[static_cast<uint32_t>(entered) % Capacity]; }
+  void enqueue() { entered = static_cast<uint32_t>(entered) + 1; }
+
+  uint32_t stage_begin(int k) const { return static_cast<uint32_t>(left[k]); }
+  uint32_t stage_end(int k) const { return k == 0 ? static_cast<uint32_t>(entered) : static_cast<uint32_t>(left[k - 1]); }
+  bool has(int k) const { return stage_end(k) != stage_begin(k); }
+  Item* first(int k) { return &items[stage_begin(k) % Capacity]; }
+  void advance(int k) { left[k] = static_cast<uint32_t>(left[k]) + 1; }
+};
+
+// ---- unpack queue -------------------------------------------------------------------------------------------------
+struct PageToken {  // struct devmemtoken / pgtok_t, src/devcomm/unpack_defs1.h:39-44
+  uint32_t token_start;
+  uint32_t token_count;
+};
+
+// Mapped host memory of one comm.  The prefix is NCCL's netUnpackMeta, bit for bit; the completion words that the
+// GPU engine writes follow it.
+struct QueueMeta {
+  struct netUnpackMeta nccl;
+  struct alignas(64) DoneWord {
+    uint64_t value;
+  } done[kQueueDepth];
+};
+
+struct QueueRecord {  // struct tcpxRecord, src/devcomm/unpack_defs1.h:46-51
+  size_t flow_cnts[kQueueDepth];
+  size_t pgtok_cnts[kQueueDepth][kMaxFlows];
+  int flows[kQueueDepth][kMaxFlows];
+  PageToken pgtoks[kQueueDepth][kMaxFlows][kSlotPages];
+};
+
+struct UnpackQueue {  // struct tcpxNetDeviceQueue, src/devcomm/unpack_defs1.h:53-59
+  QueueMeta* meta = nullptr;      // host address
+  QueueMeta* meta_dev = nullptr;  // device alias
+  struct unpackNetDeviceHandle* dev_handle = nullptr;  // device memory
+  uint64_t head = 0, tail = 0;
+  int dev = 0;
+  QueueRecord record;
+};
+
+struct UnpackSlot {  // struct unpackSlot, src/devcomm/unpack_defs1.h:61-74
+  bool active = false;
+  uint64_t idx = 0;
+  union loadMeta* mem = nullptr;
+  uint64_t* cnt = nullptr;  // nullptr also marks "no slot allocated yet" (src/net_tcpx.cc:890)
+  uint64_t cnt_cache = 0;
+  size_t* flow_cnt = nullptr;
+  size_t* pgtok_cnts = nullptr;  // [kMaxFlows]
+  int* flows = nullptr;          // [kMaxFlows]
+  PageToken* pgtoks = nullptr;   // [kMaxFlows][kSlotPages]
+};
+
+ncclResult_t unpack_queue_new(int dev, bool passive, UnpackQueue** queue);
+void unpack_queue_free(UnpackQueue* queue);
+// src/devcomm/nccl/unpack1.h:30-65
+void unpack_queue_next_free(UnpackQueue* queue, UnpackSlot* slot);
+
+// ---- synthetic devmem socket --------------------------------------------------------------------------------------
+struct DevmemVec {  // struct devmemvec, src/sock/tcpx.h:130-134
+  uint32_t frag_offset;
+  uint32_t frag_size;
+  uint32_t frag_token;
+};
+
+struct DataPipe {  // struct tcpxDataPipe, src/sock/datapipe.h:25-46
+  std::vector<char> ctrl_data;           // control-message buffer handed to recvmsg
+  std::vector<union loadMeta> scatter_list;  // [kSlotPages]
+  uint64_t cnt_cache = 0;
+  int bytes_cnt = 0;
+  size_t* pgtok_cnt = nullptr;
+  PageToken* pgtoks = nullptr;
+  DataPipe();
+};
+
+struct DeviceState;
+
+// One data flow's receive queue: what the kernel has for this socket.  recvmsg() hands out at most `max_bytes`
+// and at most the control buffer's worth of fragments, one SCM_DEVMEM_OFFSET control message each, splitting a
+// fragment when the byte budget ends inside it (the kernel does the same at the end of a recvmsg).
+struct DevmemSocket {
+  std::mutex mu;
+  std::deque<tcpxSynthFrag> rx;
+  uint32_t max_frags_per_recvmsg = 0;  // 0 = no extra limit
+  DeviceState* device = nullptr;       // page accounting
+  ssize_t recvmsg(struct msghdr* msg, size_t max_bytes);
+  // setsockopt(SO_DEVMEM_DONTNEED): gives page references back (src/sock/tcpx.h:299-307).
+  int dontneed(const PageToken* tokens, size_t n);
+};
+
+// Walks the control messages of one recvmsg and appends one descriptor per devmem fragment to the pipe, coalescing
+// consecutive page tokens (process_recv_cmsg, src/sock/tcpx.h:136-228).  Returns the bytes described, or -1 with
+// *result set when the reference would have stopped the process.
+ssize_t process_recv_cmsg(struct msghdr* msg, DataPipe* pipe, int offset, uint64_t dst_base_offset,
+                          ncclResult_t* result);
+// recvmsg + process_recv_cmsg for one task (gpudirectTCPXRecv, src/sock/tcpx.h:230-297).
+ssize_t devmem_recv(DevmemSocket* sock, int size, int offset, DataPipe* pipe, uint64_t dst_base_offset,
+                    ncclResult_t* result);
+
+// ---- requests and tasks -------------------------------------------------------------------------------------------
+struct Comm;
+struct Request;
+
+struct Task {  // struct tcpxTask, src/work_queue.h:38-59 (receive-side fields)
+  int op = 0;
+  int size = 0;
+  int offset = 0;
+  int request_offset = 0;
+  void* data = nullptr;
+  Request* r = nullptr;
+  ncclResult_t result = ncclSuccess;
+  DataPipe* pipe = nullptr;
+  int flow = 0;
+};
+
+enum TaskStage { kTaskActive = 0, kTaskCompleting = 1, kTaskInactive = 2, kTaskStages = 3 };
+struct TaskRing : StageRing<Task, kMaxTasks, kTaskStages, std::atomic<uint32_t>> {
+  TaskRing();
+  ~TaskRing();
+};
+
+struct Request {  // struct tcpxRequest, src/work_queue.h:63-76
+  Comm* comm = nullptr;
+  void* data = nullptr;
+  int op = 0;
+  int mem_type = 0;
+  int next_flow = -1;  // next_sock_id: >= 0 once a control message is pending for this request
+  int next_size = 0;
+  int offset = 0;
+  int size = 0;
+  int size_pending = 0;
+  UnpackSlot slot;
+  // Engine hand-off: the slot has been submitted, and the value its completion word will take.
+  bool published = false;
+  uint64_t done_value = 0;
+};
+
+enum RequestStage { kReqPosted = 0, kReqActive = 1, kReqTransmitting = 2, kReqInactive = 3, kReqStages = 4 };
+using RequestRing = StageRing<Request, kMaxRequests, kReqStages, uint32_t>;
+
+struct CtrlMessage {  // struct tcpxCtrl, src/common.h:127-133 (16 bytes on the wire)
+  uint16_t type;
+  uint16_t index;
+  uint32_t size;
+  uint32_t offset;
+  uint32_t total;
+} __attribute__((__packed__));
+static_assert(sizeof(CtrlMessage) == 16, "control message is 16 bytes");
+
+struct MemHandle {  // struct tcpxMemHandle, src/common.h:90-98
+  void* ptr;
+  int mem_type;
+};
+
+struct FlowData {  // struct tcpxFdData, src/common.h:144-157 (receive-side fields)
+  DevmemSocket sock;
+  TaskRing tasks;
+  uint64_t bytes = 0;
+};
+
+struct Comm {  // struct tcpxComm, src/common.h:159-216
+  bool passive = false;
+  int dev = 0;
+  int num_flows = 0;
+  int end_flow_idx = 0;
+  FlowData flows[kMaxFlows];
+  std::mutex ctrl_mu;
+  std::deque<CtrlMessage> ctrl_rx;  // the control socket's receive queue
+  RequestRing rq;
+  UnpackQueue* queue = nullptr;
+  DeviceState* device = nullptr;
+  uint64_t done_seq = 0;
+  // Optional socket thread (persistentSocketThread, src/net_tcpx.cc:252-384).
+  std::thread helper;
+  std::atomic<bool> helper_stop{false};
+  bool use_helper = false;
+};
+
+struct ListenComm {  // struct tcpxListenComm, src/common.h:112-124
+  int dev;
+  uint64_t id;
+};
+
+// ---- per-GPU and global state -------------------------------------------------------------------------------------
+struct QueueBlock {  // mapped metadata + device handle, recycled between comms (freed only when the engine is stopped)
+  QueueMeta* meta;
+  QueueMeta* meta_dev;
+  struct unpackNetDeviceHandle* dev_handle;
+};
+
+struct DeviceState {
+  int dev = 0;
+  std::mutex mu;
+  void* arena = nullptr;
+  size_t arena_bytes = 0;
+  std::unique_ptr<std::atomic<int32_t>[]> page_refs;  // references held by the plugin, per arena page
+  size_t n_pages = 0;
+  std::atomic<uint64_t> pages_outstanding{0};
+  tcpxuEngine* engine = nullptr;
+  bool engine_started = false;
+  int comms = 0;
+  std::vector<QueueBlock> free_blocks;
+};
+
+struct Global {
+  std::mutex mu;
+  bool initialized = false;
+  ncclDebugLogger_t logger = nullptr;
+  const tcpxDeviceOps* ops = nullptr;
+  bool ops_injected = false;
+  int n_devices = 0;
+  DeviceState devices[kMaxDevices];
+  // Flags (environment, range-checked in tcpxInit like TCPX_GET_INT_FLAG, src/net_tcpx.cc:440-452).
+  int flows_per_comm = 4;
+  int use_helper_thread = 0;
+  bool fail_stop = true;
+  char dev_names[kMaxDevices][32];
+  char pci_paths[kMaxDevices][64];
+};
+extern Global g;
+
+const tcpxDeviceOps* default_device_ops();  // binds libtcpxu_hip.so, or nullptr (reason logged)
+ncclResult_t device_result(int rc, const char* what);
+// Called where the reference stops the process; honours tcpxSetFailStopForTesting.
+ncclResult_t fail_stop(const char* what);
+
+}  // namespace tcpx
+
+#endif  // TCPX_AMD_PLUGIN_INTERNAL_H_

@@ -144,7 +144,8 @@ void gen_adversarial(tcpxSynthWorkload& w, uint64_t total) {
       uint32_t page;
       do page = static_cast<uint32_t>(pages.below(n_pages)); while (used_in[page] == window);
       used_in[page] = window;
-      const uint32_t in_page = static_cast<uint32_t>(offsets.between(0, kPage - len));
+      // An empty fragment still points into its page (offset 0..4095).
+      const uint32_t in_page = static_cast<uint32_t>(offsets.between(0, kPage - std::max(len, 1u)));
       w.add(page, in_page, len, static_cast<uint32_t>(w.descs.size() % w.info.n_flows), done + in_req);
       in_req += len;
     }

@@ -1,0 +1,411 @@
+"""Host logic of the plugin (no GPU): ncclNet_v7 surface, request ring, slot ring, descriptor builder, page
+recycle, completion semantics.  The GPU is replaced by tests/emu (host memory + the CPU oracle as the copier),
+installed through the plugin's testing seam; nothing here measures or ships that path.
+
+Reference behaviour that each test pins is cited as src/...:line of google/nccl-plugin-gpudirecttcpx.
+"""
+import ctypes
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+import __graft_entry__ as graft
+from plugin_common import ROOT, expected_bytes, load_emu
+
+sys.path.insert(0, os.path.join(ROOT, "oracle"))
+import host_logic  # noqa: E402  (test infrastructure)
+
+ARENA_BYTES = 64 << 20
+INTERNAL_ERROR, INVALID_ARGUMENT, INVALID_USAGE = 3, 4, 5
+
+
+@pytest.fixture(scope="module")
+def env(pkg):
+    emu = load_emu()
+    lib = pkg.plugin_lib()
+    assert lib.tcpxSetDeviceOpsForTesting(emu.emu_ops()) == 0
+    assert lib.tcpxSetFailStopForTesting(0) == 0
+    assert lib.tcpxInit(None) == 0
+    base = ctypes.c_void_p()
+    assert lib.tcpxSynthArenaCreate(0, ARENA_BYTES, ctypes.byref(base)) == 0
+    from nccl_plugin_gpudirecttcpx_amd import synth_driver
+
+    class Env:
+        pass
+
+    e = Env()
+    e.pkg, e.lib, e.emu, e.driver, e.arena = pkg, lib, emu, synth_driver, base.value
+    e.arena_np = np.frombuffer((ctypes.c_uint8 * ARENA_BYTES).from_address(base.value), dtype=np.uint8)
+    yield e
+    assert lib.tcpxFinalize() == 0
+    assert emu.emu_counter(1) == 0 and emu.emu_counter(2) == 0 and emu.emu_counter(3) == 0, "finalize leaked"
+    lib.tcpxSetFailStopForTesting(1)
+    assert lib.tcpxSetDeviceOpsForTesting(None) == 0
+
+
+@pytest.fixture
+def comm(env):
+    c = env.driver.RecvComm(0)
+    env.emu.emu_set_hold(0)
+    env.emu.emu_set_ring_full(0)
+    yield c
+    env.emu.emu_set_hold(0)
+    env.emu.emu_release(1 << 20)
+    c.close()
+
+
+def host_buffer(nbytes):
+    buf = np.full(nbytes, 0xA5, dtype=np.uint8)
+    return buf, buf.ctypes.data
+
+
+def test_v7_table_matches_reference_layout(env):
+    """Name string, 19 members in order, regMrDmaBuf absent, closeSend == closeRecv (src/nccl_plugin.cc:22-42)."""
+    lib, t = env.lib, env.lib.table
+    assert ctypes.string_at(t.name) == b"GPUDirectTCPX_v7"
+    assert ctypes.sizeof(env.pkg.NetV7) == 19 * 8
+
+    def addr(name):
+        return ctypes.cast(getattr(lib, name), ctypes.c_void_p).value
+
+    expect = {
+        "init": "tcpxInit", "devices": "tcpxDevices", "getProperties": "tcpxGetProperties", "listen": "tcpxListen",
+        "connect": "tcpxConnect_v5", "accept": "tcpxAccept_v5", "regMr": "tcpxRegMr", "deregMr": "tcpxDeregMr",
+        "isend": "tcpxIsend_v5", "irecv": "tcpxIrecv_v5", "iflush": "tcpxIflush_v5", "test": "tcpxTest",
+        "closeSend": "tcpxClose", "closeRecv": "tcpxClose", "closeListen": "tcpxCloseListen",
+        "getDeviceMr": "tcpxGetDeviceMr", "irecvConsumed": "tcpxIrecvConsumed",
+    }  # fmt: skip
+    for member, fn in expect.items():
+        assert getattr(t, member) == addr(fn), member
+    assert t.regMrDmaBuf is None
+
+
+def test_properties_and_device_handle(env, comm):
+    """src/net_tcpx.cc:725-744 and 1463-1467."""
+    n = ctypes.c_int()
+    assert env.lib.tcpxDevices(ctypes.byref(n)) == 0 and n.value == 1
+    p = env.pkg.NetProperties()
+    assert env.lib.tcpxGetProperties(0, ctypes.byref(p)) == 0
+    assert (p.guid, p.ptrSupport, p.port, p.maxComms, p.latency, p.maxRecvs) == (0, 3, 0, 65536, 0.0, 1)
+    assert (p.netDeviceType, p.netDeviceVersion, p.speed) == (1, 7, 10000)
+    assert env.lib.tcpxGetProperties(5, ctypes.byref(p)) == INTERNAL_ERROR
+    h = comm.dev_handle
+    assert (h.netDeviceType, h.netDeviceVersion, h.size, h.needsProxyProgress) == (1, 7, 24, 1)
+    # the 24-byte device handle: {meta, bounce_buf, head = -1} (src/devcomm/nccl/unpack1.cu:54-63)
+    raw = (ctypes.c_uint64 * 3).from_address(h.handle)
+    assert raw[1] == env.arena and raw[2] == 2**64 - 1 and raw[0] != 0
+
+
+def fill_arena(env, wl):
+    assert wl.info.pool_bytes <= ARENA_BYTES
+    pool = env.arena_np[: wl.info.pool_bytes]
+    wl.fill_window(0, pool)
+    return pool
+
+
+@pytest.mark.parametrize("config,shrink", [(1, 0), (2, 2), (3, 4), (4, 5), (5, 3)])
+def test_receive_workloads_byte_exact(env, comm, config, shrink):
+    wl = env.pkg.Workload(config, seed=0xAB00 + config, shrink=shrink)
+    pool = fill_arena(env, wl)
+    buf, ptr = host_buffer(int(wl.info.dst_bytes) + 64)
+    env.driver.run_workload(comm, wl, ptr, n_flows=4, window=8)
+    want = expected_bytes(pool, wl.frags, wl.requests, int(wl.info.dst_bytes) + 64)
+    assert np.array_equal(buf, want)
+    assert comm.outstanding_pages() == 0, "pages not recycled (src/sock/tcpx.h:310-326)"
+    head, tail, idx = comm.queue_state()
+    assert head == tail == len(wl.requests) and len(set(idx)) == 1 and idx[0] == len(wl.requests)
+
+
+def test_partial_recvmsg_and_window_one(env, comm):
+    """Fragments trickle in three per recvmsg; one request in flight at a time."""
+    wl = env.pkg.Workload(2, seed=77, shrink=3)
+    pool = fill_arena(env, wl)
+    assert env.lib.tcpxSynthSetRecvmsgLimit(comm.comm, 3) == 0
+    buf, ptr = host_buffer(int(wl.info.dst_bytes))
+    env.driver.run_workload(comm, wl, ptr, n_flows=4, window=1)
+    assert np.array_equal(buf, expected_bytes(pool, wl.frags, wl.requests, int(wl.info.dst_bytes)))
+    assert comm.outstanding_pages() == 0
+
+
+def drive_until_transmitted(comm, req, limit=100000):
+    """Polls test() until every fragment of the request has been turned into descriptors (the engine is held)."""
+    for _ in range(limit):
+        rc, done, _ = comm.test(req)
+        assert rc == 0 and done == 0
+        if comm.emu.emu_pending() > 0:
+            return
+    raise AssertionError("request never reached the engine")
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_descriptors_match_restated_builder(env, comm, seed):
+    """The slot's descriptor list equals what process_recv_cmsg (src/sock/tcpx.h:136-228) produces for the same
+    control messages: one flow, random chunk sizes, random fragments per recvmsg."""
+    rng = np.random.default_rng(seed)
+    comm.emu = env.emu
+    n = int(rng.integers(5, 300))
+    sizes = rng.integers(1, 4097, size=n).astype(np.uint32)
+    pages = rng.choice(ARENA_BYTES // 4096, size=n, replace=False).astype(np.uint32)
+    in_page = (rng.integers(0, 4097, size=n) % (4097 - sizes)).astype(np.uint32)
+    # make some page tokens consecutive so that runs get coalesced
+    for i in range(1, n):
+        if rng.random() < 0.3:
+            pages[i] = (pages[i - 1] + 1) % (ARENA_BYTES // 4096)
+    frags = np.zeros(n, dtype=env.pkg.Workload(1, shrink=6).frag_dtype)
+    frags["frag_offset"], frags["frag_size"], frags["frag_token"] = pages * 4096 + in_page, sizes, pages
+    total = int(sizes.sum())
+    per_recvmsg = int(rng.integers(1, 9))
+    assert env.lib.tcpxSynthSetRecvmsgLimit(comm.comm, per_recvmsg) == 0
+    # chunks: random cut points on fragment boundaries, all on flow 0
+    cuts = sorted(set(rng.integers(1, n, size=int(rng.integers(0, 4))).tolist())) if n > 1 else []
+    bounds = [0] + cuts + [n]
+    env.emu.emu_set_hold(1)
+    buf, ptr = host_buffer(total + 16)
+    mh = comm.reg(ptr, total)
+    rc, req = comm.irecv(ptr, total, mh)
+    assert rc == 0
+    # restated builder, fed exactly what the synthetic socket will hand out
+    want, tokens, off = [], [], 0
+    for a, b in zip(bounds[:-1], bounds[1:]):
+        chunk_bytes = int(sizes[a:b].sum())
+        comm.ctrl(0, chunk_bytes, off, total)
+        scatter, task_off = [], 0
+        for k in range(a, b, per_recvmsg):
+            part = [(int(f["frag_offset"]), int(f["frag_size"]), int(f["frag_token"])) for f in frags[k : min(k + per_recvmsg, b)]]
+            task_off += host_logic.process_recv_cmsg(part, scatter, tokens, task_off, off)
+        want += scatter
+        off += chunk_bytes
+    comm.deliver(0, frags)
+    drive_until_transmitted(comm, req)
+    head, tail, _ = comm.queue_state()
+    rows, cnt = comm.slot(head % 16)
+    assert cnt == n
+    got = [(int(r["src_off"]), int(r["len"]), int(r["dst_off"])) for r in rows[:n]]
+    assert got == want
+    assert comm.outstanding_pages() == n  # one reference per control message until consumed
+    env.emu.emu_release(1)
+    rc, done, size = comm.test(req)
+    assert (rc, done) == (0, 1) and size == -12345, "test() never writes *size (src/net_tcpx.cc:1311-1374)"
+    assert comm.consumed(req) == 0
+    assert comm.outstanding_pages() == 0
+    comm.dereg(mh)
+    want_buf = np.full(total + 16, 0xA5, dtype=np.uint8)
+    pos = 0
+    for f in frags:
+        want_buf[pos : pos + int(f["frag_size"])] = env.arena_np[int(f["frag_offset"]) : int(f["frag_offset"]) + int(f["frag_size"])]
+        pos += int(f["frag_size"])
+    assert np.array_equal(buf, want_buf)
+
+
+def simple_request(env, comm, nbytes=8192, page=0):
+    frags = np.zeros(nbytes // 4096, dtype=env.pkg.Workload(1, shrink=6).frag_dtype)
+    frags["frag_offset"] = (page + np.arange(len(frags))) * 4096
+    frags["frag_size"] = 4096
+    frags["frag_token"] = page + np.arange(len(frags))
+    return frags
+
+
+def test_done_only_after_the_copy_completed(env, comm):
+    """done=1 is reported when the engine's completion word arrives, not when descriptors are published."""
+    comm.emu = env.emu
+    env.emu.emu_set_hold(1)
+    buf, ptr = host_buffer(8192)
+    mh = comm.reg(ptr, 8192)
+    rc, req = comm.irecv(ptr, 8192, mh)
+    comm.ctrl(1, 8192, 0, 8192)
+    comm.deliver(1, simple_request(env, comm))
+    drive_until_transmitted(comm, req)
+    for _ in range(50):
+        assert comm.test(req)[:2] == (0, 0)
+    assert (buf == 0xA5).all()
+    submitted = env.emu.emu_counter(0)
+    env.emu.emu_release(1)
+    assert comm.test(req)[:2] == (0, 1)
+    assert env.emu.emu_counter(0) == submitted, "a request is submitted to the engine exactly once"
+    assert np.array_equal(buf, env.arena_np[:8192])
+    assert comm.consumed(req) == 0
+    comm.dereg(mh)
+
+
+def test_engine_ring_full_is_retried(env, comm):
+    buf, ptr = host_buffer(8192)
+    mh = comm.reg(ptr, 8192)
+    rc, req = comm.irecv(ptr, 8192, mh)
+    comm.ctrl(0, 8192, 0, 8192)
+    comm.deliver(0, simple_request(env, comm))
+    env.emu.emu_set_ring_full(1)
+    for _ in range(20):
+        assert comm.test(req)[:2] == (0, 0)
+    env.emu.emu_set_ring_full(0)
+    for _ in range(20):
+        rc, done, _ = comm.test(req)
+        assert rc == 0
+        if done:
+            break
+    assert done == 1 and np.array_equal(buf, env.arena_np[:8192])
+    assert comm.consumed(req) == 0
+    comm.dereg(mh)
+
+
+def test_irecv_argument_errors_and_ring_capacity(env, comm):
+    """n != 1, NULL mhandle, 17th request: ncclInternalError (src/net_tcpx.cc:926, 866-873)."""
+    buf, ptr = host_buffer(4096)
+    mh = comm.reg(ptr, 4096)
+    data = (ctypes.c_void_p * 2)(ptr, ptr)
+    sizes = (ctypes.c_int * 2)(1, 1)
+    tags = (ctypes.c_int * 2)()
+    mhs = (ctypes.c_void_p * 2)(mh, mh)
+    req = ctypes.c_void_p()
+    assert env.lib.tcpxIrecv_v5(comm.comm, 2, data, sizes, tags, mhs, ctypes.byref(req)) == INTERNAL_ERROR
+    assert comm.irecv(ptr, 4096, None)[0] == INTERNAL_ERROR
+    reqs = []
+    for _ in range(16):
+        rc, r = comm.irecv(ptr, 4096, mh)
+        assert rc == 0
+        reqs.append(r)
+    assert comm.irecv(ptr, 4096, mh)[0] == INTERNAL_ERROR
+    assert comm.queue_state()[2] == [0, 0, 0, 0, 16]
+    # drain them as empty messages so that the comm closes clean
+    for r in reqs:
+        comm.ctrl(0, 0, 0, 0, env.pkg.CTRL_INLINE)
+    for r in reqs:
+        for _ in range(10):
+            rc, done, _ = comm.test(r)
+            assert rc == 0
+            if done:
+                break
+        assert done == 1
+        assert comm.consumed(r) == 0
+    comm.dereg(mh)
+    assert env.lib.tcpxRegMr(None, ptr, 10, 1, ctypes.byref(req)) == INTERNAL_ERROR
+    assert env.lib.tcpxRegMr(comm.comm, ptr, 10, 99, ctypes.byref(req)) == INTERNAL_ERROR
+    assert env.lib.tcpxDeregMr(comm.comm, None) == 0
+
+
+def test_zero_size_message(env, comm):
+    """An empty message takes a slot, completes with cnt = 0 and is consumed through the fast path
+    (src/net_tcpx.cc:1248-1276, 1361, 1500-1504)."""
+    buf, ptr = host_buffer(64)
+    mh = comm.reg(ptr, 64)
+    rc, req = comm.irecv(ptr, 64, mh)
+    assert comm.test(req)[:2] == (0, 0)  # nothing arrived yet
+    comm.ctrl(0, 0, 0, 0, env.pkg.CTRL_INLINE)
+    assert comm.test(req)[:2] == (0, 1)
+    head, tail, _ = comm.queue_state()
+    assert (head, tail) == (0, 1)
+    assert comm.slot(0)[1] == 0
+    sizes = (ctypes.c_int * 1)(777)
+    reqs = (ctypes.c_void_p * 1)(req)
+    assert env.lib.tcpxIflush_v5(comm.comm, 1, None, sizes, None, reqs) == 0 and sizes[0] == 0  # src/net_tcpx.cc:946-954
+    assert env.lib.tcpxIflush_v5(comm.comm, 2, None, sizes, None, reqs) == INTERNAL_ERROR
+    assert comm.consumed(req) == 0
+    assert comm.queue_state()[:2] == (1, 1)
+    assert (buf == 0xA5).all()
+    comm.dereg(mh)
+
+
+def test_order_and_consume_errors(env, comm):
+    """test(NULL); test() out of order; irecvConsumed with NULL / n != 1 / wrong request / before completion
+    (src/net_tcpx.cc:1315-1328, 1479-1535)."""
+    assert env.lib.tcpxTest(None, ctypes.byref(ctypes.c_int()), None) == INTERNAL_ERROR
+    buf, ptr = host_buffer(16384)
+    mh = comm.reg(ptr, 16384)
+    rc, r0 = comm.irecv(ptr, 8192, mh)
+    rc, r1 = comm.irecv(ptr + 8192, 8192, mh)
+    assert env.lib.tcpxIrecvConsumed(comm.comm, 1, None) == INTERNAL_ERROR
+    assert env.lib.tcpxIrecvConsumed(comm.comm, 2, r0) == INTERNAL_ERROR
+    for i, r in enumerate((r0, r1)):
+        comm.ctrl(i, 8192, 0, 8192)
+        comm.deliver(i, simple_request(env, comm, page=2 * i))
+    # both requests have all their data; the second one may not be tested before the first (1322-1328)
+    for _ in range(20):
+        rc, done, _ = comm.test(r1)
+        if rc != 0:
+            break
+    assert rc == INTERNAL_ERROR
+    assert comm.consumed(r0) == INTERNAL_ERROR  # not completed yet: no INACTIVE request (1512-1515)
+    for r in (r0, r1):
+        for _ in range(20):
+            rc, done, _ = comm.test(r)
+            assert rc == 0
+            if done:
+                break
+        assert done == 1
+    assert comm.consumed(r1) == INTERNAL_ERROR  # not the oldest (1517-1521)
+    assert comm.consumed(r0) == 0 and comm.consumed(r1) == 0
+    assert np.array_equal(buf, env.arena_np[:16384])
+    assert comm.outstanding_pages() == 0
+    comm.dereg(mh)
+
+
+def test_too_many_fragments_is_fatal(env, comm):
+    """2048 descriptors in one task stop the reference (src/sock/tcpx.h:183-187); with fail-stop switched off for
+    the test the same condition surfaces as ncclInternalError."""
+    n = 2100
+    frags = np.zeros(n, dtype=env.pkg.Workload(1, shrink=6).frag_dtype)
+    frags["frag_offset"] = np.arange(n) * 4096
+    frags["frag_size"] = 2
+    frags["frag_token"] = np.arange(n)
+    buf, ptr = host_buffer(2 * n)
+    mh = comm.reg(ptr, 2 * n)
+    rc, req = comm.irecv(ptr, 2 * n, mh)
+    comm.ctrl(0, 2 * n, 0, 2 * n)
+    comm.deliver(0, frags)
+    rc = 0
+    for _ in range(50):
+        rc, done, _ = comm.test(req)
+        if rc != 0:
+            break
+    assert rc == INTERNAL_ERROR
+    comm.dereg(mh)
+
+
+def test_devmem_contract_is_enforced(env, comm):
+    bad = simple_request(env, comm)
+    bad["frag_offset"][0] = 4000
+    bad["frag_size"][0] = 200  # crosses a page
+    assert env.lib.tcpxSynthDeliver(comm.comm, 0, bad.ctypes.data, len(bad)) == INVALID_ARGUMENT
+    bad = simple_request(env, comm)
+    bad["frag_offset"][0] = ARENA_BYTES  # outside the arena
+    assert env.lib.tcpxSynthDeliver(comm.comm, 0, bad.ctypes.data, len(bad)) == INVALID_ARGUMENT
+    assert env.lib.tcpxSynthDeliver(comm.comm, 9, bad.ctypes.data, 0) == INVALID_ARGUMENT
+
+
+def test_send_side_is_absent(env):
+    handle = ctypes.create_string_buffer(128)
+    lc, sc, req = ctypes.c_void_p(), ctypes.c_void_p(), ctypes.c_void_p()
+    assert env.lib.tcpxListen(0, handle, ctypes.byref(lc)) == 0
+    assert env.lib.tcpxConnect_v5(0, handle, ctypes.byref(sc), None) == 0
+    assert env.lib.tcpxIsend_v5(sc, None, 0, 0, None, ctypes.byref(req)) == INTERNAL_ERROR
+    assert env.lib.tcpxClose(sc) == 0 and env.lib.tcpxCloseListen(lc) == 0
+
+
+def test_device_ops_cannot_be_swapped_after_init(env):
+    assert env.lib.tcpxSetDeviceOpsForTesting(None) == INVALID_USAGE
+
+
+def test_init_fails_loudly_without_the_hip_layer(tmp_path):
+    """No GPU library, no fallback: tcpxInit reports ncclSystemError (run in a fresh process, with the plugin copied
+    to a directory that holds no libtcpxu_hip.so)."""
+    code = (
+        "import ctypes,shutil,sys\n"
+        "shutil.copy(r'%s/nccl-plugin-gpudirecttcpx_amd/lib/libnccl-net.so', r'%s/libnccl-net.so')\n"
+        "lib=ctypes.CDLL(r'%s/libnccl-net.so')\n"
+        "rc=lib.tcpxInit(None)\n"
+        "print('rc',rc); sys.exit(0 if rc==2 else 1)\n" % (ROOT, tmp_path, tmp_path)
+    )
+    env = dict(os.environ, LD_LIBRARY_PATH="")
+    p = subprocess.run([sys.executable, "-c", code], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env, timeout=120)
+    assert p.returncode == 0, p.stdout
+
+
+def test_socket_thread_mode(tmp_path):
+    """The same receive with fragments consumed by a helper thread per comm (src/net_tcpx.cc:252-384) and 8 flows."""
+    script = os.path.join(ROOT, "tests", "helper_thread_case.py")
+    env = dict(os.environ, NCCL_GPUDIRECTTCPX_AMD_HELPER_THREAD="1", NCCL_GPUDIRECTTCPX_AMD_FLOWS="8")
+    p = subprocess.run([sys.executable, script], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env, timeout=300)
+    assert p.returncode == 0, p.stdout
+    assert "helper-thread case ok" in p.stdout
