@@ -111,12 +111,15 @@ typedef struct tcpxuEngineConfig {
   uint32_t ring_entries;    /* submission ring size, power of two >= 16, 0 = default (1024) */
   uint32_t workgroups;      /* persistent grid size, 0 = fill the GPU */
   uint32_t descs_per_ticket;/* descriptors one workgroup takes at a time, 0 = default */
-  uint32_t spin_limit;      /* 0 = poll until stopped; otherwise the kernel exits by itself after this many
-                               empty polls of the ring (a bounded wait, for tests of the timeout path) */
+  uint32_t spin_limit;      /* the kernel leaves by itself after this many consecutive empty polls of the ring
+                               (about 1.2 us each) and is launched again by the next submission, so that a
+                               device-wide synchronize never waits on an idle engine; 0 = default (400, about
+                               half a millisecond), 0xFFFFFFFF = never leave */
 } tcpxuEngineConfig;
 
 int tcpxuEngineCreate(int device, const tcpxuEngineConfig* config, tcpxuEngine** engine);
-/* Launches the persistent kernel.  The engine can be started and stopped repeatedly. */
+/* Launches the persistent kernel.  The engine can be started and stopped repeatedly; a submission made while
+ * the kernel is away (never started after a stop excepted) brings it back. */
 int tcpxuEngineStart(tcpxuEngine* engine);
 /* Asks the kernel to drain and exit, waits for it, and reports the duration of that launch in
  * microseconds as measured by HIP events on the engine's stream (elapsed_us may be NULL). */
@@ -137,7 +140,7 @@ int tcpxuEngineCompleted(tcpxuEngine* engine, uint64_t* completed);
 /* The configuration in effect (defaults resolved: actual grid size, ring size, ticket size). */
 int tcpxuEngineGetConfig(tcpxuEngine* engine, tcpxuEngineConfig* config);
 
-/* 1 if the persistent kernel is running, 0 if stopped or exited by its spin limit. */
+/* 1 if the persistent kernel is running, 0 if stopped or away after being idle. */
 int tcpxuEngineRunning(tcpxuEngine* engine, int* running);
 
 /* ---- streaming driver (measurement helper) ------------------------------------------------------------ */

@@ -56,6 +56,8 @@ constexpr uint32_t kMaxDescsPerTicket = 64;
 constexpr uint32_t kMaxDescsPerSubmission = 1u << 20;
 constexpr uint32_t kStopReplicas = 64;
 constexpr uint32_t kPollEntries = 4;  // submission entries fetched per leader poll
+constexpr uint32_t kNeverIdleOut = 0xFFFFFFFFu;
+constexpr uint32_t kDefaultIdlePolls = 400;  // empty polls (about 1.2 us each) before the kernel leaves by itself
 constexpr int kTcpxuInProgress = TCPXU_IN_PROGRESS;
 
 // 64-byte record: four 16-byte sectors of three payload words and one stamp word.
@@ -72,7 +74,8 @@ struct HostCtl {  // mapped host memory
   alignas(64) uint64_t stop;       // host -> GPU: drain and exit
   alignas(64) uint64_t head;       // GPU -> host: submissions the leader has consumed
   alignas(64) uint64_t completed;  // GPU -> host: submissions fully unpacked (mirrored when idle and at exit)
-  alignas(64) uint64_t exited;     // GPU -> host: 0 running, 1 stopped on request, 2 spin limit reached
+  alignas(64) uint64_t exited;     // GPU -> host: 0 running, 1 stopped on request, 2 left after being idle
+  alignas(64) uint64_t exiting;    // GPU -> host: the leader is about to leave for idleness (see leader_loop)
   alignas(64) Record ring[1];      // ring_entries follow
 };
 
@@ -222,7 +225,21 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
         mirrored = c;
       }
     }
-    if (spin_limit != 0 && nothing_there && ++idle > spin_limit) {
+    if (spin_limit != kNeverIdleOut && nothing_there && ++idle > spin_limit) {
+      // Idle for long enough: leave, so that a device-wide synchronize by anybody returns.  The host relaunches
+      // the kernel with its next submission.  A submission must not fall between "the leader stopped looking"
+      // and "the host thinks the kernel is running": the leader announces that it is leaving, then looks once
+      // more; the host publishes, then checks the announcement.  Each side stores before it loads (and PCIe
+      // keeps a read behind the posted write issued before it), so at least one of them sees the other.
+      if (lane == 0) sys_store(&ctl->exiting, static_cast<uint64_t>(1));
+      drain_memory_ops();
+      const uint32_t again = sys_load(&ctl->ring[s & ring_mask].w[lane & 15]);
+      const bool there = ((lane & 3) == 3 && lane < 16) ? (again == static_cast<uint32_t>(s + 1)) : true;
+      if (__all(there)) {
+        if (lane == 0) sys_store(&ctl->exiting, static_cast<uint64_t>(0));
+        idle = 0;
+        continue;
+      }
       reason = 2;
       break;
     }
@@ -437,7 +454,8 @@ struct tcpxuEngine {
   uint32_t* jobs_done = nullptr;   // [ring_entries], device memory
   uint32_t* job_target = nullptr;  // [ring_entries], device memory, leader-private
   uint64_t tail = 0;  // host copy
-  bool launched = false;
+  bool launched = false;  // between a launch and the Stop that reaps it (the kernel may have left by itself)
+  uint64_t launches = 0;
   // Mapped slot ring of the streaming driver.  Allocated on first use and kept until the engine is destroyed:
   // hipHostFree waits for every stream of the device, so nothing may be freed while the kernel runs.
   void* stream_host = nullptr;
@@ -492,7 +510,7 @@ int tcpxuEngineCreate(int device, const tcpxuEngineConfig* config, tcpxuEngine**
   e->ring_entries = cfg.ring_entries;
   e->workgroups = cfg.workgroups;
   e->per_ticket = cfg.descs_per_ticket;
-  e->spin_limit = cfg.spin_limit;
+  e->spin_limit = cfg.spin_limit != 0 ? cfg.spin_limit : kDefaultIdlePolls;
   {
     const char* ve = getenv("TCPXU_ENGINE_EAGER");
     const char* vb = getenv("TCPXU_ENGINE_BACKOFF_CAP");
@@ -527,13 +545,8 @@ int tcpxuEngineCreate(int device, const tcpxuEngineConfig* config, tcpxuEngine**
   return TCPXU_SUCCESS;
 }
 
-int tcpxuEngineStart(tcpxuEngine* e) {
-  if (!e) return TCPXU_INVALID_ARGUMENT;
-  std::lock_guard<std::mutex> lock(e->mu);
-  if (e->launched) {
-    set_error("engine already started");
-    return TCPXU_INVALID_USAGE;
-  }
+// Launches the kernel.  Caller holds e->mu; any previous launch has ended (its exit word is set).
+static int launch_locked(tcpxuEngine* e) {
   TCPXU_TRY(use_device(e->device));
   // Per-launch state: exit bookkeeping and stop words start from zero; positions and counters are kept.
   TCPXU_HIP(hipMemsetAsync(reinterpret_cast<uint8_t*>(e->st) + offsetof(DevState, exited_wgs), 0,
@@ -541,6 +554,7 @@ int tcpxuEngineStart(tcpxuEngine* e) {
   std::atomic_thread_fence(std::memory_order_seq_cst);
   e->ctl->stop = 0;
   e->ctl->exited = 0;
+  e->ctl->exiting = 0;
   std::atomic_thread_fence(std::memory_order_seq_cst);
   TCPXU_HIP(hipEventRecord(e->ev_start, e->stream));
   hipLaunchKernelGGL(unpack_engine_kernel, dim3(e->workgroups), dim3(kEngineThreads), 0, e->stream, e->ctl_dev, e->st,
@@ -548,7 +562,22 @@ int tcpxuEngineStart(tcpxuEngine* e) {
   TCPXU_HIP(hipGetLastError());
   TCPXU_HIP(hipEventRecord(e->ev_stop, e->stream));
   e->launched = true;
+  e->launches += 1;
   return TCPXU_SUCCESS;
+}
+
+static uint64_t host_load(const uint64_t* p) {
+  return reinterpret_cast<const std::atomic<uint64_t>*>(p)->load(std::memory_order_acquire);
+}
+
+int tcpxuEngineStart(tcpxuEngine* e) {
+  if (!e) return TCPXU_INVALID_ARGUMENT;
+  std::lock_guard<std::mutex> lock(e->mu);
+  if (e->launched && host_load(&e->ctl->exited) == 0) {
+    set_error("engine already started");
+    return TCPXU_INVALID_USAGE;
+  }
+  return launch_locked(e);
 }
 
 int tcpxuEngineStop(tcpxuEngine* e, double* elapsed_us) {
@@ -635,6 +664,20 @@ int tcpxuEngineSubmit(tcpxuEngine* e, const void* bounce_base, void* dst_base, c
   std::atomic_thread_fence(std::memory_order_release);
   e->tail += 1;
   reinterpret_cast<std::atomic<uint64_t>*>(&e->ctl->tail)->store(e->tail, std::memory_order_release);
+  // The kernel may have left for idleness, or be leaving right now (see leader_loop): publish first, then look.
+  if (e->launched) {
+    std::atomic_thread_fence(std::memory_order_seq_cst);
+    if (host_load(&e->ctl->exiting) != 0 && host_load(&e->ctl->exited) == 0) {
+      const auto t0 = std::chrono::steady_clock::now();
+      while (host_load(&e->ctl->exiting) != 0 && host_load(&e->ctl->exited) == 0) {
+        if (std::chrono::steady_clock::now() - t0 > std::chrono::seconds(5)) {
+          set_error("engine kernel announced that it is leaving and never did");
+          return TCPXU_INTERNAL_ERROR;
+        }
+      }
+    }
+    if (host_load(&e->ctl->exited) == 2) TCPXU_TRY(launch_locked(e));  // it left by itself: bring it back
+  }
   return TCPXU_SUCCESS;
 }
 

@@ -155,7 +155,7 @@ def test_engine_restart_and_empty_submission(pkg, hip, oracle):
     expect = oracle_expected(oracle, pool, descs, 100 * 4096 + 4096)
     g = GpuBuffers(pool, descs, 100 * 4096 + 4096)
     m = Mapped(pkg, hip, descs, 4)
-    e = Engine(pkg, hip)
+    e = Engine(pkg, hip, spin_limit=0xFFFFFFFF)  # never leaves by itself: running() is then deterministic
     for round_ in range(3):
         g.reset()
         for f in range(4):
@@ -208,6 +208,36 @@ def test_engine_spin_limit_exits_by_itself(pkg, hip):
         time.sleep(0.01)
     e.stop()  # reaps the finished launch
     e.destroy()
+
+
+def test_engine_leaves_when_idle_and_returns_on_submit(pkg, hip, oracle):
+    """Default configuration: the kernel leaves after about half a millisecond without work, so a device-wide
+    synchronize returns, and the next submission brings it back without any call besides submit."""
+    import torch
+
+    pool = np.random.default_rng(9).integers(0, 256, size=1 << 20, dtype=np.uint8)
+    descs = make_descs([(i * 4096 + 3, 4000, i * 4000) for i in range(128)])
+    expect = oracle_expected(oracle, pool, descs, 128 * 4000)
+    g = GpuBuffers(pool, descs, 128 * 4000)
+    m = Mapped(pkg, hip, descs, 8)
+    e = Engine(pkg, hip)
+    e.start()
+    for round_ in range(4):
+        g.reset()  # contains a device-wide synchronize: returns only because the idle kernel has left
+        deadline = time.time() + 20
+        while e.running():
+            assert time.time() < deadline
+            time.sleep(0.001)
+        e.submit(g.pool.data_ptr(), g.dst_base, m.desc_dev(0), 64, m.flag_dev(2 * round_), 1)
+        e.submit(g.pool.data_ptr(), g.dst_base, m.desc_dev(64), 64, m.flag_dev(2 * round_ + 1), 1)
+        m.wait(2 * round_, 1)
+        m.wait(2 * round_ + 1, 1)
+        torch.cuda.synchronize()
+        assert first_difference(g.result(), expect) is None
+    e.stop()
+    assert e.completed() == 8
+    e.destroy()
+    m.free()
 
 
 def test_engine_argument_errors(pkg, hip):

@@ -1,0 +1,132 @@
+"""End-to-end GPU parity of the plugin path: irecv -> synthetic fragments -> descriptor builder -> mapped slot ->
+persistent engine -> completion word -> test() -> irecvConsumed, byte-exact against the CPU oracle, on all five
+workloads at their full sizes.  Bounce arena, receive buffers and engine are the real HIP ones.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+
+import __graft_entry__ as graft
+from conftest import GUARD, SENTINEL, first_difference
+
+pytestmark = pytest.mark.gpu
+
+ARENA_BYTES = 1 << 30
+
+
+@pytest.fixture(scope="module")
+def env(pkg):
+    import torch
+
+    lib = pkg.plugin_lib()
+    assert lib.tcpxSetDeviceOpsForTesting(None) == 0  # the real HIP layer
+    assert lib.tcpxInit(None) == 0, "tcpxInit must succeed on a GPU box"
+    base = ctypes.c_void_p()
+    assert lib.tcpxSynthArenaCreate(0, ARENA_BYTES, ctypes.byref(base)) == 0
+    from nccl_plugin_gpudirecttcpx_amd import synth_driver
+
+    class Env:
+        pass
+
+    e = Env()
+    e.pkg, e.lib, e.driver, e.arena, e.torch, e.hip = pkg, lib, synth_driver, base.value, torch, pkg.hip_layer()
+    yield e
+    assert lib.tcpxFinalize() == 0
+
+
+def upload(env, pool, offset=0):
+    pkg = env.pkg
+    pkg.check(env.hip.tcpxuCopyToDevice(0, env.arena + offset, pool.ctypes.data, pool.nbytes), "tcpxuCopyToDevice")
+
+
+@pytest.mark.parametrize("config", [1, 2, 3, 4])
+def test_plugin_workloads_full_size(env, oracle, config):
+    torch = env.torch
+    wl = env.pkg.Workload(config, seed=0xC0FFEE00 + config)
+    info = wl.info
+    pool = np.empty(info.pool_bytes, dtype=np.uint8)
+    wl.fill_window(0, pool)
+    upload(env, pool)
+    expect = np.full(GUARD + info.dst_bytes + GUARD, SENTINEL, dtype=np.uint8)
+    graft.oracle_unpack(oracle, expect[GUARD : GUARD + info.dst_bytes], pool, np.ascontiguousarray(wl.descs))
+    dst = torch.full((GUARD + info.dst_bytes + GUARD,), SENTINEL, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    comm = env.driver.RecvComm(0)
+    print("plugin case: config %d, %d requests, %d fragments" % (config, info.n_requests, info.n_descs), flush=True)
+    env.driver.run_workload(comm, wl, dst.data_ptr() + GUARD, n_flows=4, window=8, timeout_s=30)
+    got = dst.cpu().numpy()  # read back while the engine kernel is still running
+    assert comm.outstanding_pages() == 0
+    head, tail, _ = comm.queue_state()
+    assert head == tail == info.n_requests
+    comm.close()
+    assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
+
+
+def test_plugin_adversarial_with_page_reuse(env, oracle):
+    """32 MiB, lengths 1..4096 with empty fragments, destination base +3, pages refilled between requests:
+    a request's pages are recycled by irecvConsumed before the next window's payload overwrites them."""
+    torch = env.torch
+    wl = env.pkg.Workload(5, seed=0xC0FFEE05)
+    info = wl.info
+    pool = np.empty(info.pool_bytes, dtype=np.uint8)
+    base = GUARD + info.dst_misalign
+    expect = np.full(base + info.dst_bytes + GUARD, SENTINEL, dtype=np.uint8)
+    dst = torch.full((base + info.dst_bytes + GUARD,), SENTINEL, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    comm = env.driver.RecvComm(0)
+    mh = comm.reg(dst.data_ptr() + base, int(info.dst_bytes))
+    for i, r in enumerate(wl.requests):
+        first, n, total = int(r["first_desc"]), int(r["n_descs"]), int(r["bytes"])
+        wl.fill_window(int(r["window"]), pool)
+        upload(env, pool)
+        graft.oracle_unpack(oracle, expect[base : base + info.dst_bytes], pool, np.ascontiguousarray(wl.descs[first : first + n]))
+        rc, req = comm.irecv(dst.data_ptr() + base + int(r["dst_off"]), total, mh)
+        assert rc == 0
+        env.driver.feed_request(comm, wl.frags[first : first + n], total, 2)
+        print("window %d: %d fragments, %d bytes" % (i, n, total), flush=True)
+        import time
+
+        deadline = time.time() + 30
+        while True:
+            rc, done, _ = comm.test(req)
+            assert rc == 0
+            if done:
+                break
+            assert time.time() < deadline, "request %d did not complete" % i
+        assert comm.outstanding_pages() > 0
+        assert comm.consumed(req) == 0
+        assert comm.outstanding_pages() == 0
+    got = dst.cpu().numpy()
+    comm.dereg(mh)
+    comm.close()
+    assert first_difference(got, expect) is None, repr(first_difference(got, expect))
+
+
+def test_two_comms_share_one_engine(env, oracle):
+    torch = env.torch
+    wls = [env.pkg.Workload(2, seed=100 + i, shrink=1) for i in range(2)]
+    pool = np.empty(wls[0].info.pool_bytes, dtype=np.uint8)
+    wls[0].fill_window(0, pool)
+    upload(env, pool)
+    comms = [env.driver.RecvComm(0) for _ in wls]
+    outs = []
+    for c, wl in zip(comms, wls):
+        dst = torch.full((int(wl.info.dst_bytes) + 2 * GUARD,), SENTINEL, dtype=torch.uint8, device="cuda:0")
+        torch.cuda.synchronize()
+        env.driver.run_workload(c, wl, dst.data_ptr() + GUARD, n_flows=4, window=4, timeout_s=30)
+        outs.append(dst)
+    for c, wl, dst in zip(comms, wls, outs):
+        expect = np.full(int(wl.info.dst_bytes) + 2 * GUARD, SENTINEL, dtype=np.uint8)
+        graft.oracle_unpack(oracle, expect[GUARD : GUARD + int(wl.info.dst_bytes)], pool, np.ascontiguousarray(wl.descs))
+        assert first_difference(dst.cpu().numpy(), expect) is None
+        c.close()
+
+
+def test_hip_layer_is_what_init_bound(env):
+    """The plugin on a GPU box runs on libtcpxu_hip.so: the device count it reports is the HIP layer's."""
+    n = ctypes.c_int()
+    m = ctypes.c_int()
+    assert env.lib.tcpxDevices(ctypes.byref(n)) == 0
+    env.pkg.check(env.hip.tcpxuDeviceCount(ctypes.byref(m)), "tcpxuDeviceCount")
+    assert n.value == m.value >= 1
