@@ -26,6 +26,10 @@ import numpy as np
 
 import __graft_entry__ as graft
 
+# HBM bytes moved per algorithmic byte (2 x fragment bytes) by unpack_engine_kernel on the headline workload:
+# hardware counters FETCH_SIZE (x1.99974, its reading for a copy kernel of known size) and WRITE_SIZE (x1.0),
+# 8977134 KiB + 9148340 KiB against 2 x 9011200 KiB over one launch of 1100 steps.
+TRAFFIC_PER_ALGORITHMIC_BYTE = 1.0057
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 CHUNK_CONFIG = 2
 
@@ -59,6 +63,14 @@ def main():
     ap.add_argument("--depth", type=int, default=16, help="slots of the mapped ring in flight")
     ap.add_argument("--cpu-seconds", type=float, default=8.0, help="time budget per CPU baseline leg")
     ap.add_argument("--skip-extras", action="store_true", help="only the headline measurement")
+    ap.add_argument(
+        "--calibrate-copy",
+        type=int,
+        default=0,
+        metavar="MIB",
+        help="run only the plain copy kernel on MIB mebibytes (10 launches) and exit: a kernel of known traffic "
+        "against which hardware counters (FETCH_SIZE, WRITE_SIZE) are scaled",
+    )
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU; --gpus %d is not supported (every GPU would run an independent copy)" % args.gpus)
@@ -70,6 +82,15 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     dev = 0
+    if args.calibrate_copy > 0:
+        n = args.calibrate_copy << 20
+        a = torch.empty(n, dtype=torch.uint8, device="cuda:0").random_(0, 256)
+        b = torch.empty(n, dtype=torch.uint8, device="cuda:0")
+        torch.cuda.synchronize()
+        us = ctypes.c_double()
+        pkg.check(hip.tcpxuCopyKernelTimed(dev, b.data_ptr(), a.data_ptr(), n, 0, 10, ctypes.byref(us)), "tcpxuCopyKernelTimed")
+        print(json.dumps({"kernel": "copy_kernel", "launches": 10, "bytes_read_per_launch": n, "bytes_written_per_launch": n, "launch_us": round(us.value, 2)}))
+        return
     name = ctypes.create_string_buffer(256)
     cus = ctypes.c_int()
     pkg.check(hip.tcpxuDeviceInfo(dev, name, 256, ctypes.byref(cus)), "tcpxuDeviceInfo")
@@ -113,25 +134,29 @@ def main():
     eff = pkg.EngineConfig()
     pkg.check(hip.tcpxuEngineGetConfig(engine, ctypes.byref(eff)), "tcpxuEngineGetConfig")
 
-    def run(items, depth, want_latency=False):
+    def run(items, depth, warmup_items=0, want_latency=False):
         wall, kern = ctypes.c_double(), ctypes.c_double()
         lat = (ctypes.c_double * len(items))() if want_latency else None
-        rc = hip.tcpxuEngineRunTimed(engine, items, len(items), depth, 20000, ctypes.byref(wall), ctypes.byref(kern), lat)
+        rc = hip.tcpxuEngineRunTimed(
+            engine, items, len(items), warmup_items, depth, 20000, ctypes.byref(wall), ctypes.byref(kern), lat
+        )
         pkg.check(rc, "tcpxuEngineRunTimed")
         return wall.value, kern.value, (np.asarray(lat[:]) if want_latency else None)
 
-    # ---- warmup, then exactly K timed steps inside one launch of the persistent kernel ---------------------
-    if args.warmup > 0:
-        run(item_array(0, args.warmup), args.depth)
-    timed_items = item_array(args.warmup, args.steps)
+    # ---- W warm-up steps, then exactly K timed steps, all inside ONE launch of the persistent kernel -------
+    # `value` is timed by the host over the K steps only (publish of the first timed slot -> last completion);
+    # the roofline is the kernel's: all W+K steps' bytes over the launch's duration from HIP events, which is
+    # also what a kernel trace of this command shows for the launch.
+    all_items = item_array(0, args.warmup + args.steps)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    wall_us, kernel_us, _ = run(timed_items, args.depth)
+    wall_us, kernel_us, _ = run(all_items, args.depth, warmup_items=args.warmup * slots_per_step)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     payload = float(sum(workloads[(args.warmup + s) % args.chunks].info.payload_bytes for s in range(args.steps)))
+    launch_payload = float(sum(workloads[s % args.chunks].info.payload_bytes for s in range(args.warmup + args.steps)))
     value_gbps = payload / (wall_us * 1e-6) / 1e9
-    achieved = 2.0 * payload / (kernel_us * 1e-6) / 1e9
+    achieved = 2.0 * launch_payload / (kernel_us * 1e-6) / 1e9
 
     # ---- parity spot check: the last chunk written must equal the oracle's bytes ---------------------------
     oracle = graft.load_oracle()
@@ -173,8 +198,12 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": None,
-            "bytes_per_launch": 2.0 * payload,
+            "traffic": round(2.0 * launch_payload * TRAFFIC_PER_ALGORITHMIC_BYTE),
+            "traffic_source": "FETCH_SIZE and WRITE_SIZE of this kernel on this workload (two rocprofv3 --pmc runs, scaled by "
+            "the same counters on the plain copy kernel: x1.99974 and x1.0) came to %.4f x the algorithmic bytes; "
+            "that ratio times bytes_per_launch" % TRAFFIC_PER_ALGORITHMIC_BYTE,
+            "bytes_per_launch": 2.0 * launch_payload,
+            "steps_per_launch": args.warmup + args.steps,
             "launch_us": round(kernel_us, 1),
         },
         "parity_ok": parity_ok,
@@ -198,12 +227,15 @@ def main():
         _, _, lat64k = run(lat_items, 1, want_latency=True)
         lat4m_items = item_array(0, 200)
         _, _, lat4m = run(lat4m_items, 1, want_latency=True)
+        # the same 64 KiB requests back to back, 16 in flight: requests per second of the small-message storm
+        storm_wall, _, _ = run(lat_items, 16)
         result["latency_us"] = {
             "definition": "host publish of a slot -> host poller observes the completion word, one request in flight",
             "request_64KiB_16_descs": {"p50": round(percentile(lat64k, 50), 2), "p99": round(percentile(lat64k, 99), 2)},
             "request_4MiB_1078_descs": {"p50": round(percentile(lat4m, 50), 2), "p99": round(percentile(lat4m, 99), 2)},
         }
         result["p50_request_us"] = result["latency_us"]["request_64KiB_16_descs"]["p50"]
+        result["storm_64KiB_requests_per_s"] = round(n_lat / (storm_wall * 1e-6))
 
         # Launch-per-batch kernel on the same chunk and on the 256 MiB bulk workload, and a plain copy kernel.
         us = ctypes.c_double()

@@ -165,11 +165,19 @@ typedef struct tcpxuStreamItem {
 int tcpxuEngineStream(tcpxuEngine* engine, const tcpxuStreamItem* items, uint64_t n_items, uint32_t depth,
                       uint32_t stall_timeout_ms, double* wall_us, double* latency_us);
 
+/* Same, with the first `warmup_items` items left out of *wall_us: the clock starts at the publish of item
+ * `warmup_items` and stops at the last completion. */
+int tcpxuEngineStreamWarm(tcpxuEngine* engine, const tcpxuStreamItem* items, uint64_t n_items,
+                          uint64_t warmup_items, uint32_t depth, uint32_t stall_timeout_ms, double* wall_us,
+                          double* latency_us);
+
 /* tcpxuEngineStart + tcpxuEngineStream + tcpxuEngineStop in one call on a stopped engine, so that the
- * persistent kernel's launch covers exactly these items; *kernel_us is that launch's duration from HIP events
- * on the engine's stream (the figure a kernel trace shows for it). */
-int tcpxuEngineRunTimed(tcpxuEngine* engine, const tcpxuStreamItem* items, uint64_t n_items, uint32_t depth,
-                        uint32_t stall_timeout_ms, double* wall_us, double* kernel_us, double* latency_us);
+ * persistent kernel's launch covers exactly these items (warm-up included); *kernel_us is that launch's duration
+ * from HIP events on the engine's stream (the figure a kernel trace shows for it), *wall_us as in
+ * tcpxuEngineStreamWarm. */
+int tcpxuEngineRunTimed(tcpxuEngine* engine, const tcpxuStreamItem* items, uint64_t n_items,
+                        uint64_t warmup_items, uint32_t depth, uint32_t stall_timeout_ms, double* wall_us,
+                        double* kernel_us, double* latency_us);
 
 #ifdef __cplusplus
 }

@@ -177,11 +177,25 @@ _HIP_PROTOTYPES = {
             ctypes.POINTER(ctypes.c_double),
         ],
     ),
+    "tcpxuEngineStreamWarm": (
+        ctypes.c_int,
+        [
+            ctypes.c_void_p,
+            ctypes.POINTER(StreamItem),
+            ctypes.c_uint64,
+            ctypes.c_uint64,
+            ctypes.c_uint32,
+            ctypes.c_uint32,
+            ctypes.POINTER(ctypes.c_double),
+            ctypes.POINTER(ctypes.c_double),
+        ],
+    ),
     "tcpxuEngineRunTimed": (
         ctypes.c_int,
         [
             ctypes.c_void_p,
             ctypes.POINTER(StreamItem),
+            ctypes.c_uint64,
             ctypes.c_uint64,
             ctypes.c_uint32,
             ctypes.c_uint32,

@@ -706,6 +706,11 @@ int tcpxuEngineRunning(tcpxuEngine* e, int* running) {
 
 int tcpxuEngineStream(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_items, uint32_t depth,
                       uint32_t stall_timeout_ms, double* wall_us, double* latency_us) {
+  return tcpxuEngineStreamWarm(e, items, n_items, 0, depth, stall_timeout_ms, wall_us, latency_us);
+}
+
+int tcpxuEngineStreamWarm(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_items, uint64_t warmup_items,
+                          uint32_t depth, uint32_t stall_timeout_ms, double* wall_us, double* latency_us) {
   if (!e || !items || !wall_us || depth == 0 || depth > TCPXU_QUEUE_DEPTH) return TCPXU_INVALID_ARGUMENT;
   for (uint64_t i = 0; i < n_items; ++i) {
     if (items[i].n_descs > TCPXU_SLOT_PAGES) {
@@ -743,7 +748,7 @@ int tcpxuEngineStream(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_i
   std::vector<clock::time_point> published(depth);
   int rc = TCPXU_SUCCESS;
   uint64_t next_submit = 0, next_done = 0;
-  const auto t_begin = clock::now();
+  auto t_begin = clock::now();
   auto last_progress = t_begin;
   auto t_end = t_begin;
   while (next_done < n_items) {
@@ -768,6 +773,7 @@ int tcpxuEngineStream(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_i
       if (it.n_descs && !descs_in_hbm && !(skip_copy && next_submit >= depth))
         memcpy(slot_host, it.descs_host, sizeof(tcpxuLoadMeta) * it.n_descs);
       published[slot] = clock::now();
+      if (next_submit == warmup_items) t_begin = published[slot];
       const void* descs_dev = db + flags_bytes + slot_bytes * slot;
       if (descs_in_hbm && it.n_descs) descs_dev = hbm_copies[it.descs_host];
       rc = tcpxuEngineSubmit(e, it.bounce_base, it.dst_base, descs_dev, it.n_descs,
@@ -796,8 +802,9 @@ int tcpxuEngineStream(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_i
   return rc;
 }
 
-int tcpxuEngineRunTimed(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_items, uint32_t depth,
-                        uint32_t stall_timeout_ms, double* wall_us, double* kernel_us, double* latency_us) {
+int tcpxuEngineRunTimed(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_items, uint64_t warmup_items,
+                        uint32_t depth, uint32_t stall_timeout_ms, double* wall_us, double* kernel_us,
+                        double* latency_us) {
   if (!e || !kernel_us) return TCPXU_INVALID_ARGUMENT;
   // Touch the stream block before the launch so that no allocation happens while the kernel is timed.
   if (!e->stream_host) {
@@ -805,7 +812,7 @@ int tcpxuEngineRunTimed(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n
     TCPXU_TRY(tcpxuMappedAlloc(e->device, bytes, &e->stream_host, &e->stream_dev));
   }
   TCPXU_TRY(tcpxuEngineStart(e));
-  const int rc = tcpxuEngineStream(e, items, n_items, depth, stall_timeout_ms, wall_us, latency_us);
+  const int rc = tcpxuEngineStreamWarm(e, items, n_items, warmup_items, depth, stall_timeout_ms, wall_us, latency_us);
   const int rc_stop = tcpxuEngineStop(e, kernel_us);
   return rc != TCPXU_SUCCESS ? rc : rc_stop;
 }
