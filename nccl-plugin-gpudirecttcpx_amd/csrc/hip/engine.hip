@@ -36,7 +36,6 @@
 #include <mutex>
 #include <new>
 #include <thread>
-#include <unordered_map>
 #include <vector>
 
 #include "hip_common.h"
@@ -730,20 +729,6 @@ int tcpxuEngineStreamWarm(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t
   uint8_t* hb = static_cast<uint8_t*>(e->stream_host);
   uint8_t* db = static_cast<uint8_t*>(e->stream_dev);
   memset(hb, 0, flags_bytes);
-  // Probe switch for tuning: after the ring's first lap, reuse the descriptors already in each slot.
-  const bool skip_copy = getenv("TCPXU_STREAM_SKIP_COPY") != nullptr;
-  // Probe switch for tuning: descriptors pre-staged in device memory instead of the mapped slots.
-  const bool descs_in_hbm = getenv("TCPXU_STREAM_DESCS_IN_HBM") != nullptr;
-  std::unordered_map<const void*, void*> hbm_copies;
-  if (descs_in_hbm) {
-    for (uint64_t i = 0; i < n_items; ++i) {
-      if (!items[i].n_descs || hbm_copies.count(items[i].descs_host)) continue;
-      void* d = nullptr;
-      TCPXU_HIP(hipMalloc(&d, sizeof(tcpxuLoadMeta) * items[i].n_descs));
-      TCPXU_HIP(hipMemcpy(d, items[i].descs_host, sizeof(tcpxuLoadMeta) * items[i].n_descs, hipMemcpyHostToDevice));
-      hbm_copies[items[i].descs_host] = d;  // leaked on purpose: probe only
-    }
-  }
   using clock = std::chrono::steady_clock;
   std::vector<clock::time_point> published(depth);
   int rc = TCPXU_SUCCESS;
@@ -770,12 +755,11 @@ int tcpxuEngineStreamWarm(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t
       const uint32_t slot = static_cast<uint32_t>(next_submit % depth);
       const tcpxuStreamItem& it = items[next_submit];
       uint8_t* slot_host = hb + flags_bytes + slot_bytes * slot;
-      if (it.n_descs && !descs_in_hbm && !(skip_copy && next_submit >= depth))
+      if (it.n_descs)
         memcpy(slot_host, it.descs_host, sizeof(tcpxuLoadMeta) * it.n_descs);
       published[slot] = clock::now();
       if (next_submit == warmup_items) t_begin = published[slot];
       const void* descs_dev = db + flags_bytes + slot_bytes * slot;
-      if (descs_in_hbm && it.n_descs) descs_dev = hbm_copies[it.descs_host];
       rc = tcpxuEngineSubmit(e, it.bounce_base, it.dst_base, descs_dev, it.n_descs,
                              db + flag_stride * slot, next_submit + 1);
       if (rc == kTcpxuInProgress) {
