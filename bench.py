@@ -6,8 +6,10 @@
 One "step" is the unpack of one 8 MiB chunk of the 4-flow workload (about 2155 descriptors of at most 4 KiB,
 byte-unaligned sources in a 256 MiB bounce pool, contiguous destination), cut into two 4 MiB requests the way
 NCCL slices an 8 MiB chunk.  The chunk goes through the persistent engine exactly as the plugin drives it:
-descriptors are copied into a slot of the 16-deep mapped ring, the slot is published, the GPU unpacks it and
-writes a completion word that the host polls -- no kernel launch per request.  Successive steps use different
+descriptors are copied into a slot of a 16-deep mapped ring, the slot is published, the GPU unpacks it and
+writes a completion word that the host polls -- no kernel launch per request.  One engine serves every receive
+comm of the GPU; the headline keeps `--comms` (4) comms busy, each with the reference's queue depth of 16, taking
+turns; the same run with a single comm is reported beside it (`single_comm`).  Successive steps use different
 descriptor lists and different destinations (a ring of chunks bigger than the 256 MiB Infinity Cache), so the
 figure is HBM traffic, not cache hits.  Bounce pool, descriptor lists and destinations are resident before the
 timed region starts; nothing crosses PCIe during it except descriptors and completion words.
@@ -60,7 +62,8 @@ def main():
     ap.add_argument("--steps", type=int, default=4000)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--chunks", type=int, default=48, help="distinct chunks (descriptor lists + destinations) cycled through")
-    ap.add_argument("--depth", type=int, default=16, help="slots of the mapped ring in flight")
+    ap.add_argument("--comms", type=int, default=4, help="receive comms kept busy on the one engine (1..4)")
+    ap.add_argument("--depth", type=int, default=16, help="slots of one comm's mapped ring in flight (the unpack queue depth)")
     ap.add_argument("--cpu-seconds", type=float, default=8.0, help="time budget per CPU baseline leg")
     ap.add_argument("--skip-extras", action="store_true", help="only the headline measurement")
     ap.add_argument(
@@ -72,6 +75,8 @@ def main():
         "against which hardware counters (FETCH_SIZE, WRITE_SIZE) are scaled",
     )
     args = ap.parse_args()
+    if not 1 <= args.comms <= 4 or not 1 <= args.depth <= 16:
+        sys.exit("bench.py: --comms must be 1..4 and --depth 1..16")
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU; --gpus %d is not supported (every GPU would run an independent copy)" % args.gpus)
 
@@ -148,9 +153,11 @@ def main():
     # the roofline is the kernel's: all W+K steps' bytes over the launch's duration from HIP events, which is
     # also what a kernel trace of this command shows for the launch.
     all_items = item_array(0, args.warmup + args.steps)
+    # An untimed launch first: brings the clocks up from idle and touches every page once.
+    run(item_array(0, max(args.warmup, 1)), args.comms * args.depth)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    wall_us, kernel_us, _ = run(all_items, args.depth, warmup_items=args.warmup * slots_per_step)
+    wall_us, kernel_us, _ = run(all_items, args.comms * args.depth, warmup_items=args.warmup * slots_per_step)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     payload = float(sum(workloads[(args.warmup + s) % args.chunks].info.payload_bytes for s in range(args.steps)))
@@ -181,15 +188,17 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": "8 MiB chunk, 4 interleaved flows, ~2155 fragments (90%% 4096 B, 10%% U[64,4095]), byte-unaligned "
-            "sources in a 256 MiB pool, 2 x 4 MiB requests per chunk, %d distinct chunks cycled, ring depth %d"
-            % (args.chunks, args.depth),
+            "sources in a 256 MiB pool, 2 x 4 MiB requests per chunk, %d distinct chunks cycled; %d receive comms on "
+            "one engine, unpack queue depth %d each" % (args.chunks, args.comms, args.depth),
+            "comms": args.comms,
+            "queue_depth_per_comm": args.depth,
             "path": "persistent engine: mapped descriptor ring -> gfx950 unpack kernel -> mapped completion word",
             "descriptors_per_step": round(descs_per_step, 1),
             "slots_per_step": slots_per_step,
             "device": name.value.decode(),
             "compute_units": cus.value,
             "engine_workgroups": eff.workgroups,
-            "descs_per_ticket": eff.descs_per_ticket,
+            "descs_per_ticket": eff.descs_per_ticket if eff.descs_per_ticket else "8..32 by backlog",
         },
         "roofline": {
             "bound": "hbm",
@@ -209,6 +218,18 @@ def main():
         "parity_ok": parity_ok,
         "timed_region_s": round(t1 - t0, 4),
     }
+
+    if args.comms > 1:
+        # The same steps with one comm only: 16 slots (at most 64 MiB) in flight, a launch of its own.
+        w1, k1, _ = run(all_items, args.depth, warmup_items=args.warmup * slots_per_step)
+        result["single_comm"] = {
+            "value": round(payload / (w1 * 1e-6) / 1e9, 2),
+            "unit": "GB/s",
+            "ms_per_step": round(w1 / 1000.0 / args.steps, 6),
+            "roofline_achieved": round(2.0 * launch_payload / (k1 * 1e-6) / 1e9, 1),
+            "roofline_frac": round(2.0 * launch_payload / (k1 * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+            "launch_us": round(k1, 1),
+        }
 
     if not args.skip_extras:
         # Request completion latency, one request in flight: publish -> host poller sees the completion word.

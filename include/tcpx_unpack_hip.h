@@ -110,7 +110,9 @@ typedef struct tcpxuEngine tcpxuEngine;
 typedef struct tcpxuEngineConfig {
   uint32_t ring_entries;    /* submission ring size, power of two >= 16, 0 = default (1024) */
   uint32_t workgroups;      /* persistent grid size, 0 = fill the GPU */
-  uint32_t descs_per_ticket;/* descriptors one workgroup takes at a time, 0 = default */
+  uint32_t descs_per_ticket;/* descriptors one workgroup takes at a time (1..64); 0 = chosen per submission from
+                               the backlog of descriptors not yet unpacked: 8 when the engine is idle (lowest
+                               latency) up to 32 when every workgroup has work queued (highest throughput) */
   uint32_t spin_limit;      /* the kernel leaves by itself after this many consecutive empty polls of the ring
                                (about 1.2 us each) and is launched again by the next submission, so that a
                                device-wide synchronize never waits on an idle engine; 0 = default (400, about
@@ -137,7 +139,7 @@ int tcpxuEngineSubmit(tcpxuEngine* engine, const void* bounce_base, void* dst_ba
 /* Number of submissions the GPU has fully completed since creation (monotone; read from mapped memory). */
 int tcpxuEngineCompleted(tcpxuEngine* engine, uint64_t* completed);
 
-/* The configuration in effect (defaults resolved: actual grid size, ring size, ticket size). */
+/* The configuration in effect (defaults resolved: actual grid size, ring size; ticket size 0 = by backlog). */
 int tcpxuEngineGetConfig(tcpxuEngine* engine, tcpxuEngineConfig* config);
 
 /* 1 if the persistent kernel is running, 0 if stopped or away after being idle. */
@@ -154,8 +156,12 @@ typedef struct tcpxuStreamItem {
   uint32_t reserved;
 } tcpxuStreamItem;
 
+/* Slots the streaming driver can keep in flight: the unpack queues of four receive comms. */
+#define TCPXU_STREAM_MAX_DEPTH (4 * TCPXU_QUEUE_DEPTH)
+
 /* Drives a started engine the way the plugin's proxy loop does, from one host thread, with no Python in the
- * loop: a mapped ring of `depth` slots (1..TCPXU_QUEUE_DEPTH) of TCPXU_SLOT_PAGES descriptors each; for every
+ * loop: a mapped ring of `depth` slots (1..TCPXU_STREAM_MAX_DEPTH; TCPXU_QUEUE_DEPTH is one comm's unpack queue,
+ * a multiple of it is that many comms taking turns) of TCPXU_SLOT_PAGES descriptors each; for every
  * item, in order: wait until the slot's previous occupant has completed, copy the item's descriptors into the
  * slot (the memcpy of src/net_tcpx.cc:1128-1130), publish it (src/net_tcpx.cc:1354-1357), and poll completion
  * words in FIFO order (the tcpxTest / tcpxIrecvConsumed cadence).  Writes the wall time from the first publish

@@ -52,9 +52,21 @@ namespace {
 
 constexpr uint32_t kTicketRing = 1u << 16;  // tickets in flight at most
 constexpr uint32_t kMaxDescsPerTicket = 64;
+// Ticket size when the caller does not fix one.  A ticket occupies a workgroup for one pick-up (a claim, the
+// ticket record, the descriptors over PCIe: a few microseconds) plus its copy.  While workgroups are waiting for
+// work, small tickets finish a submission sooner (more workgroups share it); once tickets queue up behind busy
+// workgroups, larger ones spend less of each workgroup's time on pick-ups.  `backlog` estimates the descriptors of
+// all submissions not yet completed, counting each in full until it completes (how far the slots in flight have
+// got depends on the ticket size itself and would feed back).  The steps are where throughput measured at 1 to
+// 64 slots of 4 MiB in flight changed hands between sizes; 8 is one fragment per copy wavefront.
+__device__ __forceinline__ uint32_t ticket_size_for(uint32_t backlog, uint32_t workers) {
+  const uint32_t per_worker = backlog / workers;
+  return per_worker < 13 ? 8u : per_worker < 18 ? 12u : per_worker < 30 ? 16u : per_worker < 75 ? 24u : 32u;
+}
 constexpr uint32_t kMaxDescsPerSubmission = 1u << 20;
 constexpr uint32_t kStopReplicas = 64;
-constexpr uint32_t kPollEntries = 4;  // submission entries fetched per leader poll
+constexpr uint32_t kPollEntries = 16;  // submission entries fetched per leader poll (16 B per lane)
+constexpr uint32_t kAuxTicketsDone = 32, kAuxHostStop = 33, kAuxJobsCompleted = 34;  // lanes of the auxiliary load
 constexpr uint32_t kNeverIdleOut = 0xFFFFFFFFu;
 constexpr uint32_t kDefaultIdlePolls = 400;  // empty polls (about 1.2 us each) before the kernel leaves by itself
 constexpr int kTcpxuInProgress = TCPXU_IN_PROGRESS;
@@ -122,7 +134,7 @@ __device__ __forceinline__ uint32_t lane_value(uint32_t v, uint32_t src_lane) {
 }
 
 __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uint32_t* job_target,
-                            uint32_t ring_mask, uint32_t per_ticket, uint32_t spin_limit) {
+                            uint32_t ring_mask, uint32_t fixed_per_ticket, uint32_t spin_limit) {
   const uint32_t lane = threadIdx.x;
   uint64_t s = sys_load(&st->sub_head);
   uint64_t tickets_out = sys_load(&st->tickets_out);
@@ -131,35 +143,43 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
   uint32_t reason = 0;
   // Fixed per-lane roles in the auxiliary load (second load of every poll), so that both loads of a poll are
   // issued back to back by all lanes and waited for once:
-  //   lanes 0-3  jobs_done of the job slots of entries s..s+3      lanes 4-7  job_target of the same slots
-  //   lane 8     low word of tickets_done                          lane 9     low word of the host stop word
-  //   other lanes repeat lane 9.
+  //   lanes 0-15  jobs_done of the job slots of entries s..s+15    lanes 16-31  job_target of the same slots
+  //   lane 32     low word of tickets_done                         lane 33      low word of the host stop word
+  //   lane 34     low word of jobs_completed                       other lanes repeat lane 33.
   const uint32_t* const tickets_done_lo = reinterpret_cast<const uint32_t*>(&st->tickets_done);
   const uint32_t* const host_stop_lo = reinterpret_cast<const uint32_t*>(&ctl->stop);
+  const uint32_t* const jobs_completed_lo = reinterpret_cast<const uint32_t*>(&st->jobs_completed);
 
   for (;;) {
-    // One round trip fetches entries s .. s+3: lane 16k+i reads word i of entry s+k.
-    const uint32_t k_of_lane = lane >> 4;
-    const uint32_t word = sys_load(&ctl->ring[(s + k_of_lane) & ring_mask].w[lane & 15]);
+    // One round trip fetches entries s .. s+15: lane 4k+j reads sector j (three payload words and the stamp) of
+    // entry s+k.
+    const uint32_t k_of_lane = lane >> 2;
+    const u32x4 sect = load_vec_sys(reinterpret_cast<const uint8_t*>(&ctl->ring[(s + k_of_lane) & ring_mask]) + 16 * (lane & 3));
     const uint32_t* aux_addr = host_stop_lo;
     if (lane < kPollEntries) aux_addr = &jobs_done[(s + lane) & ring_mask];
     else if (lane < 2 * kPollEntries) aux_addr = &job_target[(s + lane - kPollEntries) & ring_mask];
-    else if (lane == 8) aux_addr = tickets_done_lo;
+    else if (lane == kAuxTicketsDone) aux_addr = tickets_done_lo;
+    else if (lane == kAuxJobsCompleted) aux_addr = jobs_completed_lo;
     const uint32_t aux = sys_load(aux_addr);
 
     const uint32_t expect = static_cast<uint32_t>(s + k_of_lane + 1);
-    const bool stamp_ok = ((lane & 3) == 3) ? (word == expect) : true;
-    const uint64_t ok_mask = __ballot(stamp_ok);
-    const uint32_t tickets_done = lane_value(aux, 8);
+    const uint64_t ok_mask = __ballot(sect.w == expect);
+    const uint32_t tickets_done = lane_value(aux, kAuxTicketsDone);
+    const uint32_t jobs_completed = lane_value(aux, kAuxJobsCompleted);
+    // Payload word i of entry k: component i % 3 of sector i / 3, held by lane 4k + i / 3.
+    auto payload_of = [&](uint32_t first_lane, int i) {
+      const uint32_t src = first_lane + static_cast<uint32_t>(i / 3);
+      return lane_value(i % 3 == 0 ? sect.x : i % 3 == 1 ? sect.y : sect.z, src);
+    };
 
     uint32_t consumed = 0;
 #pragma unroll 1
     for (uint32_t k = 0; k < kPollEntries; ++k) {
-      if (((ok_mask >> (16 * k)) & 0xFFFFull) != 0xFFFFull) break;
-      const uint32_t fl = 16 * k;  // first lane of entry k
-      const uint32_t n = lane_value(word, fl + payload_slot(10));
-      const uint32_t flag_lo = lane_value(word, fl + payload_slot(6)), flag_hi = lane_value(word, fl + payload_slot(7));
-      const uint32_t val_lo = lane_value(word, fl + payload_slot(8)), val_hi = lane_value(word, fl + payload_slot(9));
+      if (((ok_mask >> (4 * k)) & 0xFull) != 0xFull) break;
+      const uint32_t fl = 4 * k;  // first lane of entry k
+      const uint32_t n = payload_of(fl, 10);
+      const uint32_t flag_lo = payload_of(fl, 6), flag_hi = payload_of(fl, 7);
+      const uint32_t val_lo = payload_of(fl, 8), val_hi = payload_of(fl, 9);
       if (n == 0) {
         if (lane == 0) {
           sys_store(reinterpret_cast<uint64_t*>((static_cast<uint64_t>(flag_hi) << 32) | flag_lo),
@@ -167,6 +187,10 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
           __hip_atomic_fetch_add(&st->jobs_completed, 1ull, __ATOMIC_RELAXED, SYS);
         }
       } else {
+        // Submissions not yet completed, this one included, taken to be as long as this one.
+        const uint32_t in_flight = static_cast<uint32_t>(s + k) - jobs_completed + 1u;
+        const uint32_t backlog = in_flight > (1u << 20) / n ? (1u << 20) : in_flight * n;
+        const uint32_t per_ticket = fixed_per_ticket != 0 ? fixed_per_ticket : ticket_size_for(backlog, gridDim.x - 1);
         const uint32_t nt = (n + per_ticket - 1) / per_ticket;
         const uint32_t slot = static_cast<uint32_t>(s + k) & ring_mask;
         const uint32_t done_now = lane_value(aux, k);
@@ -178,20 +202,22 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
         if (static_cast<uint32_t>(tickets_out) + nt - tickets_done > kTicketRing) break;
         const uint32_t target = target_prev + nt;
         if (lane == 0) sys_store(&job_target[slot], target);
-        const uint32_t bounce_lo = lane_value(word, fl + payload_slot(0)), bounce_hi = lane_value(word, fl + payload_slot(1));
-        const uint32_t dst_lo = lane_value(word, fl + payload_slot(2)), dst_hi = lane_value(word, fl + payload_slot(3));
-        const uint64_t descs =
-            (static_cast<uint64_t>(lane_value(word, fl + payload_slot(5))) << 32) | lane_value(word, fl + payload_slot(4));
-        for (uint32_t i = lane; i < nt; i += kWaveLanes) {
+        const uint32_t bounce_lo = payload_of(fl, 0), bounce_hi = payload_of(fl, 1);
+        const uint32_t dst_lo = payload_of(fl, 2), dst_hi = payload_of(fl, 3);
+        const uint64_t descs = (static_cast<uint64_t>(payload_of(fl, 5)) << 32) | payload_of(fl, 4);
+        // Four neighbouring lanes write the four sectors of one ticket, so that one store instruction of the
+        // wavefront fills 16 consecutive tickets (1 KiB of whole lines).
+        const uint32_t sector = lane & 3u;
+        for (uint32_t i = lane >> 2; i < nt; i += kWaveLanes / 4) {
           const uint64_t d = descs + static_cast<uint64_t>(i) * per_ticket * sizeof(tcpxuLoadMeta);
           const uint32_t count = std::min(per_ticket, n - i * per_ticket);
           const uint64_t t = tickets_out + i;
           const uint32_t stamp = static_cast<uint32_t>(t + 1);
-          uint8_t* rec = reinterpret_cast<uint8_t*>(&st->tickets[t & (kTicketRing - 1)]);
-          store_vec_sys(rec, u32x4{bounce_lo, bounce_hi, dst_lo, stamp});
-          store_vec_sys(rec + 16, u32x4{dst_hi, static_cast<uint32_t>(d), static_cast<uint32_t>(d >> 32), stamp});
-          store_vec_sys(rec + 32, u32x4{flag_lo, flag_hi, val_lo, stamp});
-          store_vec_sys(rec + 48, u32x4{val_hi, count | (slot << 8), target, stamp});
+          u32x4 v{bounce_lo, bounce_hi, dst_lo, stamp};
+          if (sector == 1) v = u32x4{dst_hi, static_cast<uint32_t>(d), static_cast<uint32_t>(d >> 32), stamp};
+          if (sector == 2) v = u32x4{flag_lo, flag_hi, val_lo, stamp};
+          if (sector == 3) v = u32x4{val_hi, count | (slot << 8), target, stamp};
+          store_vec_sys(reinterpret_cast<uint8_t*>(&st->tickets[t & (kTicketRing - 1)]) + 16 * sector, v);
         }
         tickets_out += nt;
       }
@@ -205,8 +231,8 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
     }
 
     // Nothing could be consumed this round.
-    const bool nothing_there = (ok_mask & 0xFFFFull) != 0xFFFFull;
-    if (lane_value(aux, 9) != 0 && nothing_there) {
+    const bool nothing_there = (ok_mask & 0xFull) != 0xFull;
+    if (lane_value(aux, kAuxHostStop) != 0 && nothing_there) {
       // Stop requested and entry s not there.  The host wrote its last tail before the stop word, so a tail
       // read now bounds what is still to come.
       uint64_t tail_now = 0;
@@ -257,10 +283,10 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
 }
 
 // ---- worker -------------------------------------------------------------------------------------------------------
-// A worker workgroup is kCopyWaves copy wavefronts and one fetcher wavefront.  The fetcher stays one ticket ahead:
-// while the copy wavefronts move ticket i, it claims a number, polls that ticket's slot and pulls the ticket's
-// descriptors over PCIe into the other LDS stage.  Copy wavefronts therefore never wait for PCIe: between two
-// tickets they only meet the fetcher at one barrier.  The copy wavefront that finishes a ticket last counts it.
+// A worker workgroup is kCopyWaves copy wavefronts and one fetcher wavefront.  Towards the end of ticket i the
+// fetcher claims a number, polls that ticket's slot and pulls the ticket's descriptors over PCIe into the other
+// LDS stage; between two tickets the copy wavefronts only meet the fetcher at one barrier.  The copy wavefront
+// that finishes a ticket last counts it.
 #ifndef TCPXU_ENGINE_COPY_WAVES
 #define TCPXU_ENGINE_COPY_WAVES 8
 #endif
@@ -321,23 +347,29 @@ __device__ void retire_ticket(DevState* st, uint32_t* jobs_done, const Stage* st
 }
 
 // Copy wavefront `wave` of kCopyWaves: fragments wave, wave + kCopyWaves, ... of the staged ticket.
-__device__ void copy_ticket(const Stage* stage, uint32_t wave, uint32_t lane) {
+__device__ void copy_ticket(const Stage* stage, uint32_t wave, uint32_t lane, uint32_t* waves_on_last) {
   auto uniform = [](uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(v)); };
   const uint8_t* bounce = reinterpret_cast<const uint8_t*>((static_cast<uint64_t>(uniform(stage->payload[1])) << 32) |
                                                            uniform(stage->payload[0]));
   uint8_t* dst =
       reinterpret_cast<uint8_t*>((static_cast<uint64_t>(uniform(stage->payload[3])) << 32) | uniform(stage->payload[2]));
   const uint32_t n = uniform(stage->payload[10]) & 0xFFu;
-  wave_copy_descriptors<TCPXU_ENGINE_TWO_ROUNDS>(stage->desc, n, wave, kCopyWaves, bounce, dst, lane);
+  wave_copy_descriptors<TCPXU_ENGINE_TWO_ROUNDS>(stage->desc, n, wave, kCopyWaves, bounce, dst, lane, [&] {
+    if (lane == 0) __hip_atomic_fetch_add(waves_on_last, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  });
 }
 
 __device__ void worker_loop(DevState* st, uint32_t* jobs_done, uint32_t flags) {
   __shared__ Stage stages[2];
   __shared__ uint32_t s_waves_done;  // copy wavefronts that have finished (and drained) a ticket, running total
+  __shared__ uint32_t s_waves_on_last;  // copy wavefronts that have turned to their last fragment of a ticket, ditto
   const uint32_t tid = threadIdx.x;
   const uint32_t lane = tid & (kWaveLanes - 1);
   const uint32_t wave = tid / kWaveLanes;
-  if (tid == 0) s_waves_done = 0;
+  if (tid == 0) {
+    s_waves_done = 0;
+    s_waves_on_last = 0;
+  }
   __syncthreads();
 
   if (wave == kCopyWaves) {
@@ -346,19 +378,23 @@ __device__ void worker_loop(DevState* st, uint32_t* jobs_done, uint32_t flags) {
     // copy wavefronts at the barrier.
     //
     // When to claim the next ticket number.  Numbers are served in order, so a number claimed by a workgroup
-    // that is still busy keeps its ticket waiting even if other workgroups are idle.  A fetcher therefore claims
-    // ahead of time ("eager") only while tickets are queueing up -- its previous ticket was already there at the
-    // first look -- and otherwise claims when its copy wavefronts have finished.
+    // that is still busy keeps its ticket waiting even if other workgroups are idle; a number claimed only when
+    // the workgroup is idle leaves the whole pick-up (claim, ticket record, descriptors over PCIe) exposed.  The
+    // fetcher claims when every copy wavefront has turned to its last fragment of the current ticket: what is
+    // left of the copy then takes about as long as the pick-up, so neither waits for the other.  (flags bit 1
+    // clear: claim only when the copy has finished; bit 0 set: claim right away while tickets are queueing up,
+    // i.e. the previous ticket was already there at the first look.)
     const uint32_t* stop_word = &st->stop[blockIdx.x % kStopReplicas].value;
     uint32_t staged = 0;
     bool eager = false;
     const bool allow_eager = (flags & 1u) != 0;
+    const uint32_t* const claim_gate = (flags & 2u) != 0 ? &s_waves_on_last : &s_waves_done;
     const uint32_t backoff_cap = (flags >> 8) & 0xFFu;
     for (;;) {
       Stage* next = &stages[staged & 1];
       if (!eager) {
         // Wait for the copy of ticket staged-1 to finish (LDS only: no memory traffic while waiting).
-        while (__hip_atomic_load(&s_waves_done, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != staged * kCopyWaves)
+        while (__hip_atomic_load(claim_gate, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != staged * kCopyWaves)
           __builtin_amdgcn_s_sleep(1);
       }
       uint64_t t = 0;
@@ -398,7 +434,7 @@ __device__ void worker_loop(DevState* st, uint32_t* jobs_done, uint32_t flags) {
       __syncthreads();  // stage i&1 is ready
       const Stage* stage = &stages[i & 1];
       if (stage->go == 0) break;
-      copy_ticket(stage, wave, lane);
+      copy_ticket(stage, wave, lane, &s_waves_on_last);
       drain_memory_ops();  // this wavefront's write-through stores are acknowledged
       uint32_t arrived = 0;
       if (lane == 0)
@@ -444,7 +480,7 @@ struct tcpxuEngine {
   uint32_t workgroups = 0;
   uint32_t per_ticket = 0;
   uint32_t spin_limit = 0;
-  uint32_t flags = 0;  // bit 0: fetchers may claim ahead; bits 8-15: idle poll backoff cap
+  uint32_t flags = 0;  // bits 0-1: when fetchers claim (see worker_loop); bits 8-15: idle poll backoff cap
   hipStream_t stream = nullptr;
   hipEvent_t ev_start = nullptr, ev_stop = nullptr;
   HostCtl* ctl = nullptr;      // host address of the mapped control block
@@ -477,11 +513,11 @@ int tcpxuEngineCreate(int device, const tcpxuEngineConfig* config, tcpxuEngine**
     return TCPXU_INVALID_ARGUMENT;
   }
   if (cfg.descs_per_ticket == 0) {
-    const char* v = getenv("TCPXU_DESCS_PER_TICKET");
-    cfg.descs_per_ticket = (v && *v) ? static_cast<uint32_t>(atoi(v)) : 16;
+    const char* v = getenv("TCPXU_DESCS_PER_TICKET");  // tuning aid: fixes the size; unset = by backlog
+    if (v && *v) cfg.descs_per_ticket = static_cast<uint32_t>(atoi(v));
   }
-  if (cfg.descs_per_ticket == 0 || cfg.descs_per_ticket > kMaxDescsPerTicket) {
-    set_error("descs_per_ticket %u must be in [1,%u]", cfg.descs_per_ticket, kMaxDescsPerTicket);
+  if (cfg.descs_per_ticket > kMaxDescsPerTicket) {
+    set_error("descs_per_ticket %u must be in [0,%u]", cfg.descs_per_ticket, kMaxDescsPerTicket);
     return TCPXU_INVALID_ARGUMENT;
   }
   TCPXU_TRY(use_device(device));
@@ -513,7 +549,7 @@ int tcpxuEngineCreate(int device, const tcpxuEngineConfig* config, tcpxuEngine**
   {
     const char* ve = getenv("TCPXU_ENGINE_EAGER");
     const char* vb = getenv("TCPXU_ENGINE_BACKOFF_CAP");
-    const uint32_t eager = (ve && *ve) ? static_cast<uint32_t>(atoi(ve)) & 1u : 0u;
+    const uint32_t eager = (ve && *ve) ? static_cast<uint32_t>(atoi(ve)) & 3u : 2u;
     const uint32_t cap = (vb && *vb) ? static_cast<uint32_t>(atoi(vb)) & 0xFFu : 8u;
     e->flags = eager | (cap << 8);
   }
@@ -710,7 +746,7 @@ int tcpxuEngineStream(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_i
 
 int tcpxuEngineStreamWarm(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_items, uint64_t warmup_items,
                           uint32_t depth, uint32_t stall_timeout_ms, double* wall_us, double* latency_us) {
-  if (!e || !items || !wall_us || depth == 0 || depth > TCPXU_QUEUE_DEPTH) return TCPXU_INVALID_ARGUMENT;
+  if (!e || !items || !wall_us || depth == 0 || depth > TCPXU_STREAM_MAX_DEPTH) return TCPXU_INVALID_ARGUMENT;
   for (uint64_t i = 0; i < n_items; ++i) {
     if (items[i].n_descs > TCPXU_SLOT_PAGES) {
       set_error("stream item %llu has %u descriptors, a slot holds %d", static_cast<unsigned long long>(i),
@@ -722,9 +758,9 @@ int tcpxuEngineStreamWarm(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t
   // Mapped block: `depth` completion words (one cache line each), then `depth` descriptor slots.
   const size_t flag_stride = 64;
   const size_t slot_bytes = sizeof(tcpxuLoadMeta) * TCPXU_SLOT_PAGES;
-  const size_t flags_bytes = flag_stride * TCPXU_QUEUE_DEPTH;
+  const size_t flags_bytes = flag_stride * TCPXU_STREAM_MAX_DEPTH;
   if (!e->stream_host)
-    TCPXU_TRY(tcpxuMappedAlloc(e->device, flags_bytes + slot_bytes * TCPXU_QUEUE_DEPTH, &e->stream_host,
+    TCPXU_TRY(tcpxuMappedAlloc(e->device, flags_bytes + slot_bytes * TCPXU_STREAM_MAX_DEPTH, &e->stream_host,
                                &e->stream_dev));
   uint8_t* hb = static_cast<uint8_t*>(e->stream_host);
   uint8_t* db = static_cast<uint8_t*>(e->stream_dev);
@@ -792,7 +828,7 @@ int tcpxuEngineRunTimed(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n
   if (!e || !kernel_us) return TCPXU_INVALID_ARGUMENT;
   // Touch the stream block before the launch so that no allocation happens while the kernel is timed.
   if (!e->stream_host) {
-    const size_t bytes = 64 * TCPXU_QUEUE_DEPTH + sizeof(tcpxuLoadMeta) * TCPXU_SLOT_PAGES * TCPXU_QUEUE_DEPTH;
+    const size_t bytes = (64 + sizeof(tcpxuLoadMeta) * TCPXU_SLOT_PAGES) * TCPXU_STREAM_MAX_DEPTH;
     TCPXU_TRY(tcpxuMappedAlloc(e->device, bytes, &e->stream_host, &e->stream_dev));
   }
   TCPXU_TRY(tcpxuEngineStart(e));

@@ -58,7 +58,7 @@ __global__ __launch_bounds__(kWgThreads) void unpack_batch_kernel(const uint8_t*
         *reinterpret_cast<u32x4*>(&staged[tid]) = raw;
       }
       __syncthreads();
-      wave_copy_descriptors<TCPXU_BATCH_TWO_ROUNDS>(staged, cnt, wave, kWavesPerWg, bounce, dst, lane);
+      wave_copy_descriptors<TCPXU_BATCH_TWO_ROUNDS>(staged, cnt, wave, kWavesPerWg, bounce, dst, lane, [] {});
       __syncthreads();
     }
   }

@@ -278,10 +278,12 @@ struct FragmentRounds {
 // wavefront; neighbours in the list decide which destination lines are shared.  The loads of the next round
 // are issued before the stores of the current one (kTwoRoundsInFlight); two register sets alternate so that no
 // register is copied while a load into it is in flight.  `bounce` and `dst` must be wave-uniform.
-template <bool kTwoRoundsInFlight>
+// `on_last_fragment()` is called exactly once, when the wavefront turns to the last descriptor of its share (at
+// once if it has none): a caller that feeds the wavefront can use it to start fetching more work.
+template <bool kTwoRoundsInFlight, typename OnLastFragment>
 __device__ __forceinline__ void wave_copy_descriptors(const tcpxuLoadMeta* descs, uint32_t n, uint32_t first,
                                                       uint32_t stride, const uint8_t* bounce, uint8_t* dst,
-                                                      uint32_t lane) {
+                                                      uint32_t lane, OnLastFragment&& on_last_fragment) {
   // Everything that describes a fragment is wave-uniform; saying so keeps it in scalar registers and leaves
   // the vector registers to the payload in flight.
   auto uniform = [](uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(v)); };
@@ -290,6 +292,7 @@ __device__ __forceinline__ void wave_copy_descriptors(const tcpxuLoadMeta* descs
   };
   const uint64_t dst_addr = reinterpret_cast<uint64_t>(dst);
   uint32_t j = uniform(first);
+  if (j >= n) on_last_fragment();
   FragmentRounds fr;
   // Next round of this wavefront's work, or false when there is none.  `prev` is the round before it.
   auto produce = [&](CopyRound& out, const CopyRound& prev) -> bool {
@@ -300,6 +303,7 @@ __device__ __forceinline__ void wave_copy_descriptors(const tcpxuLoadMeta* descs
     while (j < n) {
       const uint32_t cur = j;
       j += stride;
+      if (j >= n) on_last_fragment();
       const tcpxuLoadMeta d = descs[cur];
       const uint32_t len = uniform(d.len);
       if (len == 0) continue;
