@@ -30,8 +30,8 @@ import __graft_entry__ as graft
 
 # HBM bytes moved per algorithmic byte (2 x fragment bytes) by unpack_engine_kernel on the headline workload:
 # hardware counters FETCH_SIZE (x1.99974, its reading for a copy kernel of known size) and WRITE_SIZE (x1.0),
-# 8977134 KiB + 9148340 KiB against 2 x 9011200 KiB over one launch of 1100 steps.
-TRAFFIC_PER_ALGORITHMIC_BYTE = 1.0057
+# 8950944 KiB + 9120550 KiB against 2 x 9011200 KiB over one launch of 1100 steps.
+TRAFFIC_PER_ALGORITHMIC_BYTE = 1.0027
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 CHUNK_CONFIG = 2
 
@@ -66,6 +66,12 @@ def main():
     ap.add_argument("--depth", type=int, default=16, help="slots of one comm's mapped ring in flight (the unpack queue depth)")
     ap.add_argument("--cpu-seconds", type=float, default=8.0, help="time budget per CPU baseline leg")
     ap.add_argument("--skip-extras", action="store_true", help="only the headline measurement")
+    ap.add_argument(
+        "--one-launch",
+        action="store_true",
+        help="exactly one launch of the engine kernel in the process (no untimed launch before it, no single-comm run, "
+        "no extras): what a kernel trace or a counter run of the headline should see",
+    )
     ap.add_argument(
         "--calibrate-copy",
         type=int,
@@ -154,7 +160,8 @@ def main():
     # also what a kernel trace of this command shows for the launch.
     all_items = item_array(0, args.warmup + args.steps)
     # An untimed launch first: brings the clocks up from idle and touches every page once.
-    run(item_array(0, max(args.warmup, 1)), args.comms * args.depth)
+    if not args.one_launch:
+        run(item_array(0, max(args.warmup, 1)), args.comms * args.depth)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     wall_us, kernel_us, _ = run(all_items, args.comms * args.depth, warmup_items=args.warmup * slots_per_step)
@@ -219,7 +226,7 @@ def main():
         "timed_region_s": round(t1 - t0, 4),
     }
 
-    if args.comms > 1:
+    if args.comms > 1 and not args.one_launch:
         # The same steps with one comm only: 16 slots (at most 64 MiB) in flight, a launch of its own.
         w1, k1, _ = run(all_items, args.depth, warmup_items=args.warmup * slots_per_step)
         result["single_comm"] = {
@@ -231,7 +238,7 @@ def main():
             "launch_us": round(k1, 1),
         }
 
-    if not args.skip_extras:
+    if not args.skip_extras and not args.one_launch:
         # Request completion latency, one request in flight: publish -> host poller sees the completion word.
         storm = pkg.Workload(3, seed=0xC0FFEE03)
         sd = np.array(storm.descs, copy=True)
