@@ -1,7 +1,7 @@
 /*
  * tcpx_plugin.h -- C entry points of the plugin library (libnccl-net.so) of the MI355X receive-side unpack path.
  *
- * Three groups:
+ * Four groups:
  *   1. the ncclNet_v7 functions, under the names the reference gives them (src/net_tcpx.h:22-62), which the
  *      exported `ncclNetPlugin_v7` table points to (src/nccl_plugin.cc:22-42);
  *   2. the synthetic devmem socket: this build has no NIC and no sockets, so what the peer's control socket
@@ -10,7 +10,8 @@
  *   3. the device-operations table through which the plugin reaches the GPU.  By default it is bound to
  *      libtcpxu_hip.so (include/tcpx_unpack_hip.h) and initialisation fails if that cannot be loaded or no GPU
  *      is present.  A test may install another table BEFORE tcpxInit to exercise the host logic without a GPU;
- *      the plugin never picks a substitute by itself.
+ *      the plugin never picks a substitute by itself;
+ *   4. observability: slowness watches, counters and state-transition tracepoints (src/timeout.cc, src/stats/).
  */
 #ifndef TCPX_PLUGIN_H_
 #define TCPX_PLUGIN_H_
@@ -118,6 +119,63 @@ ncclResult_t tcpxSetDeviceOpsForTesting(const tcpxDeviceOps* ops);
  * src/net_tcpx.cc:1350-1353) return ncclInternalError instead, so a test can observe them in-process.
  * Default 1 = fail-stop like the reference. */
 ncclResult_t tcpxSetFailStopForTesting(int enabled);
+
+/* ---- 4. observability ------------------------------------------------------------------------------------ */
+/*
+ * Flags read by tcpxInit (names and ranges as in the reference, src/net_tcpx.cc:105-116,519-550, src/flags.cc:119-150):
+ *   NCCL_GPUDIRECTTCPX_TIMEOUT_THRESHOLD_NS   a watched wait is reported once it has lasted this long (10 s; >= 100 us)
+ *   NCCL_GPUDIRECTTCPX_TIMEOUT_FREQUENCY_NS   ... and again at this interval (30 s; >= 100 us)
+ *   NCCL_GPUDIRECTTCPX_SLOWNESS_SWITCH        which waits are watched: SENDRECV (recvmsg finds nothing), RX_CTRL (no
+ *                                             control message for the active request), UNPACK (the GPU holds a slot;
+ *                                             this build's own), TX_COMP (send side: accepted, never armed), ALL
+ *   NCCL_GPUDIRECTTCPX_SLOWNESS_REPORT        which of them also print a warning (default: all that are watched)
+ *   NCCL_GPUDIRECTTCPX_TELEMETRY_ENABLE_TASK_LEVEL_STATS / ..._REQUEST_LEVEL_STATS   record tracepoint events
+ *   NCCL_GPUDIRECTTCPX_TELEMETRY_SAMPLING_FACTOR   keep only objects whose address is a multiple of this
+ */
+
+/* Receive-side members of struct tcpxSocketStats (src/stats/monitoring.h:25-39), one per data flow. */
+typedef struct tcpxFlowStats {
+  uint64_t flow_id;
+  uint64_t rx_ctrl_done_cnt; /* control messages that named this flow */
+  uint64_t rx_cnt;           /* recvmsg calls, counted while task-level stats are on (src/stats/tracepoint.cc:72-82) */
+  uint64_t rx_slow_cnt;      /* slowness reports of recvmsg (src/stats/tracepoint.cc:22-52) */
+} tcpxFlowStats;
+
+typedef struct tcpxCommStats {
+  uint64_t rx_ctrl_slow_cnt; /* slowness reports while waiting for a control message (src/net_tcpx.cc:1234-1246) */
+  uint64_t unpack_cnt;       /* slots handed to the GPU */
+  uint64_t unpack_slow_cnt;  /* slowness reports while the GPU held a slot (no counterpart in the reference) */
+  uint64_t unpack_ns;        /* publish -> completion word seen by tcpxTest, summed over unpack_cnt slots */
+  uint64_t trace_dropped;    /* tracepoint events lost because nobody drained the buffer */
+} tcpxCommStats;
+
+ncclResult_t tcpxGetFlowStats(void* recvComm, uint32_t flow, tcpxFlowStats* stats);
+ncclResult_t tcpxGetCommStats(void* recvComm, tcpxCommStats* stats);
+
+/* One tracepoint: a request ('R') or task ('T') entered `state`, numbered as in the exported lines of the
+ * reference (src/stats/tracepoint.h:57-75): requests 0 FREE, 1 INACTIVE, 2 TRANSMITTING, 3 ACTIVE, 4 POSTED;
+ * tasks 0 FREE, 1 INACTIVE, 2 COMPLETING, 3 ACTIVE.  Fired where the reference fires TCPX_TP
+ * (src/work_queue.h:156-211). */
+typedef struct tcpxTraceEvent {
+  char kind;
+  uint8_t passive;
+  uint16_t state;
+  uint32_t reserved;
+  uint64_t object;   /* address of the request or task */
+  int64_t timestamp; /* nanoseconds: wall clock since the epoch, or the injected clock */
+} tcpxTraceEvent;
+
+/* Takes up to `max` events of the comm, oldest first, waiting up to `wait_ms` for the first
+ * (StatsBuffer::dequeue, src/stats/stats_buffer.h:74-93).  *n = 0 if tracing is off. */
+ncclResult_t tcpxTraceDrain(void* recvComm, tcpxTraceEvent* events, uint32_t max, uint32_t wait_ms, uint32_t* n);
+
+/* The line the reference's exporter writes for an event: "R 0x... <passive> <state> <timestamp>"
+ * (src/stats/stats_buffer.h:52-56).  Returns snprintf's result. */
+int tcpxTraceFormat(const tcpxTraceEvent* event, char* line, size_t len);
+
+/* Replaces the clock of the slowness watches and tracepoints (NULL restores CLOCK_MONOTONIC / the wall clock):
+ * the injectable `timenow` of struct tcpxTimeoutDetection::Config (src/timeout.h:26-30).  For tests. */
+ncclResult_t tcpxSetClockForTesting(uint64_t (*now_ns)(void));
 
 #ifdef __cplusplus
 }

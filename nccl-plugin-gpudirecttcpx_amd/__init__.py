@@ -258,6 +258,39 @@ class NetDeviceHandle(ctypes.Structure):
     ]
 
 
+class FlowStats(ctypes.Structure):
+    """tcpxFlowStats (include/tcpx_plugin.h)."""
+
+    _fields_ = [("flow_id", ctypes.c_uint64), ("rx_ctrl_done_cnt", ctypes.c_uint64), ("rx_cnt", ctypes.c_uint64), ("rx_slow_cnt", ctypes.c_uint64)]
+
+
+class CommStats(ctypes.Structure):
+    """tcpxCommStats (include/tcpx_plugin.h)."""
+
+    _fields_ = [
+        ("rx_ctrl_slow_cnt", ctypes.c_uint64),
+        ("unpack_cnt", ctypes.c_uint64),
+        ("unpack_slow_cnt", ctypes.c_uint64),
+        ("unpack_ns", ctypes.c_uint64),
+        ("trace_dropped", ctypes.c_uint64),
+    ]
+
+
+class TraceEvent(ctypes.Structure):
+    """tcpxTraceEvent (include/tcpx_plugin.h)."""
+
+    _fields_ = [
+        ("kind", ctypes.c_char),
+        ("passive", ctypes.c_uint8),
+        ("state", ctypes.c_uint16),
+        ("reserved", ctypes.c_uint32),
+        ("object", ctypes.c_uint64),
+        ("timestamp", ctypes.c_int64),
+    ]
+
+
+CLOCK_FN = ctypes.CFUNCTYPE(ctypes.c_uint64)
+
 _V = ctypes.c_void_p
 _VP = ctypes.POINTER(ctypes.c_void_p)
 _IP = ctypes.POINTER(ctypes.c_int)
@@ -306,6 +339,14 @@ _PLUGIN_PROTOTYPES = {
     "tcpxDebugSlot": (ctypes.c_int, [_V, ctypes.c_uint32, _VP, ctypes.POINTER(ctypes.c_uint64)]),
     "tcpxSetDeviceOpsForTesting": (ctypes.c_int, [_V]),
     "tcpxSetFailStopForTesting": (ctypes.c_int, [ctypes.c_int]),
+    "tcpxGetFlowStats": (ctypes.c_int, [_V, ctypes.c_uint32, ctypes.POINTER(FlowStats)]),
+    "tcpxGetCommStats": (ctypes.c_int, [_V, ctypes.POINTER(CommStats)]),
+    "tcpxTraceDrain": (
+        ctypes.c_int,
+        [_V, ctypes.POINTER(TraceEvent), ctypes.c_uint32, ctypes.c_uint32, ctypes.POINTER(ctypes.c_uint32)],
+    ),
+    "tcpxTraceFormat": (ctypes.c_int, [ctypes.POINTER(TraceEvent), ctypes.c_char_p, ctypes.c_size_t]),
+    "tcpxSetClockForTesting": (ctypes.c_int, [_V]),
 }
 
 NCCL_PTR_HOST, NCCL_PTR_CUDA = 1, 2

@@ -6,10 +6,13 @@
 // completion word, i.e. after the payload is in the receive buffer -- in the reference done=1 means "descriptor
 // count published" and NCCL's own kernel does the copy later.  Everything else (states, order checks, result
 // codes) follows src/net_tcpx.cc.
+#include <errno.h>
+#include <limits.h>
 #include <sched.h>
 
 #include <algorithm>
 #include <atomic>
+#include <chrono>
 #include <cstdarg>
 #include <cstdio>
 
@@ -61,6 +64,61 @@ void int_flag(int* flag, const char* name, long lo, long hi) {
   *flag = static_cast<int>(x);
 }
 
+void int64_flag(int64_t* flag, const char* name, long long lo) {  // [lo, LLONG_MAX)
+  char env[128];
+  snprintf(env, sizeof env, "NCCL_GPUDIRECTTCPX_%s", name);
+  const char* v = getenv(env);
+  if (!v || !*v) return;
+  char* end = nullptr;
+  const long long x = strtoll(v, &end, 0);
+  if (end == v || x < lo || x == LLONG_MAX) {
+    WARN("%s=%s ignored: not an integer in [%lld, LLONG_MAX)", env, v, lo);
+    return;
+  }
+  *flag = x;
+}
+
+// parseSlownessSwitchFlags, src/flags.cc:119-150: which waits are watched, and which of those are reported.
+void parse_slowness_flags() {
+  static const char kDefault[] = "TX_COMP,SENDRECV,RX_CTRL,UNPACK";
+  for (int i = 0; i < kSlowKinds; ++i) g.slow_switch[i] = g.slow_report[i] = 0;
+  const char* sw = getenv("NCCL_GPUDIRECTTCPX_SLOWNESS_SWITCH");
+  parse_slowness_switches(sw ? sw : kDefault, g.slow_switch);
+  const char* rp = getenv("NCCL_GPUDIRECTTCPX_SLOWNESS_REPORT");
+  parse_slowness_switches(rp ? rp : kDefault, g.slow_report);
+  for (int i = 0; i < kSlowKinds; ++i) {
+    if (!g.slow_switch[i] && g.slow_report[i]) {
+      INFO(NCCL_INIT, "%s slowness: detection is disabled, hence turning report off", kSlownessNames[i]);
+      g.slow_report[i] = 0;
+    }
+    INFO(NCCL_INIT, "%s slowness: detection %d report %d", kSlownessNames[i], g.slow_switch[i], g.slow_report[i]);
+  }
+}
+
+// Timestamp of a tracepoint: the wall clock like the reference's exporter lines, or the injected clock.
+int64_t trace_timestamp() {
+  if (g.clock_injected) return static_cast<int64_t>(g.clock());
+  return std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::system_clock::now().time_since_epoch()).count();
+}
+// tcpxTP_REQUEST / tcpxTP_TASK state tracepoints (src/stats/tracepoint.cc:84-103,178-232).
+void tp_request(Comm* comm, const Request* r, int state) {
+  if (g.request_stats && comm->trace) comm->trace->enqueue('R', r, comm->passive, state, trace_timestamp(), g.sampling_factor);
+}
+void tp_task(Comm* comm, const Task* t, int state) {
+  if (g.task_stats && comm->trace) comm->trace->enqueue('T', t, comm->passive, state, trace_timestamp(), g.sampling_factor);
+}
+// The ring transitions with their tracepoints, fired on the item that is about to move (src/work_queue.h:156-211).
+void request_advance(Comm* comm, int stage) {
+  static const int kEntered[kReqStages] = {kReqPostedTs, kReqTransmittingTs, kReqInactiveTs, kReqFreeTs};
+  tp_request(comm, comm->rq.first(stage), kEntered[stage]);
+  comm->rq.advance(stage);
+}
+void task_advance(Comm* comm, TaskRing* tasks, int stage) {
+  static const int kEntered[kTaskStages] = {kTaskCompletingTs, kTaskInactiveTs, kTaskFreeTs};
+  tp_task(comm, tasks->first(stage), kEntered[stage]);
+  tasks->advance(stage);
+}
+
 inline bool ctrl_done(const Request* r) { return r->next_flow >= 0; }  // CTRL_DONE, src/net_tcpx.cc:956
 // REQUEST_DONE, src/net_tcpx.cc:959-960
 inline bool request_done(const Request* r) {
@@ -79,15 +137,29 @@ ncclResult_t flow_progress(Comm* comm, int flow) {
       t->result = res;
       return res;
     }
+    // TCPX_TASK_TP_RECVMSG (src/net_tcpx.cc:167, src/stats/tracepoint.cc:72-82): a recvmsg that finds nothing
+    // yet is a possible slowness; the call itself is counted while task-level stats are on.
+    if (bytes < 0 && g.slow_switch[kSlowSendRecv] && (errno == EAGAIN || errno == EWOULDBLOCK || errno == EINTR || errno == ENOBUFS)) {
+      uint64_t nanos = 0;
+      if (t->watch.should_warn(g.clock, &nanos)) {
+        fd->rx_slow_cnt.fetch_add(1, std::memory_order_relaxed);
+        if (g.slow_report[kSlowSendRecv]) {
+          WARN("%p:%p, nic %d, %s, flow %d recv timeout error %d, %s: [%d/%d]/%d cnt %u, nanos %lu", static_cast<void*>(t),
+               static_cast<void*>(comm), comm->dev, g.dev_names[comm->dev], flow, errno, strerror(errno), t->offset, t->size,
+               t->r->size, t->watch.same_count, static_cast<unsigned long>(nanos));
+        }
+      }
+    }
+    if (g.task_stats) fd->rx_cnt.fetch_add(1, std::memory_order_relaxed);
     if (bytes > 0) {
       t->offset += static_cast<int>(bytes);
       fd->bytes += static_cast<uint64_t>(bytes);
     }
-    if (t->offset == t->size) tasks->advance(kTaskActive);  // ACTIVE -> COMPLETING
+    if (t->offset == t->size) task_advance(comm, tasks, kTaskActive);  // ACTIVE -> COMPLETING
   }
   if (tasks->has(kTaskCompleting)) {
     // The reference asks gpu_inline_test here, which always answers "done" (src/devcomm/nccl/inline.cu:55-60).
-    tasks->advance(kTaskCompleting);  // COMPLETING -> INACTIVE
+    task_advance(comm, tasks, kTaskCompleting);  // COMPLETING -> INACTIVE
   }
   return ncclSuccess;
 }
@@ -121,6 +193,7 @@ void enqueue_task(Comm* comm, Request* r) {
   t->request_offset = r->offset;
   t->size = sz;
   t->flow = flow;
+  t->watch.configure(static_cast<uint64_t>(g.timeout_threshold_ns), static_cast<uint64_t>(g.timeout_frequency_ns));
   t->pipe->cnt_cache = 0;
   t->pipe->bytes_cnt = 0;
   if (comm->passive) {
@@ -131,9 +204,10 @@ void enqueue_task(Comm* comm, Request* r) {
     // Unlike the reference, the count is not zeroed here: a request may put several chunks on the same flow, and
     // every chunk's pages must be given back when the request is consumed.  It is zeroed when the slot is taken.
   }
+  tp_task(comm, t, kTaskActiveTs);
   tasks->enqueue();  // FREE -> ACTIVE
   r->offset += sz;
-  if (r->size == r->offset) comm->rq.advance(kReqActive);  // REQUEST_INACTIVE -> finish_active
+  if (r->size == r->offset) request_advance(comm, kReqActive);  // REQUEST_INACTIVE -> finish_active
 }
 
 // tcpxCommProgress, src/net_tcpx.cc:1099-1308 (receive branch)
@@ -164,12 +238,12 @@ ncclResult_t comm_progress(Comm* comm) {
         u->cnt_cache += t->pipe->cnt_cache;
         t->pipe->cnt_cache = 0;
       }
-      tasks->advance(kTaskInactive);  // INACTIVE -> FREE
+      task_advance(comm, tasks, kTaskInactive);  // INACTIVE -> FREE
     }
     if (tasks->has_free()) any_flow_has_room = true;
   }
 
-  if (comm->rq.has(kReqPosted)) comm->rq.advance(kReqPosted);  // POSTED -> ACTIVE (src/net_tcpx.cc:1158-1180)
+  if (comm->rq.has(kReqPosted)) request_advance(comm, kReqPosted);  // POSTED -> ACTIVE (src/net_tcpx.cc:1158-1180)
 
   if (!comm->rq.has(kReqActive) || !any_flow_has_room) return ncclSuccess;
   Request* ar = comm->rq.first(kReqActive);
@@ -178,16 +252,34 @@ ncclResult_t comm_progress(Comm* comm) {
   do {  // src/net_tcpx.cc:1231-1304
     if (!ctrl_done(ar)) {
       CtrlMessage ctrl;
+      bool got_ctrl = false;
       {
         std::lock_guard<std::mutex> lock(comm->ctrl_mu);
-        if (comm->ctrl_rx.empty()) break;
-        ctrl = comm->ctrl_rx.front();
-        comm->ctrl_rx.pop_front();
+        if (!comm->ctrl_rx.empty()) {
+          ctrl = comm->ctrl_rx.front();
+          comm->ctrl_rx.pop_front();
+          got_ctrl = true;
+        }
       }
+      // Every look at the control socket counts towards its slowness watch; a message resets it
+      // (src/net_tcpx.cc:1234-1246).
+      if (g.slow_switch[kSlowRxCtrl]) {
+        uint64_t nanos = 0;
+        if (comm->ctrl_watch.should_warn(g.clock, &nanos)) {
+          comm->rx_ctrl_slow_cnt++;
+          if (g.slow_report[kSlowRxCtrl]) {
+            WARN("%p:%p, nic %d, %s, rx ctrl timeout cnt %u, nanos %lu", static_cast<void*>(ar), static_cast<void*>(comm),
+                 comm->dev, g.dev_names[comm->dev], comm->ctrl_watch.same_count, static_cast<unsigned long>(nanos));
+          }
+        }
+      }
+      if (!got_ctrl) break;
+      if (g.slow_switch[kSlowRxCtrl]) comm->ctrl_watch.reset();
       if (ctrl.type != TCPX_CTRL_INLINE && ctrl.index >= comm->num_flows) {
         WARN("control message names flow %u, comm has %d", ctrl.index, comm->num_flows);
         return ncclInternalError;
       }
+      if (ctrl.type != TCPX_CTRL_INLINE) comm->flows[ctrl.index].rx_ctrl_done_cnt.fetch_add(1, std::memory_order_relaxed);
       ar->next_flow = ctrl.index;  // tcpxCtrlRecv, src/net_tcpx.cc:995-1014
       ar->next_size = static_cast<int>(ctrl.size);
       if (ar->size_pending < 0) ar->size_pending = ar->size = static_cast<int>(ctrl.total);
@@ -209,7 +301,7 @@ ncclResult_t comm_progress(Comm* comm) {
           WARN("payload through the control socket is not supported for device memory");
           return ncclInternalError;
         }
-        comm->rq.advance(kReqActive);  // -> TRANSMITTING
+        request_advance(comm, kReqActive);  // -> TRANSMITTING
         break;
       }
     }
@@ -289,8 +381,21 @@ ncclResult_t tcpxInit(ncclDebugLogger_t logFunction) {
   std::lock_guard<std::mutex> lock(g.mu);
   g.logger = logFunction;
   if (g.initialized) return ncclSuccess;
+  // Flags start from their defaults at every initialisation (a process may finalise and initialise again).
+  g.flows_per_comm = 4;
+  g.use_helper_thread = 0;
+  g.timeout_threshold_ns = 10000000000LL;
+  g.timeout_frequency_ns = 30000000000LL;
+  g.task_stats = g.request_stats = 0;
+  g.sampling_factor = 1;
   int_flag(&g.flows_per_comm, "AMD_FLOWS", 1, kMaxFlows);
   int_flag(&g.use_helper_thread, "AMD_HELPER_THREAD", 0, 1);
+  int64_flag(&g.timeout_threshold_ns, "TIMEOUT_THRESHOLD_NS", 100 * 1000);  // src/net_tcpx.cc:519-524
+  int64_flag(&g.timeout_frequency_ns, "TIMEOUT_FREQUENCY_NS", 100 * 1000);
+  int_flag(&g.task_stats, "TELEMETRY_ENABLE_TASK_LEVEL_STATS", 0, 1);
+  int_flag(&g.request_stats, "TELEMETRY_ENABLE_REQUEST_LEVEL_STATS", 0, 1);
+  int_flag(&g.sampling_factor, "TELEMETRY_SAMPLING_FACTOR", 1, INT_MAX - 1);
+  parse_slowness_flags();
   if (!g.ops_injected) {
     g.ops = default_device_ops();
     if (!g.ops) {
@@ -413,6 +518,8 @@ static ncclResult_t new_comm(int dev, bool passive, Comm** out) {
   c->num_flows = g.flows_per_comm;
   c->use_helper = g.use_helper_thread != 0;
   for (int f = 0; f < kMaxFlows; ++f) c->flows[f].sock.device = c->device;
+  c->ctrl_watch.configure(static_cast<uint64_t>(g.timeout_threshold_ns), static_cast<uint64_t>(g.timeout_frequency_ns));
+  if (g.task_stats || g.request_stats) c->trace.reset(new TraceBuffer(kTraceEvents));
   *out = c;
   return ncclSuccess;
 }
@@ -516,6 +623,7 @@ static ncclResult_t get_request(Comm* comm, int op, void* data, int size, MemHan
   r->published = false;
   r->done_value = 0;
   *req = r;
+  tp_request(comm, r, kReqActiveTs);  // the reference names the enqueue tracepoint "active" (src/work_queue.h:189-192)
   comm->rq.enqueue();  // FREE -> POSTED
   return ncclSuccess;
 }
@@ -587,15 +695,33 @@ ncclResult_t tcpxTest(void* request, int* done, int* size) {
         }
         TCPXCHECK(device_result(rc, "engine_submit"));
         r->published = true;
+        r->published_ns = g.clock();
+        r->unpack_watch.configure(static_cast<uint64_t>(g.timeout_threshold_ns), static_cast<uint64_t>(g.timeout_frequency_ns));
+        comm->unpack_cnt++;
       }
       const uint64_t seen =
           reinterpret_cast<std::atomic<uint64_t>*>(&q->meta->done[r->slot.idx].value)->load(std::memory_order_acquire);
-      if (seen != r->done_value) return ncclSuccess;  // the GPU is still copying
+      if (seen != r->done_value) {  // the GPU is still copying
+        uint64_t nanos = 0;
+        if (g.slow_switch[kSlowUnpack] && r->unpack_watch.should_warn(g.clock, &nanos)) {
+          comm->unpack_slow_cnt++;
+          if (g.slow_report[kSlowUnpack]) {
+            WARN("%p:%p, gpu %d, unpack timeout: slot %lu (%lu descriptors, %d bytes) submitted, completion word %lu, expected %lu, "
+                 "queue head %lu tail %lu, cnt %u, nanos %lu",
+                 static_cast<void*>(r), static_cast<void*>(comm), comm->dev, static_cast<unsigned long>(r->slot.idx),
+                 static_cast<unsigned long>(r->slot.cnt_cache), r->size, static_cast<unsigned long>(seen),
+                 static_cast<unsigned long>(r->done_value), static_cast<unsigned long>(q->head),
+                 static_cast<unsigned long>(q->tail), r->unpack_watch.same_count, static_cast<unsigned long>(nanos));
+          }
+        }
+        return ncclSuccess;
+      }
+      comm->unpack_ns += g.clock() - r->published_ns;
     } else {
       *r->slot.cnt = 0;  // src/net_tcpx.cc:1361
     }
   }
-  comm->rq.advance(kReqTransmitting);  // -> INACTIVE
+  request_advance(comm, kReqTransmitting);  // -> INACTIVE
   *done = 1;
   return ncclSuccess;
 }
@@ -614,7 +740,7 @@ ncclResult_t tcpxIrecvConsumed(void* ocomm, int n, void* request) {
     return ncclSuccess;
   }
   if (!r->size) {  // skip empty (src/net_tcpx.cc:1500-1504)
-    comm->rq.advance(kReqInactive);
+    request_advance(comm, kReqInactive);
     q->head += 1;
     return ncclSuccess;
   }
@@ -642,7 +768,7 @@ ncclResult_t tcpxIrecvConsumed(void* ocomm, int n, void* request) {
     return ncclInternalError;
   }
   TCPXCHECK(recycle_pages(comm, q_idx));
-  comm->rq.advance(kReqInactive);  // INACTIVE -> FREE
+  request_advance(comm, kReqInactive);  // INACTIVE -> FREE
   q->head += 1;
   return ncclSuccess;
 }
@@ -740,6 +866,41 @@ ncclResult_t tcpxDebugSlot(void* recvComm, uint32_t slot_idx, const union loadMe
   if (!comm || !comm->queue || slot_idx >= static_cast<uint32_t>(kQueueDepth)) return ncclInvalidArgument;
   if (descs) *descs = comm->queue->meta->nccl.mem[slot_idx];
   if (cnt) *cnt = comm->queue->meta->nccl.cnt[slot_idx];
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxGetFlowStats(void* recvComm, uint32_t flow, tcpxFlowStats* stats) {
+  Comm* comm = static_cast<Comm*>(recvComm);
+  if (!comm || !stats || flow >= static_cast<uint32_t>(comm->num_flows)) return ncclInvalidArgument;
+  const FlowData* fd = &comm->flows[flow];
+  stats->flow_id = flow;
+  stats->rx_ctrl_done_cnt = fd->rx_ctrl_done_cnt.load(std::memory_order_relaxed);
+  stats->rx_cnt = fd->rx_cnt.load(std::memory_order_relaxed);
+  stats->rx_slow_cnt = fd->rx_slow_cnt.load(std::memory_order_relaxed);
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxGetCommStats(void* recvComm, tcpxCommStats* stats) {
+  Comm* comm = static_cast<Comm*>(recvComm);
+  if (!comm || !stats) return ncclInvalidArgument;
+  stats->rx_ctrl_slow_cnt = comm->rx_ctrl_slow_cnt;
+  stats->unpack_cnt = comm->unpack_cnt;
+  stats->unpack_slow_cnt = comm->unpack_slow_cnt;
+  stats->unpack_ns = comm->unpack_ns;
+  stats->trace_dropped = comm->trace ? comm->trace->dropped() : 0;
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxTraceDrain(void* recvComm, tcpxTraceEvent* events, uint32_t max, uint32_t wait_ms, uint32_t* n) {
+  Comm* comm = static_cast<Comm*>(recvComm);
+  if (!comm || !n || (max != 0 && !events)) return ncclInvalidArgument;
+  *n = comm->trace ? comm->trace->dequeue(events, max, wait_ms) : 0;
+  return ncclSuccess;
+}
+
+ncclResult_t tcpxSetClockForTesting(uint64_t (*now_ns)(void)) {
+  g.clock = now_ns ? now_ns : monotonic_ns;
+  g.clock_injected = now_ns != nullptr;
   return ncclSuccess;
 }
 

@@ -29,6 +29,7 @@
 #include <vector>
 
 #include "tcpx_plugin.h"
+#include "trace.h"
 
 namespace tcpx {
 
@@ -186,6 +187,7 @@ struct Comm;
 struct Request;
 
 struct Task {  // struct tcpxTask, src/work_queue.h:38-59 (receive-side fields)
+  SlownessWatch watch;  // recvmsg finding nothing, over and over (tcpxTask::timeout)
   int op = 0;
   int size = 0;
   int offset = 0;
@@ -217,6 +219,8 @@ struct Request {  // struct tcpxRequest, src/work_queue.h:63-76
   // Engine hand-off: the slot has been submitted, and the value its completion word will take.
   bool published = false;
   uint64_t done_value = 0;
+  uint64_t published_ns = 0;
+  SlownessWatch unpack_watch;  // the GPU holds the slot and the completion word does not come
 };
 
 enum RequestStage { kReqPosted = 0, kReqActive = 1, kReqTransmitting = 2, kReqInactive = 3, kReqStages = 4 };
@@ -240,6 +244,8 @@ struct FlowData {  // struct tcpxFdData, src/common.h:144-157 (receive-side fiel
   DevmemSocket sock;
   TaskRing tasks;
   uint64_t bytes = 0;
+  // struct tcpxSocketStats (receive side); the socket thread counts, the proxy thread reads.
+  std::atomic<uint64_t> rx_ctrl_done_cnt{0}, rx_cnt{0}, rx_slow_cnt{0};
 };
 
 struct Comm {  // struct tcpxComm, src/common.h:159-216
@@ -254,6 +260,9 @@ struct Comm {  // struct tcpxComm, src/common.h:159-216
   UnpackQueue* queue = nullptr;
   DeviceState* device = nullptr;
   uint64_t done_seq = 0;
+  SlownessWatch ctrl_watch;  // tcpxComm::ctrl_timeout
+  uint64_t rx_ctrl_slow_cnt = 0, unpack_cnt = 0, unpack_slow_cnt = 0, unpack_ns = 0;
+  std::unique_ptr<TraceBuffer> trace;  // tcpxComm::statsbuf; allocated when a stats level is on
   // Optional socket thread (persistentSocketThread, src/net_tcpx.cc:252-384).
   std::thread helper;
   std::atomic<bool> helper_stop{false};
@@ -298,6 +307,16 @@ struct Global {
   int flows_per_comm = 4;
   int use_helper_thread = 0;
   bool fail_stop = true;
+  // Observability (src/flags.cc:44-70, src/net_tcpx.cc:105-116).
+  ClockFn clock = monotonic_ns;
+  bool clock_injected = false;
+  int64_t timeout_threshold_ns = 10000000000LL;  // 10 s
+  int64_t timeout_frequency_ns = 30000000000LL;  // 30 s
+  int slow_switch[kSlowKinds] = {0, 0, 0, 0};
+  int slow_report[kSlowKinds] = {0, 0, 0, 0};
+  int task_stats = 0;
+  int request_stats = 0;
+  int sampling_factor = 1;
   char dev_names[kMaxDevices][32];
   char pci_paths[kMaxDevices][64];
 };

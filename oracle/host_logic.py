@@ -100,3 +100,67 @@ class RequestRing:
 def request_done(size, size_pending, ctrl_pending):
     """REQUEST_DONE (src/net_tcpx.cc:959-960)."""
     return (size == 0 and ctrl_pending) or (size != 0 and size_pending == 0)
+
+
+class SlownessWatch:
+    """struct tcpxTimeoutDetection (src/timeout.h:25-44).  Times are integers of one unit (nanoseconds)."""
+
+    def __init__(self, threshold_ns, frequency_ns):
+        self.threshold_ns = threshold_ns
+        self.frequency_ns = frequency_ns
+        self.reset()
+        self.first = 0
+        self.prev = 0
+
+    def reset(self):
+        """tcpxTimeoutDetectionReset (src/timeout.cc:44-47)."""
+        self.past_threshold = False
+        self.same_count = 0
+
+    def should_warn(self, now):
+        """tcpxTimeoutDetectionShouldWarn (src/timeout.cc:52-75): (warn, nanos since the first look).
+          :53-56  the first look after a reset notes the time and never warns
+          :60-65  until the threshold has been passed: warn once when now - first >= threshold
+          :66-71  afterwards: warn when now - previous warning >= frequency
+          :73     a warning moves the 'previous warning' time"""
+        self.same_count += 1
+        if self.same_count == 1:
+            self.first = now
+            return False, None
+        if not self.past_threshold:
+            nanos = now - self.first
+            if nanos < self.threshold_ns:
+                return False, None
+            self.past_threshold = True
+        else:
+            if now - self.prev < self.frequency_ns:
+                return False, None
+            nanos = now - self.first
+        self.prev = now
+        return True, nanos
+
+
+SLOWNESS_NAMES = ("TX_COMP", "SENDRECV", "RX_CTRL", "UNPACK")  # src/flags.cc:84-89, plus this build's UNPACK
+
+
+def parse_slowness_switches(text, switches):
+    """parseSlownessSwitchFlagInternal (src/flags.cc:91-117): comma-separated names, case-insensitive, ALL turns
+    every switch on, unknown names are ignored, nothing is ever turned off."""
+    if text is None:
+        return switches
+    for opt in text.split(","):
+        if not opt:
+            continue  # strtok skips empty fields
+        if opt.upper() == "ALL":
+            switches = [1] * len(switches)
+        for i, name in enumerate(SLOWNESS_NAMES):
+            if opt.upper() == name:
+                switches[i] = 1
+    return switches
+
+
+# Codes of the exported tracepoint lines (src/stats/tracepoint.h:57-75) and the transition that fires each
+# (src/work_queue.h:156-170, 189-211): the tracepoint names the state the item is entering, except that the
+# request's enqueue (FREE -> POSTED) is traced as ACTIVE and its finish_posted (POSTED -> ACTIVE) as POSTED.
+REQUEST_TRACE_SEQUENCE = (3, 4, 2, 1, 0)  # enqueue, finish_posted, finish_active, finish_transmitting, dequeue
+TASK_TRACE_SEQUENCE = (3, 2, 1, 0)  # enqueue, finish_active, finish_completing, dequeue

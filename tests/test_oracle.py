@@ -174,3 +174,46 @@ def test_request_ring_invariants():
         assert rq.invariant()
     assert host_logic.request_done(0, -1, True) and not host_logic.request_done(0, -1, False)
     assert host_logic.request_done(10, 0, False) and not host_logic.request_done(10, 4, True)
+
+
+def test_slowness_watch_hand_computed_and_invariants():
+    """struct tcpxTimeoutDetection (src/timeout.cc:44-75) against looks worked out on paper, then what must hold
+    for any sequence of looks: never on the first look, never before the threshold, reports at least
+    `frequency` apart, nanos = time since the first look."""
+    for case in VECTORS["slowness_watch"]:
+        w = host_logic.SlownessWatch(case["threshold"], case["frequency"])
+        for look in case["looks"]:
+            if look == "reset":
+                w.reset()
+                continue
+            now, warn, nanos = look
+            assert w.should_warn(now) == (warn, nanos), (case["ref"], look)
+    rng = np.random.default_rng(11)
+    for threshold, frequency in ((1000, 300), (50, 5000), (1, 1)):
+        w = host_logic.SlownessWatch(threshold, frequency)
+        now, first, last_report, reports = 0, None, None, 0
+        for i in range(3000):
+            now += int(rng.integers(0, 400))
+            if rng.random() < 0.01:
+                w.reset()
+                first, last_report = None, None
+                continue
+            warn, nanos = w.should_warn(now)
+            if first is None:
+                first = now
+                assert not warn
+                continue
+            if warn:
+                assert nanos == now - first and nanos >= threshold
+                assert last_report is None or now - last_report >= frequency
+                last_report = now
+                reports += 1
+            else:
+                assert now - first < threshold or (last_report is not None and now - last_report < frequency)
+        assert reports > 0
+
+
+def test_slowness_switches_hand_computed():
+    for case in VECTORS["slowness_switches"]:
+        assert host_logic.parse_slowness_switches(case["text"], list(case["before"])) == case["after"], case["ref"]
+    assert host_logic.parse_slowness_switches(None, [0, 1, 0, 0]) == [0, 1, 0, 0]
