@@ -59,6 +59,12 @@ def test_plugin_workloads_full_size(env, oracle, config):
     assert comm.outstanding_pages() == 0
     head, tail, _ = comm.queue_state()
     assert head == tail == info.n_requests
+    # Counters of the hand-off to the GPU: one slot per request, each timed, none slow (threshold 10 s).
+    stats = env.pkg.CommStats()
+    assert env.lib.tcpxGetCommStats(comm.comm, ctypes.byref(stats)) == 0
+    assert stats.unpack_cnt == info.n_requests and stats.unpack_slow_cnt == 0 and stats.rx_ctrl_slow_cnt == 0
+    assert 0 < stats.unpack_ns < 30e9
+    print("plugin case: mean publish->done %.1f us" % (stats.unpack_ns / stats.unpack_cnt / 1e3), flush=True)
     comm.close()
     assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
 
