@@ -253,3 +253,49 @@ def test_engine_argument_errors(pkg, hip):
     bad = pkg.EngineConfig(0, 0, 65, 0)
     assert hip.tcpxuEngineCreate(0, ctypes.byref(bad), ctypes.byref(h)) == pkg.INVALID_ARGUMENT
     e.destroy()
+
+
+@pytest.mark.parametrize("depth", [1, 5, 16, 64])
+def test_engine_stream_depths(pkg, hip, oracle, depth):
+    """The streaming driver (mapped slot ring, warm-up + timed items in one launch) at 1 to 64 slots in flight:
+    the leader then cuts tickets of 8 to 32 descriptors by backlog, and every size must give the oracle's bytes.
+    Eight distinct 8 MiB chunks, each twice, so every destination is written by two passes of the ring."""
+    import torch
+
+    chunks = [pkg.Workload(2, seed=0xBEEF00 + 31 * c) for c in range(8)]
+    info0 = chunks[0].info
+    cb = info0.payload_bytes
+    pool = np.empty(info0.pool_bytes, dtype=np.uint8)
+    chunks[0].fill_window(0, pool)  # one pool for all chunks: the oracle and the GPU read the same bytes
+    expect = np.full(GUARD + len(chunks) * cb + GUARD, SENTINEL, dtype=np.uint8)
+    keep, flat = [], []
+    for c, wl in enumerate(chunks):
+        assert wl.info.pool_bytes == info0.pool_bytes and wl.info.payload_bytes == cb
+        lo = GUARD + c * cb
+        expect[lo : lo + cb] = oracle_expected(oracle, pool, wl.descs, cb, 0)[GUARD : GUARD + cb]
+    pool_d = torch.from_numpy(pool).to("cuda:0")
+    dst_d = torch.full((expect.nbytes,), SENTINEL, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    for rep in range(2):
+        for c, wl in enumerate(chunks):
+            for r in wl.requests:
+                d = np.ascontiguousarray(wl.descs[int(r["first_desc"]) : int(r["first_desc"]) + int(r["n_descs"])])
+                keep.append(d)
+                flat.append((pool_d.data_ptr(), dst_d.data_ptr() + GUARD + c * cb, d.ctypes.data, len(d)))
+    items = (pkg.StreamItem * len(flat))()
+    for i, (b, d, p, n) in enumerate(flat):
+        items[i].bounce_base, items[i].dst_base, items[i].descs_host, items[i].n_descs = b, d, p, n
+    e = Engine(pkg, hip)
+    print("engine stream case: depth=%d items=%d" % (depth, len(flat)), flush=True)
+    wall, kern = ctypes.c_double(), ctypes.c_double()
+    lat = (ctypes.c_double * len(flat))()
+    rc = hip.tcpxuEngineRunTimed(e.h, items, len(flat), 4, depth, 20000, ctypes.byref(wall), ctypes.byref(kern), lat)
+    pkg.check(rc, "tcpxuEngineRunTimed")
+    assert e.completed() == len(flat) and 0 < wall.value <= kern.value * 1.5 and min(lat) > 0
+    e.destroy()
+    got = dst_d.cpu().numpy()
+    assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
+    # more than TCPXU_STREAM_MAX_DEPTH slots is refused before anything is launched
+    e = Engine(pkg, hip)
+    assert hip.tcpxuEngineRunTimed(e.h, items, 4, 0, 65, 1000, ctypes.byref(wall), ctypes.byref(kern), None) == pkg.INVALID_ARGUMENT
+    e.destroy()
