@@ -64,7 +64,8 @@ __global__ __launch_bounds__(kWgThreads) void unpack_batch_kernel(const uint8_t*
   }
 }
 
-// Plain copy, 64 bytes per thread per step: the yardstick for what a copy kernel reaches here.
+// Plain copy, 64 bytes per thread per step, with the payload accesses of the unpack kernels: the yardstick for
+// what a copy kernel reaches here.
 __global__ __launch_bounds__(kWgThreads) void copy_kernel(uint8_t* __restrict__ dst, const uint8_t* __restrict__ src,
                                                           uint64_t n_vec) {
   const uint64_t stride = static_cast<uint64_t>(gridDim.x) * kWgThreads;
@@ -79,7 +80,7 @@ __global__ __launch_bounds__(kWgThreads) void copy_kernel(uint8_t* __restrict__ 
 #pragma unroll
     for (int k = 0; k < kVecPerLane; ++k) {
       const uint64_t v = base + static_cast<uint64_t>(k) * kWgThreads + threadIdx.x;
-      if (v < n_vec) store_vec_sys(dst + (v << 4), r[k]);
+      if (v < n_vec) store_vec_stream(dst + (v << 4), r[k]);
     }
   }
 }
