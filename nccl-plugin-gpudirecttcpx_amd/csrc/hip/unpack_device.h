@@ -200,7 +200,17 @@ __device__ __forceinline__ void round_load(const CopyRound& c, CopyRegs& x, uint
   x.line_b = load_vec_sys(c.src_next + l.off_b);
 }
 
-__device__ __forceinline__ void round_store(const CopyRound& c, const CopyRegs& x, uint32_t lane) {
+__device__ __forceinline__ void round_store(const CopyRound& c, CopyRegs& x, uint32_t lane) {
+  // Wait for every load of the round before the first store, rather than store each vector as soon as its own
+  // load has landed (what the compiler would arrange): the round's stores then leave back to back, which
+  // measured 2-3 % faster end to end.  The registers pass through the statement so that no use of them can be
+  // scheduled before it.
+  asm volatile("s_waitcnt vmcnt(0)"
+               : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.r[2]), "+v"(x.r[3]), "+v"(x.line_a), "+v"(x.line_b),
+                 "+v"(x.tail_dword), "+v"(x.edge_byte)
+               :
+               : "memory");
+  static_assert(kVecPerLane == 4, "the statement above names the four vectors of a round");
   const LineLane l = line_lane(c, lane);
   const uint32_t skew = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(c.src_vec)) & 3u;
   const uint32_t last = c.nvec - 1;
