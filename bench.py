@@ -58,6 +58,45 @@ def cpu_baseline(oracle, wl, pool, threads, budget_s):
     return wl.info.payload_bytes / med / 1e9, iters
 
 
+def plugin_path(pkg, hip, torch, workloads, pool):
+    """The same chunks through the whole plugin (libnccl-net.so): irecv -> control messages -> synthetic recvmsg
+    with its control messages -> descriptor builder -> slot -> engine -> test() -> irecvConsumed, driven by the
+    request loop inside the library.  The host builds one descriptor per fragment here, so this is a host-bound
+    figure: what the receive path costs per fragment on one proxy thread."""
+    from nccl_plugin_gpudirecttcpx_amd import synth_driver
+
+    lib = pkg.plugin_lib()
+    if lib.tcpxInit(None) != 0:
+        return {"error": "tcpxInit failed"}
+    base = ctypes.c_void_p()
+    assert lib.tcpxSynthArenaCreate(0, pool.nbytes, ctypes.byref(base)) == 0
+    pkg.check(hip.tcpxuCopyToDevice(0, base, pool.ctypes.data, pool.nbytes), "tcpxuCopyToDevice")
+    comm = synth_driver.RecvComm(0)
+    chunk_bytes = int(workloads[0].info.payload_bytes)
+    dst = torch.empty(len(workloads) * chunk_bytes, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    seconds, frags, lat = 0.0, 0, []
+    for rep in range(3):  # the first pass warms up; the other two are timed
+        for c, wl in enumerate(workloads):
+            s, l = synth_driver.run_workload_native(comm, wl, dst.data_ptr() + c * chunk_bytes, window=8)
+            if rep > 0:
+                seconds += s
+                frags += int(wl.info.n_descs)
+                lat.extend(l)
+    stats = pkg.CommStats()
+    lib.tcpxGetCommStats(comm.comm, ctypes.byref(stats))
+    comm.close()
+    assert lib.tcpxFinalize() == 0
+    payload = 2 * len(workloads) * chunk_bytes
+    return {
+        "what": "8 MiB chunks through ncclNet_v7 (irecv/test/irecvConsumed) with the synthetic devmem socket, one proxy thread",
+        "payload_GBps": round(payload / seconds / 1e9, 2),
+        "host_ns_per_fragment": round(seconds / frags * 1e9, 1),
+        "request_fed_to_done_us_p50": round(percentile(lat, 50) * 1e6, 1),
+        "publish_to_done_us_mean": round(stats.unpack_ns / max(stats.unpack_cnt, 1) / 1e3, 2),
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -293,6 +332,9 @@ def main():
         del scratch
 
     pkg.check(hip.tcpxuEngineDestroy(engine), "tcpxuEngineDestroy")
+
+    if not args.skip_extras and not args.one_launch:
+        result["plugin_path"] = plugin_path(pkg, hip, torch, workloads[: min(8, args.chunks)], pool)
 
     # ---- CPU baseline on this machine's host cores: rank 0, bounded sample ---------------------------------
     threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16") or 16))

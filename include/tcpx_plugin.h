@@ -75,6 +75,17 @@ ncclResult_t tcpxSynthCtrlSend(void* recvComm, uint16_t type, uint16_t flow, uin
  * must already be in the arena. */
 ncclResult_t tcpxSynthDeliver(void* recvComm, uint32_t flow, const tcpxSynthFrag* frags, uint32_t n_frags);
 
+/* Plays NCCL's receive proxy, the peer and the NIC for `n_requests` requests without an interpreter in the loop:
+ * irecv at dst_base + request.dst_off, one control message per chunk (a run of consecutive fragments on one
+ * flow) and the chunk's fragments, test() until done, irecvConsumed; up to `window` (1..16) requests are kept
+ * posted.  `frags` is the whole workload's fragment array (requests index into it), the payload must already be
+ * in the arena and requests whose pages are reused must not be in one call.  Writes the wall time to *seconds
+ * and, if latency_s is not NULL, each request's fed-to-done time to latency_s[i].  ncclInternalError if a
+ * request does not complete within timeout_ms. */
+ncclResult_t tcpxSynthRunRequests(void* recvComm, const tcpxSynthFrag* frags, const tcpxSynthRequest* requests,
+                                  uint32_t n_requests, void* dst_base, uint64_t dst_bytes, uint32_t window,
+                                  uint32_t timeout_ms, double* seconds, double* latency_s);
+
 /* Limits how many fragments one synthetic recvmsg returns (default: as many as fit, at most 2048), to exercise
  * partial arrival; 0 restores the default. */
 ncclResult_t tcpxSynthSetRecvmsgLimit(void* recvComm, uint32_t max_frags_per_recvmsg);

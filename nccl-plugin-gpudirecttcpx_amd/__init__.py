@@ -331,6 +331,10 @@ _PLUGIN_PROTOTYPES = {
     ),
     "tcpxSynthDeliver": (ctypes.c_int, [_V, ctypes.c_uint32, _V, ctypes.c_uint32]),
     "tcpxSynthSetRecvmsgLimit": (ctypes.c_int, [_V, ctypes.c_uint32]),
+    "tcpxSynthRunRequests": (
+        ctypes.c_int,
+        [_V, _V, _V, ctypes.c_uint32, _V, ctypes.c_uint64, ctypes.c_uint32, ctypes.c_uint32, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)],
+    ),
     "tcpxSynthOutstandingPages": (ctypes.c_int, [_V, ctypes.POINTER(ctypes.c_uint64)]),
     "tcpxDebugQueueState": (
         ctypes.c_int,

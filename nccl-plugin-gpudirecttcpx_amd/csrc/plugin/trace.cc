@@ -83,7 +83,10 @@ void TraceBuffer::enqueue(char kind, const void* object, bool passive, int state
 uint32_t TraceBuffer::dequeue(tcpxTraceEvent* out, uint32_t max, uint32_t wait_ms) {
   std::unique_lock<std::mutex> lock(mu_);
   if (count_ == 0 && wait_ms != 0) {
-    not_empty_.wait_for(lock, std::chrono::milliseconds(wait_ms), [this] { return count_ != 0; });
+    // A deadline on the system clock makes this pthread_cond_timedwait, which thread-checking tools follow;
+    // a steady-clock wait becomes pthread_cond_clockwait, which some of them do not.
+    not_empty_.wait_until(lock, std::chrono::system_clock::now() + std::chrono::milliseconds(wait_ms),
+                          [this] { return count_ != 0; });
   }
   uint32_t n = 0;
   while (n < max && count_ != 0) {

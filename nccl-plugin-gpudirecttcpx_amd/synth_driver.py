@@ -170,3 +170,22 @@ def run_workload(comm, workload, dst_ptr, n_flows, window=8, timeout_s=60.0, aft
             raise TimeoutError("request %d did not complete" % idx)
     comm.dereg(mh)
     return latencies
+
+
+def run_workload_native(comm, workload, dst_ptr, window=8, timeout_ms=30000, first=0, count=None):
+    """The same as run_workload for requests [first, first + count), with the loop inside the plugin library
+    (tcpxSynthRunRequests): no interpreter between the calls.  Returns (wall seconds, per-request latencies)."""
+    import numpy as np
+
+    reqs = workload.requests
+    count = len(reqs) - first if count is None else count
+    seconds = ctypes.c_double()
+    lat = (ctypes.c_double * max(count, 1))()
+    frags = np.ascontiguousarray(workload.frags)
+    sub = np.ascontiguousarray(reqs[first : first + count])
+    rc = comm.lib.tcpxSynthRunRequests(
+        comm.comm, frags.ctypes.data, sub.ctypes.data, count, dst_ptr, int(workload.info.dst_bytes), window, timeout_ms,
+        ctypes.byref(seconds), lat,
+    )  # fmt: skip
+    ok(rc, "tcpxSynthRunRequests")
+    return seconds.value, list(lat[:count])

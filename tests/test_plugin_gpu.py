@@ -136,3 +136,25 @@ def test_hip_layer_is_what_init_bound(env):
     assert env.lib.tcpxDevices(ctypes.byref(n)) == 0
     env.pkg.check(env.hip.tcpxuDeviceCount(ctypes.byref(m)), "tcpxuDeviceCount")
     assert n.value == m.value >= 1
+
+
+def test_native_driver_full_size(env, oracle):
+    """The request loop inside the library (tcpxSynthRunRequests) on the 8 MiB chunk and the small-message storm."""
+    torch = env.torch
+    for config in (2, 3):
+        wl = env.pkg.Workload(config, seed=0xC0FFEE00 + config)
+        info = wl.info
+        pool = np.empty(info.pool_bytes, dtype=np.uint8)
+        wl.fill_window(0, pool)
+        upload(env, pool)
+        expect = np.full(GUARD + info.dst_bytes + GUARD, SENTINEL, dtype=np.uint8)
+        graft.oracle_unpack(oracle, expect[GUARD : GUARD + info.dst_bytes], pool, np.ascontiguousarray(wl.descs))
+        dst = torch.full((GUARD + info.dst_bytes + GUARD,), SENTINEL, dtype=torch.uint8, device="cuda:0")
+        torch.cuda.synchronize()
+        comm = env.driver.RecvComm(0)
+        print("native plugin case: config %d, %d requests" % (config, info.n_requests), flush=True)
+        seconds, lat = env.driver.run_workload_native(comm, wl, dst.data_ptr() + GUARD, window=8)
+        got = dst.cpu().numpy()
+        assert comm.outstanding_pages() == 0 and len(lat) == info.n_requests
+        comm.close()
+        assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)

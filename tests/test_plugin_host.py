@@ -119,6 +119,22 @@ def test_receive_workloads_byte_exact(env, comm, config, shrink):
     assert head == tail == len(wl.requests) and len(set(idx)) == 1 and idx[0] == len(wl.requests)
 
 
+@pytest.mark.parametrize("config,shrink", [(1, 0), (2, 2), (3, 4), (5, 3)])
+def test_native_driver_gives_the_same_bytes(env, comm, config, shrink):
+    """tcpxSynthRunRequests (the request loop inside the library) against the same expectation as the Python driver."""
+    wl = env.pkg.Workload(config, seed=0xAB00 + config, shrink=shrink)
+    pool = fill_arena(env, wl)
+    buf, ptr = host_buffer(int(wl.info.dst_bytes) + 64)
+    seconds, lat = env.driver.run_workload_native(comm, wl, ptr, window=8)
+    assert seconds > 0 and len(lat) == len(wl.requests) and min(lat) > 0
+    assert np.array_equal(buf, expected_bytes(pool, wl.frags, wl.requests, int(wl.info.dst_bytes) + 64))
+    assert comm.outstanding_pages() == 0
+    head, tail, idx = comm.queue_state()
+    assert head == tail == len(wl.requests)
+    assert env.lib.tcpxSynthRunRequests(comm.comm, None, None, 0, ptr, 64, 8, 1000, None, None) == INVALID_ARGUMENT
+    assert env.lib.tcpxSynthRunRequests(comm.comm, ptr, ptr, 0, ptr, 64, 17, 1000, None, None) == INVALID_ARGUMENT
+
+
 def test_partial_recvmsg_and_window_one(env, comm):
     """Fragments trickle in three per recvmsg; one request in flight at a time."""
     wl = env.pkg.Workload(2, seed=77, shrink=3)
