@@ -2,15 +2,15 @@
 // memory into scatter-gather copies and reports completion into mapped host memory -- no launch per request.
 //
 // Roles inside the one kernel launch
-//   workgroup 0, wavefront 0  "leader": polls the submission ring over PCIe (four entries per round trip), cuts
-//                             each submission into tickets of `descs_per_ticket` consecutive descriptors and
-//                             writes them into a device-memory ticket ring.  It never copies payload and never
-//                             waits for a store of its own.
-//   every other workgroup     "worker": claims the next ticket number with one atomic, polls that ticket's slot
-//                             until its stamps match, stages the ticket's descriptors from the mapped slot into
-//                             LDS, lets its four wavefronts copy fragments, then counts the ticket done.  Whoever
-//                             counts the last ticket of a submission writes the completion word that the host
-//                             poller reads.
+//   workgroup 0, wavefront 0  "leader": polls the submission ring over PCIe (sixteen entries per round trip),
+//                             cuts each submission into tickets of 8 to 32 consecutive descriptors (by backlog,
+//                             or of the fixed `descs_per_ticket`) and writes them into a device-memory ticket
+//                             ring.  It never copies payload.
+//   every other workgroup     "worker": one fetcher wavefront claims the next ticket number with one atomic,
+//                             polls that ticket's slot until its stamps match and stages the ticket's
+//                             descriptors from the mapped slot into LDS; the copy wavefronts copy the fragments,
+//                             and the last of them to finish counts the ticket done.  Whoever counts the last
+//                             ticket of a submission writes the completion word that the host poller reads.
 //
 // No cache maintenance.  Nothing here uses an acquire or release fence: on this GPU those become L2 write-back
 // and invalidate instructions, and thousands of pollers issuing them stall everybody.  Instead every access
@@ -42,10 +42,6 @@
 #include "tcpx_unpack_hip.h"
 #include "unpack_device.h"
 
-// One round in flight per wavefront: measured faster than two (half the registers, more wavefronts resident).
-#ifndef TCPXU_ENGINE_TWO_ROUNDS
-#define TCPXU_ENGINE_TWO_ROUNDS false
-#endif
 
 namespace tcpxu {
 namespace {
@@ -354,7 +350,7 @@ __device__ void copy_ticket(const Stage* stage, uint32_t wave, uint32_t lane, ui
   uint8_t* dst =
       reinterpret_cast<uint8_t*>((static_cast<uint64_t>(uniform(stage->payload[3])) << 32) | uniform(stage->payload[2]));
   const uint32_t n = uniform(stage->payload[10]) & 0xFFu;
-  wave_copy_descriptors<TCPXU_ENGINE_TWO_ROUNDS>(stage->desc, n, wave, kCopyWaves, bounce, dst, lane, [&] {
+  wave_copy_descriptors(stage->desc, n, wave, kCopyWaves, bounce, dst, lane, [&] {
     if (lane == 0) __hip_atomic_fetch_add(waves_on_last, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   });
 }

@@ -14,11 +14,6 @@
 #include "tcpx_unpack_hip.h"
 #include "unpack_device.h"
 
-// One round in flight per wavefront: measured faster than two (half the registers, more wavefronts resident).
-#ifndef TCPXU_BATCH_TWO_ROUNDS
-#define TCPXU_BATCH_TWO_ROUNDS false
-#endif
-
 namespace tcpxu {
 
 thread_local char g_last_error[512] = "";
@@ -58,7 +53,7 @@ __global__ __launch_bounds__(kWgThreads) void unpack_batch_kernel(const uint8_t*
         *reinterpret_cast<u32x4*>(&staged[tid]) = raw;
       }
       __syncthreads();
-      wave_copy_descriptors<TCPXU_BATCH_TWO_ROUNDS>(staged, cnt, wave, kWavesPerWg, bounce, dst, lane, [] {});
+      wave_copy_descriptors(staged, cnt, wave, kWavesPerWg, bounce, dst, lane, [] {});
       __syncthreads();
     }
   }

@@ -3,10 +3,9 @@
 // A fragment is `len` bytes (at most one 4 KiB bounce page in practice) with arbitrary byte alignment on both
 // sides.  The copy is organised around the DESTINATION: the body is written with aligned 16-byte vector stores
 // that cover whole 128-byte lines wherever a neighbouring fragment continues the line, and byte-wise heads and
-// tails remain only at the ends of a run of fragments.  Source vectors are fetched with 16-byte loads at
-// whatever alignment results (gfx950 global loads accept any alignment), so no realignment in registers is
-// needed except for the one vector that straddles two fragments.  This is a pure bandwidth copy: no MFMA, no
-// LDS for payload.
+// tails remain only at the ends of a run of fragments.  Source vectors are fetched with 16-byte loads at the
+// 4-byte aligned address just below where the destination alignment puts them and shifted into place in
+// registers.  This is a pure bandwidth copy: no MFMA, no LDS for payload.
 #ifndef TCPXU_UNPACK_DEVICE_H_
 #define TCPXU_UNPACK_DEVICE_H_
 
@@ -301,12 +300,13 @@ struct FragmentRounds {
 };
 
 // Copies descriptors first, first + stride, ... < n of a descriptor list staged in LDS with the calling
-// wavefront; neighbours in the list decide which destination lines are shared.  The loads of the next round
-// are issued before the stores of the current one (kTwoRoundsInFlight); two register sets alternate so that no
-// register is copied while a load into it is in flight.  `bounce` and `dst` must be wave-uniform.
+// wavefront; neighbours in the list decide which destination lines are shared.  One round (at most 4 KiB) is in
+// flight per wavefront: keeping a second register set to overlap the next round's loads with this round's
+// stores measured slower, because fewer wavefronts then fit on a compute unit.  `bounce` and `dst` must be
+// wave-uniform.
 // `on_last_fragment()` is called exactly once, when the wavefront turns to the last descriptor of its share (at
 // once if it has none): a caller that feeds the wavefront can use it to start fetching more work.
-template <bool kTwoRoundsInFlight, typename OnLastFragment>
+template <typename OnLastFragment>
 __device__ __forceinline__ void wave_copy_descriptors(const tcpxuLoadMeta* descs, uint32_t n, uint32_t first,
                                                       uint32_t stride, const uint8_t* bounce, uint8_t* dst,
                                                       uint32_t lane, OnLastFragment&& on_last_fragment) {
@@ -357,36 +357,15 @@ __device__ __forceinline__ void wave_copy_descriptors(const tcpxuLoadMeta* descs
     }
     return false;
   };
-  if constexpr (!kTwoRoundsInFlight) {
-    // One register set: more wavefronts fit on a compute unit, each with one round in flight.
-    CopyRound r;
-    CopyRegs x;
-    if (!produce(r, r)) return;
-    for (;;) {
-      round_load(r, x, lane);
-      round_store(r, x, lane);
-      CopyRound nxt;
-      if (!produce(nxt, r)) return;
-      r = nxt;
-    }
-  }
-  CopyRound ra, rb;
-  CopyRegs xa, xb;
-  if (!produce(ra, ra)) return;
-  round_load(ra, xa, lane);
+  CopyRound r;
+  CopyRegs x;
+  if (!produce(r, r)) return;
   for (;;) {
-    if (!produce(rb, ra)) {
-      round_store(ra, xa, lane);
-      break;
-    }
-    round_load(rb, xb, lane);
-    round_store(ra, xa, lane);
-    if (!produce(ra, rb)) {
-      round_store(rb, xb, lane);
-      break;
-    }
-    round_load(ra, xa, lane);
-    round_store(rb, xb, lane);
+    round_load(r, x, lane);
+    round_store(r, x, lane);
+    CopyRound nxt;
+    if (!produce(nxt, r)) return;
+    r = nxt;
   }
 }
 
