@@ -29,33 +29,44 @@ namespace {
 
 constexpr uint32_t kMaxDescsPerWg = 64;
 
-// Launch-per-batch unpack.  A workgroup takes `descs_per_wg` consecutive descriptors, stages them in LDS with
-// one 16-byte load per thread, then its four wavefronts take fragments in turn.
+// Launch-per-batch unpack.  A workgroup takes `descs_per_wg` consecutive descriptors at a time, stages them in
+// LDS with one 16-byte load per thread, then its four wavefronts take fragments in turn.  The descriptors of the
+// workgroup's next batch are fetched into registers before the current batch is copied and go into the other of
+// two LDS stages, so that a batch costs one barrier and no exposed descriptor fetch.
 __global__ __launch_bounds__(kWgThreads) void unpack_batch_kernel(const uint8_t* __restrict__ bounce,
                                                                    uint8_t* __restrict__ dst,
                                                                    const tcpxuLoadMeta* __restrict__ descs,
                                                                    uint64_t n_descs, uint32_t descs_per_wg,
                                                                    uint64_t n_batches) {
-  __shared__ tcpxuLoadMeta staged[kMaxDescsPerWg];
+  __shared__ tcpxuLoadMeta staged[2][kMaxDescsPerWg];
   const uint32_t tid = threadIdx.x;
   const uint32_t lane = tid & (kWaveLanes - 1);
   const uint32_t wave = tid / kWaveLanes;
+  const uint64_t n_slots = (n_batches + 7) / 8 * 8;  // work-item indices, some of which name no batch
 
-  for (uint64_t wg = blockIdx.x;; wg += gridDim.x) {
-    const uint64_t per_xcd = (n_batches + 7) / 8;
-    if (wg >= per_xcd * 8) break;
+  // Batch number and descriptor count of work item `wg` (count 0: none), and this thread's descriptor of it.
+  auto batch_of = [&](uint64_t wg, uint64_t* first) -> uint32_t {
+    if (wg >= n_slots) return 0;
     const uint64_t batch = xcd_contiguous_index(wg, n_batches);
-    if (batch < n_batches) {  // block-uniform
-      const uint64_t first = batch * descs_per_wg;
-      const uint32_t cnt = static_cast<uint32_t>(std::min<uint64_t>(descs_per_wg, n_descs - first));
-      if (tid < cnt) {
-        const u32x4 raw = *reinterpret_cast<const u32x4*>(descs + first + tid);
-        *reinterpret_cast<u32x4*>(&staged[tid]) = raw;
-      }
-      __syncthreads();
-      wave_copy_descriptors(staged, cnt, wave, kWavesPerWg, bounce, dst, lane, [] {});
-      __syncthreads();
-    }
+    if (batch >= n_batches) return 0;
+    *first = batch * descs_per_wg;
+    return static_cast<uint32_t>(std::min<uint64_t>(descs_per_wg, n_descs - *first));
+  };
+  auto fetch = [&](uint64_t first, uint32_t cnt) -> u32x4 {
+    return tid < cnt ? *reinterpret_cast<const u32x4*>(descs + first + tid) : u32x4{0, 0, 0, 0};
+  };
+
+  uint64_t wg = blockIdx.x, first = 0;
+  uint32_t cnt = batch_of(wg, &first);
+  u32x4 raw = fetch(first, cnt);
+  for (uint32_t stage = 0; wg < n_slots; stage ^= 1u) {
+    if (tid < cnt) *reinterpret_cast<u32x4*>(&staged[stage][tid]) = raw;
+    const uint32_t cnt_now = cnt;
+    wg += gridDim.x;
+    cnt = batch_of(wg, &first);
+    raw = fetch(first, cnt);  // in flight while this batch is copied
+    __syncthreads();          // the stage is complete; every wavefront has left the stage written two batches ago
+    wave_copy_descriptors(staged[stage], cnt_now, wave, kWavesPerWg, bounce, dst, lane, [] {});
   }
 }
 
