@@ -1,0 +1,32 @@
+"""bench.py prints exactly one JSON line with the fields its consumers rely on (short run, GPU)."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_bench_prints_one_json_line_with_the_contract_fields():
+    p = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bench.py"), "--steps", "200", "--warmup", "20", "--skip-extras", "--cpu-seconds", "0.2", "--chunks", "8", "--pools", "2"],
+        stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300, cwd=ROOT,
+    )  # fmt: skip
+    assert p.returncode == 0, p.stderr[-2000:]
+    lines = [l for l in p.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1, p.stdout
+    r = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling", "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
+        assert key in r, key
+    assert r["n_gpus"] == 1 and r["steps"] == 200 and r["warmup"] == 20 and r["unit"] == "GB/s" and r["dtype"] == "u8"
+    assert r["vs_baseline"] is None and r["higher_is_better"] is True and r["data"] == "synthetic" and "workload" in r["config"]
+    roof = r["roofline"]
+    assert roof["bound"] == "hbm" and roof["peak"] == 8000.0 and roof["unit"] == "GB/s"
+    assert abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-3 and roof["traffic"] >= roof["bytes_per_launch"]
+    assert abs(r["value"] * 1e9 * r["ms_per_step"] * 1e-3 * r["steps"] - roof["bytes_per_launch"] / 2 * 200 / 220) / (roof["bytes_per_launch"] / 2) < 0.02
+    cpu = r["cpu_baseline"]
+    assert cpu["kind"] == "port" and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["unit"] == "GB/s" and cpu["sample"]
+    assert r["parity_ok"] is True
