@@ -299,3 +299,61 @@ def test_engine_stream_depths(pkg, hip, oracle, depth):
     e = Engine(pkg, hip)
     assert hip.tcpxuEngineRunTimed(e.h, items, 4, 0, 65, 1000, ctypes.byref(wall), ctypes.byref(kern), None) == pkg.INVALID_ARGUMENT
     e.destroy()
+
+
+def test_engine_bursts_around_the_idle_exit(pkg, hip, oracle):
+    """Three host threads submit in bursts separated by pauses of about the engine's idle limit (set to some
+    60 us here), so that submissions keep meeting a kernel that is leaving, has left, or is coming back.  Every
+    request must complete and every byte must match; seeded, a few hundred relaunches in a couple of seconds."""
+    import threading
+
+    wl = pkg.Workload(3, seed=0x51DE, shrink=3)  # 256 requests of 16 x 4 KiB
+    info = wl.info
+    pool = np.empty(info.pool_bytes, dtype=np.uint8)
+    wl.fill_window(0, pool)
+    expect = oracle_expected(oracle, pool, wl.descs, info.dst_bytes, info.dst_misalign)
+    g = GpuBuffers(pool, wl.descs, info.dst_bytes, info.dst_misalign)
+    n = len(wl.requests)
+    m = Mapped(pkg, hip, np.ascontiguousarray(wl.descs), n)
+    e = Engine(pkg, hip, spin_limit=40)
+    e.start()
+    errors = []
+
+    def worker(k):
+        rng = np.random.default_rng(100 + k)
+        try:
+            mine = list(range(k, n, 3))
+            i = 0
+            while i < len(mine):
+                burst = int(rng.integers(1, 5))
+                batch = mine[i : i + burst]
+                for r in batch:
+                    req = wl.requests[r]
+                    e.submit(g.pool.data_ptr(), g.dst_base, m.desc_dev(int(req["first_desc"])), int(req["n_descs"]), m.flag_dev(r), r + 1)
+                for r in batch:
+                    m.wait(r, r + 1, seconds=30.0)
+                i += burst
+                time.sleep(float(rng.uniform(0, 150e-6)))
+        except Exception as exc:  # reported by the main thread
+            errors.append(repr(exc))
+
+    threads = [threading.Thread(target=worker, args=(k,)) for k in range(3)]
+    print("engine burst case: %d requests, 3 threads" % n, flush=True)
+    for t in threads:
+        t.start()
+    away = 0  # times the main thread found the kernel gone while the others were submitting
+    deadline = time.time() + 120
+    while any(t.is_alive() for t in threads) and time.time() < deadline:
+        away += 0 if e.running() else 1
+        time.sleep(50e-6)
+    for t in threads:
+        t.join(timeout=5)
+    assert not any(t.is_alive() for t in threads) and not errors, errors
+    print("engine burst case: kernel found away %d times" % away, flush=True)
+    assert away >= 3, "the pauses were meant to let the kernel leave now and then"
+    got = g.result()
+    e.stop()
+    assert e.completed() == n
+    e.destroy()
+    m.free()
+    assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
