@@ -50,7 +50,7 @@ def cpu_baseline(oracle, wl, pool, threads, budget_s):
     rc = oracle.tcpx_oracle_unpack_timed(dst.ctypes.data, pool.ctypes.data, descs.ctypes.data, len(descs), threads, 2, 3, probe)
     assert rc == 0
     per_iter = max(min(probe), 1e-6)
-    iters = int(max(20, min(2000, budget_s / per_iter)))
+    iters = int(max(20, min(400000, budget_s / per_iter)))
     secs = (ctypes.c_double * iters)()
     rc = oracle.tcpx_oracle_unpack_timed(dst.ctypes.data, pool.ctypes.data, descs.ctypes.data, len(descs), threads, 5, iters, secs)
     assert rc == 0
@@ -106,7 +106,7 @@ def main():
     ap.add_argument("--pools", type=int, default=16, help="copies of the 256 MiB bounce pool the chunks take turns reading from")
     ap.add_argument("--comms", type=int, default=4, help="receive comms kept busy on the one engine (1..4)")
     ap.add_argument("--depth", type=int, default=16, help="slots of one comm's mapped ring in flight (the unpack queue depth)")
-    ap.add_argument("--cpu-seconds", type=float, default=8.0, help="time budget per CPU baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=6.0, help="CPU time per baseline leg (16 threads, then 1 thread)")
     ap.add_argument("--skip-extras", action="store_true", help="only the headline measurement")
     ap.add_argument(
         "--one-launch",
