@@ -1,7 +1,7 @@
 /*
  * tcpx_plugin.h -- C entry points of the plugin library (libnccl-net.so) of the MI355X receive-side unpack path.
  *
- * Four groups:
+ * Five groups:
  *   1. the ncclNet_v7 functions, under the names the reference gives them (src/net_tcpx.h:22-62), which the
  *      exported `ncclNetPlugin_v7` table points to (src/nccl_plugin.cc:22-42);
  *   2. the synthetic devmem socket: this build has no NIC and no sockets, so what the peer's control socket
@@ -11,7 +11,8 @@
  *      libtcpxu_hip.so (include/tcpx_unpack_hip.h) and initialisation fails if that cannot be loaded or no GPU
  *      is present.  A test may install another table BEFORE tcpxInit to exercise the host logic without a GPU;
  *      the plugin never picks a substitute by itself;
- *   4. observability: slowness watches, counters and state-transition tracepoints (src/timeout.cc, src/stats/).
+ *   4. observability: slowness watches, counters and state-transition tracepoints (src/timeout.cc, src/stats/);
+ *   5. the flow scheduler (src/flow_mapper.h) on its own.
  */
 #ifndef TCPX_PLUGIN_H_
 #define TCPX_PLUGIN_H_
@@ -187,6 +188,23 @@ int tcpxTraceFormat(const tcpxTraceEvent* event, char* line, size_t len);
 /* Replaces the clock of the slowness watches and tracepoints (NULL restores CLOCK_MONOTONIC / the wall clock):
  * the injectable `timenow` of struct tcpxTimeoutDetection::Config (src/timeout.h:26-30).  For tests. */
 ncclResult_t tcpxSetClockForTesting(uint64_t (*now_ns)(void));
+
+/* ---- 5. The flow scheduler -------------------------------------------------------------------------------------
+ * Which flows may take the next chunk of a message: class FlowMapper (src/flow_mapper.h:52-65) with its two
+ * policies, FlowMapperRR (:137-157; alg 0) and FlowMapperKaty (:67-135; alg 1), selected per process by
+ * NCCL_GPUDIRECTTCPX_SCHED_ALG = "RR" | "KATY" (src/net_tcpx.cc:643-665; anything else means RR).  A receive comm
+ * refills its scheduler at every poll with the flows whose task ring has room and takes control messages only
+ * while it holds one (src/net_tcpx.cc:1114,1152-1155,1183); Pick is what the sending peer calls per chunk
+ * (src/net_tcpx.cc:1216).  These entry points drive one scheduler on its own, for tests and for a synthetic peer.
+ * `alg` NULL = the policy the last tcpxInit selected.  Flows are 0..7, priorities 0..5 (task slots in use). */
+typedef struct tcpxFlowSched tcpxFlowSched;
+ncclResult_t tcpxFlowSchedCreate(const char* alg, tcpxFlowSched** sched);
+int tcpxFlowSchedAlg(const tcpxFlowSched* sched);               /* 0 RR, 1 KATY */
+void tcpxFlowSchedReset(tcpxFlowSched* sched);                  /* FlowMapper::reset */
+int tcpxFlowSchedHasFlow(const tcpxFlowSched* sched);           /* FlowMapper::hasFlow */
+void tcpxFlowSchedSchedule(tcpxFlowSched* sched, int flow, int prio); /* FlowMapper::scheduleFlow */
+int tcpxFlowSchedPick(tcpxFlowSched* sched);                    /* FlowMapper::pickFlow: a flow, or -1 */
+void tcpxFlowSchedDestroy(tcpxFlowSched* sched);
 
 #ifdef __cplusplus
 }

@@ -351,6 +351,13 @@ _PLUGIN_PROTOTYPES = {
     ),
     "tcpxTraceFormat": (ctypes.c_int, [ctypes.POINTER(TraceEvent), ctypes.c_char_p, ctypes.c_size_t]),
     "tcpxSetClockForTesting": (ctypes.c_int, [_V]),
+    "tcpxFlowSchedCreate": (ctypes.c_int, [ctypes.c_char_p, ctypes.POINTER(_V)]),
+    "tcpxFlowSchedAlg": (ctypes.c_int, [_V]),
+    "tcpxFlowSchedReset": (None, [_V]),
+    "tcpxFlowSchedHasFlow": (ctypes.c_int, [_V]),
+    "tcpxFlowSchedSchedule": (None, [_V, ctypes.c_int, ctypes.c_int]),
+    "tcpxFlowSchedPick": (ctypes.c_int, [_V]),
+    "tcpxFlowSchedDestroy": (None, [_V]),
 }
 
 NCCL_PTR_HOST, NCCL_PTR_CUDA = 1, 2

@@ -95,6 +95,23 @@ void parse_slowness_flags() {
   }
 }
 
+// NCCL_GPUDIRECTTCPX_SCHED_ALG, src/net_tcpx.cc:643-665: "RR" when unset, and also (with a note) when not a known name.
+void parse_sched_alg() {
+  const char* v = getenv("NCCL_GPUDIRECTTCPX_SCHED_ALG");
+  if (!v) {
+    g.sched_alg = kSchedRoundRobin;
+    INFO(NCCL_INIT, "NCCL_GPUDIRECTTCPX_SCHED_ALG unset. Using RR by default");
+    return;
+  }
+  bool valid = false;
+  g.sched_alg = sched_alg_from_name(v, &valid);
+  if (valid) {
+    INFO(NCCL_INIT, "NCCL_GPUDIRECTTCPX_SCHED_ALG %s", v);
+  } else {
+    INFO(NCCL_INIT, "invalid NCCL_GPUDIRECTTCPX_SCHED_ALG %s. Using RR by default", v);
+  }
+}
+
 // Timestamp of a tracepoint: the wall clock like the reference's exporter lines, or the injected clock.
 int64_t trace_timestamp() {
   if (g.clock_injected) return static_cast<int64_t>(g.clock());
@@ -219,7 +236,7 @@ ncclResult_t comm_progress(Comm* comm) {
   }
 
   // Reap finished tasks: their descriptors move into the request's slot (src/net_tcpx.cc:1119-1151).
-  bool any_flow_has_room = false;
+  comm->sched->reset();  // src/net_tcpx.cc:1114
   for (int i = 0; i < comm->num_flows; ++i) {
     int idx = comm->end_flow_idx - i;
     if (idx < 0) idx += comm->num_flows;
@@ -240,12 +257,13 @@ ncclResult_t comm_progress(Comm* comm) {
       }
       task_advance(comm, tasks, kTaskInactive);  // INACTIVE -> FREE
     }
-    if (tasks->has_free()) any_flow_has_room = true;
+    // Priority = task slots in use: the emptiest flow is served first (src/net_tcpx.cc:1152-1155).
+    if (tasks->has_free()) comm->sched->schedule(idx, kMaxTasks - static_cast<int>(tasks->num_free()));
   }
 
   if (comm->rq.has(kReqPosted)) request_advance(comm, kReqPosted);  // POSTED -> ACTIVE (src/net_tcpx.cc:1158-1180)
 
-  if (!comm->rq.has(kReqActive) || !any_flow_has_room) return ncclSuccess;
+  if (!comm->rq.has(kReqActive) || !comm->sched->has_flow()) return ncclSuccess;
   Request* ar = comm->rq.first(kReqActive);
   if (ar->op != kOpRecv) return ncclSuccess;
 
@@ -358,6 +376,17 @@ ncclResult_t ensure_engine(DeviceState* ds) {
 }
 
 }  // namespace
+
+int sched_alg_from_name(const char* name, bool* valid) {
+  const bool rr = name && strcmp(name, "RR") == 0, katy = name && strcmp(name, "KATY") == 0;
+  if (valid) *valid = rr || katy;
+  return katy ? kSchedKaty : kSchedRoundRobin;
+}
+
+FlowScheduler* new_flow_scheduler(int alg) {
+  if (alg == kSchedKaty) return new KatyFlows(kMaxFlows, kMaxTasks);
+  return new RoundRobinFlows;
+}
 }  // namespace tcpx
 
 using namespace tcpx;
@@ -396,6 +425,7 @@ ncclResult_t tcpxInit(ncclDebugLogger_t logFunction) {
   int_flag(&g.request_stats, "TELEMETRY_ENABLE_REQUEST_LEVEL_STATS", 0, 1);
   int_flag(&g.sampling_factor, "TELEMETRY_SAMPLING_FACTOR", 1, INT_MAX - 1);
   parse_slowness_flags();
+  parse_sched_alg();
   if (!g.ops_injected) {
     g.ops = default_device_ops();
     if (!g.ops) {
@@ -517,6 +547,7 @@ static ncclResult_t new_comm(int dev, bool passive, Comm** out) {
   c->device = &g.devices[dev];
   c->num_flows = g.flows_per_comm;
   c->use_helper = g.use_helper_thread != 0;
+  c->sched.reset(new_flow_scheduler(g.sched_alg));  // src/net_tcpx.cc:1101-1112 (there: at the first progress call)
   for (int f = 0; f < kMaxFlows; ++f) c->flows[f].sock.device = c->device;
   c->ctrl_watch.configure(static_cast<uint64_t>(g.timeout_threshold_ns), static_cast<uint64_t>(g.timeout_frequency_ns));
   if (g.task_stats || g.request_stats) c->trace.reset(new TraceBuffer(kTraceEvents));
@@ -903,5 +934,33 @@ ncclResult_t tcpxSetClockForTesting(uint64_t (*now_ns)(void)) {
   g.clock_injected = now_ns != nullptr;
   return ncclSuccess;
 }
+
+// ---- the flow scheduler on its own ---------------------------------------------------------------------------------
+struct tcpxFlowSched {
+  std::unique_ptr<FlowScheduler> impl;
+  int alg;
+};
+
+ncclResult_t tcpxFlowSchedCreate(const char* alg, tcpxFlowSched** sched) {
+  if (!sched) return ncclInvalidArgument;
+  tcpxFlowSched* s = new (std::nothrow) tcpxFlowSched;
+  if (!s) return ncclSystemError;
+  // NULL: the policy of the current initialisation; a name: parsed like the flag.
+  s->alg = alg ? sched_alg_from_name(alg, nullptr) : g.sched_alg;
+  s->impl.reset(new_flow_scheduler(s->alg));
+  s->impl->reset();
+  *sched = s;
+  return ncclSuccess;
+}
+int tcpxFlowSchedAlg(const tcpxFlowSched* sched) { return sched ? sched->alg : -1; }
+void tcpxFlowSchedReset(tcpxFlowSched* sched) {
+  if (sched) sched->impl->reset();
+}
+int tcpxFlowSchedHasFlow(const tcpxFlowSched* sched) { return sched && sched->impl->has_flow() ? 1 : 0; }
+void tcpxFlowSchedSchedule(tcpxFlowSched* sched, int flow, int prio) {
+  if (sched) sched->impl->schedule(flow, prio);
+}
+int tcpxFlowSchedPick(tcpxFlowSched* sched) { return sched ? sched->impl->pick() : -1; }
+void tcpxFlowSchedDestroy(tcpxFlowSched* sched) { delete sched; }
 
 }  // extern "C"

@@ -29,6 +29,7 @@
 #include <vector>
 
 #include "tcpx_plugin.h"
+#include "flow_mapper.h"
 #include "trace.h"
 
 namespace tcpx {
@@ -254,6 +255,7 @@ struct Comm {  // struct tcpxComm, src/common.h:159-216
   int num_flows = 0;
   int end_flow_idx = 0;
   FlowData flows[kMaxFlows];
+  std::unique_ptr<FlowScheduler> sched;  // tcpxComm::flow_mapper: the flows whose task ring has room
   std::mutex ctrl_mu;
   std::deque<CtrlMessage> ctrl_rx;  // the control socket's receive queue
   RequestRing rq;
@@ -306,6 +308,7 @@ struct Global {
   // Flags (environment, range-checked in tcpxInit like TCPX_GET_INT_FLAG, src/net_tcpx.cc:440-452).
   int flows_per_comm = 4;
   int use_helper_thread = 0;
+  int sched_alg = kSchedRoundRobin;  // NCCL_GPUDIRECTTCPX_SCHED_ALG
   bool fail_stop = true;
   // Observability (src/flags.cc:44-70, src/net_tcpx.cc:105-116).
   ClockFn clock = monotonic_ns;
@@ -321,6 +324,9 @@ struct Global {
   char pci_paths[kMaxDevices][64];
 };
 extern Global g;
+
+FlowScheduler* new_flow_scheduler(int alg);  // kSchedKaty, or round robin for anything else
+int sched_alg_from_name(const char* name, bool* valid);  // "RR" / "KATY" (exact); anything else is round robin
 
 const tcpxDeviceOps* default_device_ops();  // binds libtcpxu_hip.so, or nullptr (reason logged)
 ncclResult_t device_result(int rc, const char* what);

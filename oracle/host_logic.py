@@ -164,3 +164,86 @@ def parse_slowness_switches(text, switches):
 # request's enqueue (FREE -> POSTED) is traced as ACTIVE and its finish_posted (POSTED -> ACTIVE) as POSTED.
 REQUEST_TRACE_SEQUENCE = (3, 4, 2, 1, 0)  # enqueue, finish_posted, finish_active, finish_transmitting, dequeue
 TASK_TRACE_SEQUENCE = (3, 2, 1, 0)  # enqueue, finish_active, finish_completing, dequeue
+
+
+# ---- flow schedulers (src/flow_mapper.h) ----------------------------------------------------------------------------
+MAX_TASKS = 6  # src/work_queue.h:21
+MAX_SOCKETS = 8  # src/macro.h:36
+SCHED_ALG_RR, SCHED_ALG_KATY = 0, 1  # src/flow_mapper.h:25-29
+
+
+def sched_alg_from_flag(value):
+    """NCCL_GPUDIRECTTCPX_SCHED_ALG (src/net_tcpx.cc:643-665): unset or unknown -> RR; names are case sensitive."""
+    return SCHED_ALG_KATY if value == "KATY" else SCHED_ALG_RR
+
+
+class FlowMapperRR:
+    """FlowMapperRR (src/flow_mapper.h:137-157): a stack of the scheduled flows; the priority is ignored."""
+
+    def __init__(self):
+        self.flows = []
+
+    def reset(self):
+        self.flows = []
+
+    def has_flow(self):
+        return len(self.flows) > 0
+
+    def schedule(self, flow, prio):
+        self.flows.append(flow)
+
+    def pick(self):
+        return self.flows.pop() if self.flows else -1
+
+
+class FlowMapperKaty:
+    """FlowMapperKaty (src/flow_mapper.h:67-135): one bit per (priority, flow), priority-major; the lowest set
+    bit is served, moves one priority group up while its priority is below MAX_TASKS - 1, and at most
+    NUM_QUANTA_PER_SCHED = 2 flows are served between two resets."""
+
+    QUANTA = 2
+
+    def __init__(self):
+        self.reset()
+
+    def reset(self):
+        self.bitmap = 0
+        self.quanta = self.QUANTA
+
+    def has_flow(self):
+        return self.bitmap != 0 and self.quanta > 0
+
+    def schedule(self, flow, prio):
+        if prio < 0 or prio >= MAX_TASKS:
+            return
+        self.bitmap |= 1 << (flow + MAX_SOCKETS * prio)
+
+    def pick(self):
+        if not self.has_flow():
+            return -1
+        bit = (self.bitmap & -self.bitmap).bit_length() - 1
+        prio, flow = divmod(bit, MAX_SOCKETS)
+        self.bitmap &= ~(1 << bit)
+        if prio < MAX_TASKS - 1:
+            self.bitmap |= 1 << (bit + MAX_SOCKETS)
+        self.quanta -= 1
+        return flow
+
+
+def run_flow_script(mapper, script):
+    """Replays [op, args...] steps -- "reset", ["schedule", flow, prio], "pick", "has" -- and returns the answers
+    of the pick and has steps in order."""
+    out = []
+    for step in script:
+        op = step[0]
+        if op == "reset":
+            mapper.reset()
+        elif op == "schedule":
+            mapper.schedule(step[1], step[2])
+        elif op == "pick":
+            out.append(mapper.pick())
+        elif op == "has":
+            out.append(1 if mapper.has_flow() else 0)
+        else:
+            raise ValueError(op)
+    return out

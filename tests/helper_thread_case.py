@@ -1,4 +1,5 @@
-"""Run by test_plugin_host.py::test_socket_thread_mode in its own process (the flags are read at tcpxInit)."""
+"""Run by test_plugin_host.py (test_socket_thread_mode, test_katy_scheduler_receives_the_same_bytes) in its own
+process: the flags are read at tcpxInit."""
 import ctypes
 import os
 import sys
@@ -31,5 +32,9 @@ for config, shrink in ((4, 4), (2, 2), (5, 3)):
     assert np.array_equal(buf, expected_bytes(pool, wl.frags, wl.requests, int(wl.info.dst_bytes))), config
     assert comm.outstanding_pages() == 0
     comm.close()
+sched = ctypes.c_void_p()
+assert lib.tcpxFlowSchedCreate(None, ctypes.byref(sched)) == 0
+print("sched alg", lib.tcpxFlowSchedAlg(sched))
+lib.tcpxFlowSchedDestroy(sched)
 assert lib.tcpxFinalize() == 0
 print("helper-thread case ok")

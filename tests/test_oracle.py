@@ -217,3 +217,31 @@ def test_slowness_switches_hand_computed():
     for case in VECTORS["slowness_switches"]:
         assert host_logic.parse_slowness_switches(case["text"], list(case["before"])) == case["after"], case["ref"]
     assert host_logic.parse_slowness_switches(None, [0, 1, 0, 0]) == [0, 1, 0, 0]
+
+
+def test_flow_mappers_hand_computed():
+    for case in VECTORS["flow_mapper"]:
+        mapper = host_logic.FlowMapperKaty() if case["alg"] == "KATY" else host_logic.FlowMapperRR()
+        assert host_logic.run_flow_script(mapper, case["script"]) == case["expect"], case["ref"]
+    for case in VECTORS["sched_alg_flag"]:
+        assert host_logic.sched_alg_from_flag(case["value"]) == case["alg"], case["value"]
+
+
+def test_katy_serves_the_emptiest_flow_first():
+    """What the policy is for, checked without its bitmap: per reset, at most two picks; each pick is a flow whose
+    current priority (scheduled priority plus the times it was picked since) is minimal, lowest flow on a tie."""
+    rng = np.random.default_rng(0xCA7)
+    for _ in range(300):
+        mapper = host_logic.FlowMapperKaty()
+        prio = {int(f): int(rng.integers(0, host_logic.MAX_TASKS)) for f in rng.permutation(8)[: int(rng.integers(1, 9))]}
+        for f, p in prio.items():
+            mapper.schedule(f, p)
+        for n in range(3):
+            live = {f: p for f, p in prio.items() if p < host_logic.MAX_TASKS}
+            got = mapper.pick()
+            if n == 2 or not live:
+                assert got == -1
+                break
+            best = min(live.values())
+            assert got == min(f for f, p in live.items() if p == best)
+            prio[got] += 1

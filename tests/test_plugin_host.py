@@ -5,6 +5,7 @@ installed through the plugin's testing seam; nothing here measures or ships that
 Reference behaviour that each test pins is cited as src/...:line of google/nccl-plugin-gpudirecttcpx.
 """
 import ctypes
+import json
 import os
 import subprocess
 import sys
@@ -18,6 +19,7 @@ from plugin_common import ROOT, expected_bytes, load_emu
 sys.path.insert(0, os.path.join(ROOT, "oracle"))
 import host_logic  # noqa: E402  (test infrastructure)
 
+VECTORS = json.load(open(os.path.join(ROOT, "tests", "golden", "host_logic_vectors.json")))
 ARENA_BYTES = 64 << 20
 INTERNAL_ERROR, INVALID_ARGUMENT, INVALID_USAGE = 3, 4, 5
 
@@ -425,3 +427,73 @@ def test_socket_thread_mode(tmp_path):
     p = subprocess.run([sys.executable, script], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env, timeout=300)
     assert p.returncode == 0, p.stdout
     assert "helper-thread case ok" in p.stdout
+    assert "sched alg 0" in p.stdout
+
+
+# ---- flow scheduler (src/flow_mapper.h) -----------------------------------------------------------------------------
+def run_sched_script(lib, alg, script):
+    sched = ctypes.c_void_p()
+    assert lib.tcpxFlowSchedCreate(alg.encode() if alg is not None else None, ctypes.byref(sched)) == 0
+    out = []
+    try:
+        for step in script:
+            if step[0] == "reset":
+                lib.tcpxFlowSchedReset(sched)
+            elif step[0] == "schedule":
+                lib.tcpxFlowSchedSchedule(sched, step[1], step[2])
+            elif step[0] == "pick":
+                out.append(lib.tcpxFlowSchedPick(sched))
+            else:
+                out.append(lib.tcpxFlowSchedHasFlow(sched))
+    finally:
+        lib.tcpxFlowSchedDestroy(sched)
+    return out
+
+
+def test_flow_scheduler_hand_computed(env):
+    for case in VECTORS["flow_mapper"]:
+        assert run_sched_script(env.lib, case["alg"], case["script"]) == case["expect"], case["ref"]
+    for case in VECTORS["sched_alg_flag"]:
+        if case["value"] is None:
+            continue  # NULL means "what tcpxInit selected"; the unset flag is covered by test_socket_thread_mode
+        sched = ctypes.c_void_p()
+        assert env.lib.tcpxFlowSchedCreate(case["value"].encode(), ctypes.byref(sched)) == 0
+        assert env.lib.tcpxFlowSchedAlg(sched) == case["alg"], case["value"]
+        env.lib.tcpxFlowSchedDestroy(sched)
+    assert env.lib.tcpxFlowSchedCreate(b"RR", None) == INVALID_ARGUMENT
+    assert env.lib.tcpxFlowSchedPick(None) == -1 and env.lib.tcpxFlowSchedHasFlow(None) == 0
+
+
+@pytest.mark.parametrize("alg", ["RR", "KATY"])
+def test_flow_scheduler_matches_restatement_on_random_scripts(env, alg):
+    """Random schedule/pick/reset sequences as a comm would issue them: every flow scheduled at most once between
+    two resets, at most 8 flows (the RR mapper's stack holds MAX_SOCKETS entries and is not bounds-checked)."""
+    rng = np.random.default_rng(0x5CED + len(alg))
+    for _ in range(200):
+        script = []
+        for _ in range(int(rng.integers(1, 6))):
+            script.append(["reset"])
+            flows = rng.permutation(8)[: int(rng.integers(0, 9))]
+            for f in flows:
+                script.append(["schedule", int(f), int(rng.integers(-1, 8))])
+            for _ in range(int(rng.integers(0, 6))):
+                script.append(["pick"] if rng.random() < 0.7 else ["has"])
+        mapper = host_logic.FlowMapperKaty() if alg == "KATY" else host_logic.FlowMapperRR()
+        assert run_sched_script(env.lib, alg, script) == host_logic.run_flow_script(mapper, script)
+
+
+def test_katy_scheduler_receives_the_same_bytes():
+    """NCCL_GPUDIRECTTCPX_SCHED_ALG=KATY: the comm gates on the other scheduler; the received bytes do not change."""
+    script = os.path.join(ROOT, "tests", "helper_thread_case.py")
+    env = dict(os.environ, NCCL_GPUDIRECTTCPX_SCHED_ALG="KATY", NCCL_GPUDIRECTTCPX_AMD_FLOWS="8")
+    p = subprocess.run([sys.executable, script], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env, timeout=300)
+    assert p.returncode == 0, p.stdout
+    assert "sched alg 1" in p.stdout and "helper-thread case ok" in p.stdout
+
+
+def test_unknown_scheduler_name_means_round_robin():
+    script = os.path.join(ROOT, "tests", "helper_thread_case.py")
+    env = dict(os.environ, NCCL_GPUDIRECTTCPX_SCHED_ALG="katy", NCCL_GPUDIRECTTCPX_AMD_FLOWS="8")
+    p = subprocess.run([sys.executable, script], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env, timeout=300)
+    assert p.returncode == 0, p.stdout
+    assert "sched alg 0" in p.stdout
