@@ -287,28 +287,48 @@ def main():
         # Request completion latency, one request in flight: publish -> host poller sees the completion word.
         storm = pkg.Workload(3, seed=0xC0FFEE03)
         sd = np.array(storm.descs, copy=True)
-        n_lat = 2000
-        lat_items = (pkg.StreamItem * n_lat)()
-        for i in range(n_lat):
-            r = storm.requests[i % len(storm.requests)]
-            lat_items[i].bounce_base = pool_d.data_ptr()  # offsets beyond 256 MiB are folded into this pool below
-            lat_items[i].dst_base = dst_base + int(r["dst_off"]) % (args.chunks * chunk_bytes - 65536)
-            lat_items[i].descs_host = sd.ctypes.data + 16 * int(r["first_desc"])
-            lat_items[i].n_descs = int(r["n_descs"])
-        sd["src_off"] %= info0.pool_bytes
+        # The storm's 512 MiB pool is the first two of the bounce pool's copies; with fewer it is folded into one.
+        storm_pool_bytes = min(int(storm.info.pool_bytes), args.pools * int(info0.pool_bytes))
+        sd["src_off"] %= storm_pool_bytes
+        storm_dst_bytes = args.chunks * chunk_bytes
+        n_storm = len(storm.requests)
+        storm_items = (pkg.StreamItem * n_storm)()
+        for i, r in enumerate(storm.requests):
+            storm_items[i].bounce_base = pool_d.data_ptr()
+            storm_items[i].dst_base = dst_base + (i * 65536) % (storm_dst_bytes - 65536)
+            storm_items[i].descs_host = sd.ctypes.data + 16 * int(r["first_desc"])
+            storm_items[i].n_descs = int(r["n_descs"])
         sd["dst_off"] %= 65536
-        _, _, lat64k = run(lat_items, 1, want_latency=True)
+        _, _, lat64k = run(storm_items, 1, want_latency=True)
         lat4m_items = item_array(0, 200)
         _, _, lat4m = run(lat4m_items, 1, want_latency=True)
-        # the same 64 KiB requests back to back, 16 in flight: requests per second of the small-message storm
-        storm_wall, _, _ = run(lat_items, 16)
         result["latency_us"] = {
             "definition": "host publish of a slot -> host poller observes the completion word, one request in flight",
             "request_64KiB_16_descs": {"p50": round(percentile(lat64k, 50), 2), "p99": round(percentile(lat64k, 99), 2)},
             "request_4MiB_1078_descs": {"p50": round(percentile(lat4m, 50), 2), "p99": round(percentile(lat4m, 99), 2)},
         }
         result["p50_request_us"] = result["latency_us"]["request_64KiB_16_descs"]["p50"]
-        result["storm_64KiB_requests_per_s"] = round(n_lat / (storm_wall * 1e-6))
+        # The small-message storm: all 2048 requests of 64 KiB (16 fragments of 4 KiB each), W of them in flight,
+        # W x 16 = 64 .. 2048 descriptors handed to the engine per pass of the host loop.
+        sweep = []
+        for in_flight in (4, 8, 16, 32, 64, 128):
+            w, _, lat = run(storm_items, in_flight, want_latency=True)
+            sweep.append(
+                {
+                    "requests_in_flight": in_flight,
+                    "descriptors_in_flight": 16 * in_flight,
+                    "requests_per_s": round(n_storm / (w * 1e-6)),
+                    "payload_GBps": round(n_storm * 65536 / (w * 1e-6) / 1e9, 1),
+                    "p50_us": round(percentile(lat, 50), 2),
+                    "p99_us": round(percentile(lat, 99), 2),
+                }
+            )
+        result["storm_64KiB"] = {
+            "requests": n_storm,
+            "latency": "publish of a request's slot -> host poller observes its completion word",
+            "sweep": sweep,
+        }
+        result["storm_64KiB_requests_per_s"] = next(x["requests_per_s"] for x in sweep if x["requests_in_flight"] == 16)
 
         # Launch-per-batch kernel on the same chunk and on the 256 MiB bulk workload, and a plain copy kernel.
         us = ctypes.c_double()

@@ -156,8 +156,8 @@ typedef struct tcpxuStreamItem {
   uint32_t reserved;
 } tcpxuStreamItem;
 
-/* Slots the streaming driver can keep in flight: the unpack queues of four receive comms. */
-#define TCPXU_STREAM_MAX_DEPTH (4 * TCPXU_QUEUE_DEPTH)
+/* Slots the streaming driver can keep in flight: the unpack queues of eight receive comms. */
+#define TCPXU_STREAM_MAX_DEPTH (8 * TCPXU_QUEUE_DEPTH)
 
 /* Drives a started engine the way the plugin's proxy loop does, from one host thread, with no Python in the
  * loop: a mapped ring of `depth` slots (1..TCPXU_STREAM_MAX_DEPTH; TCPXU_QUEUE_DEPTH is one comm's unpack queue,

@@ -30,3 +30,18 @@ def test_bench_prints_one_json_line_with_the_contract_fields():
     cpu = r["cpu_baseline"]
     assert cpu["kind"] == "port" and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["unit"] == "GB/s" and cpu["sample"]
     assert r["parity_ok"] is True
+
+
+def test_bench_extras_report_latency_and_the_storm_sweep():
+    p = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bench.py"), "--steps", "200", "--warmup", "20", "--cpu-seconds", "0.2", "--chunks", "8", "--pools", "2"],
+        stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300, cwd=ROOT,
+    )  # fmt: skip
+    assert p.returncode == 0, p.stderr[-2000:]
+    r = json.loads(p.stdout.strip())
+    lat = r["latency_us"]["request_64KiB_16_descs"]
+    assert 0 < lat["p50"] <= lat["p99"] and r["p50_request_us"] == lat["p50"]
+    sweep = r["storm_64KiB"]["sweep"]
+    assert [x["descriptors_in_flight"] for x in sweep] == [64, 128, 256, 512, 1024, 2048] and r["storm_64KiB"]["requests"] == 2048
+    assert all(x["requests_per_s"] > 0 and 0 < x["p50_us"] <= x["p99_us"] for x in sweep)
+    assert r["single_comm"]["value"] > 0 and r["plugin_path"]["payload_GBps"] > 0 and r["plain_copy_kernel"]["rw_GBps"] > 0

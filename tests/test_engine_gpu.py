@@ -255,7 +255,7 @@ def test_engine_argument_errors(pkg, hip):
     e.destroy()
 
 
-@pytest.mark.parametrize("depth", [1, 5, 16, 64])
+@pytest.mark.parametrize("depth", [1, 5, 16, 64, 128])
 def test_engine_stream_depths(pkg, hip, oracle, depth):
     """The streaming driver (mapped slot ring, warm-up + timed items in one launch) at 1 to 64 slots in flight:
     the leader then cuts tickets of 8 to 32 descriptors by backlog, and every size must give the oracle's bytes.
@@ -297,7 +297,7 @@ def test_engine_stream_depths(pkg, hip, oracle, depth):
     assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
     # more than TCPXU_STREAM_MAX_DEPTH slots is refused before anything is launched
     e = Engine(pkg, hip)
-    assert hip.tcpxuEngineRunTimed(e.h, items, 4, 0, 65, 1000, ctypes.byref(wall), ctypes.byref(kern), None) == pkg.INVALID_ARGUMENT
+    assert hip.tcpxuEngineRunTimed(e.h, items, 4, 0, 129, 1000, ctypes.byref(wall), ctypes.byref(kern), None) == pkg.INVALID_ARGUMENT
     e.destroy()
 
 
