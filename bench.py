@@ -349,6 +349,19 @@ def main():
         torch.cuda.synchronize()
         pkg.check(hip.tcpxuCopyKernelTimed(dev, scratch.data_ptr() + n_copy, scratch.data_ptr(), n_copy, 3, 20, ctypes.byref(us)), "copy timed")
         result["plain_copy_kernel"] = {"bytes": n_copy, "launch_us": round(us.value, 2), "rw_GBps": round(2 * n_copy / us.value / 1e3, 1)}
+        # Each half of that copy on its own (loads only, stores only, same accesses), over 2 GiB: a copy spends
+        # 1/read + 1/write per byte, so its read+write rate cannot pass 2 / (1/read + 1/write).
+        pkg.check(hip.tcpxuCopyKernelTimed(dev, None, scratch.data_ptr(), 2 * n_copy, 3, 20, ctypes.byref(us)), "read timed")
+        read_gbps = 2 * n_copy / us.value / 1e3
+        pkg.check(hip.tcpxuCopyKernelTimed(dev, scratch.data_ptr(), None, 2 * n_copy, 3, 20, ctypes.byref(us)), "fill timed")
+        write_gbps = 2 * n_copy / us.value / 1e3
+        result["hbm_yardsticks"] = {
+            "read_only_GBps": round(read_gbps, 1),
+            "write_only_GBps": round(write_gbps, 1),
+            "copy_bound_rw_GBps": round(2.0 / (1.0 / read_gbps + 1.0 / write_gbps), 1),
+            "note": "plain kernels over 2 GiB with the unpack kernel's load and store instructions; the bound is what a "
+            "copy made of these two halves could reach at best on this box, against the 8000 GB/s of the roofline",
+        }
         del scratch
 
     pkg.check(hip.tcpxuEngineDestroy(engine), "tcpxuEngineDestroy")

@@ -95,7 +95,9 @@ int tcpxuUnpackBatchTimed(int device, const void* bounce_base, void* dst_base, c
                           uint64_t n_descs, int warmup, int iters, double* mean_us);
 
 /* Plain device-to-device copy kernel of `bytes` (multiple of 16), timed the same way: the achievable-copy
- * yardstick printed beside the unpack figure, and the known-size kernel used to calibrate HBM counters. */
+ * yardstick printed beside the unpack figure, and the known-size kernel used to calibrate HBM counters.
+ * With dst == NULL only the loads are issued (a read of `bytes`), with src == NULL only the stores (a fill):
+ * what the memory system gives to each half of a copy on its own. */
 int tcpxuCopyKernelTimed(int device, void* dst, const void* src, size_t bytes, int warmup, int iters,
                          double* mean_us);
 
