@@ -160,3 +160,27 @@ def test_argument_errors(pkg, hip):
     pkg.check(hip.tcpxuArenaCreate(0, 1 << 20, ctypes.byref(p)), "arena")
     assert p.value % 4096 == 0
     pkg.check(hip.tcpxuArenaDestroy(0, p), "arena destroy")
+
+
+def test_yardstick_kernels_copy_read_fill(pkg, hip):
+    """The measurement helpers behind the benchmark's copy, read-only and write-only figures: the copy is exact
+    (odd size in vectors, so the last workgroup is partial), the read leaves its source alone, the fill writes
+    every vector of the range and nothing beyond it."""
+    import torch
+
+    n = (3 << 20) + 16 * 37
+    src = torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda:0")
+    dst = torch.full((n + 64,), SENTINEL, dtype=torch.uint8, device="cuda:0")
+    keep = src.clone()
+    us = ctypes.c_double()
+    pkg.check(hip.tcpxuCopyKernelTimed(0, dst.data_ptr(), src.data_ptr(), n, 1, 3, ctypes.byref(us)), "copy")
+    assert us.value > 0 and torch.equal(dst[:n], src) and bool((dst[n:] == SENTINEL).all())
+    pkg.check(hip.tcpxuCopyKernelTimed(0, None, src.data_ptr(), n, 1, 3, ctypes.byref(us)), "read")
+    assert us.value > 0 and torch.equal(src, keep)
+    dst.fill_(SENTINEL)
+    pkg.check(hip.tcpxuCopyKernelTimed(0, dst.data_ptr(), None, n, 1, 3, ctypes.byref(us)), "fill")
+    words = dst[:n].view(torch.int32).view(-1, 4)
+    assert us.value > 0 and bool((words[:, 2] == -0x5A5A5A5B).all()) and bool((words[:, 3] == 0x5A5A5A5A).all())
+    assert bool((dst[n:] == SENTINEL).all())
+    assert hip.tcpxuCopyKernelTimed(0, None, None, n, 1, 3, ctypes.byref(us)) == pkg.INVALID_ARGUMENT
+    assert hip.tcpxuCopyKernelTimed(0, dst.data_ptr(), src.data_ptr(), n + 8, 1, 3, ctypes.byref(us)) == pkg.INVALID_ARGUMENT
