@@ -342,7 +342,9 @@ __device__ void retire_ticket(DevState* st, uint32_t* jobs_done, const Stage* st
   }
 }
 
-// Copy wavefront `wave` of kCopyWaves: fragments wave, wave + kCopyWaves, ... of the staged ticket.
+// Copy wavefront `wave` of kCopyWaves: its run of consecutive fragments of the staged ticket (an eighth of the
+// ticket, rounded up).  A wavefront that writes one contiguous stretch of the destination after another measured
+// about 1 % faster end to end than fragments dealt out in turn (wave, wave + kCopyWaves, ...).
 __device__ void copy_ticket(const Stage* stage, uint32_t wave, uint32_t lane, uint32_t* waves_on_last) {
   auto uniform = [](uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(v)); };
   const uint8_t* bounce = reinterpret_cast<const uint8_t*>((static_cast<uint64_t>(uniform(stage->payload[1])) << 32) |
@@ -350,7 +352,10 @@ __device__ void copy_ticket(const Stage* stage, uint32_t wave, uint32_t lane, ui
   uint8_t* dst =
       reinterpret_cast<uint8_t*>((static_cast<uint64_t>(uniform(stage->payload[3])) << 32) | uniform(stage->payload[2]));
   const uint32_t n = uniform(stage->payload[10]) & 0xFFu;
-  wave_copy_descriptors(stage->desc, n, wave, kCopyWaves, bounce, dst, lane, [&] {
+  const uint32_t per = (n + kCopyWaves - 1) / kCopyWaves;
+  const uint32_t first = wave * per < n ? wave * per : n;
+  const uint32_t end = first + per < n ? first + per : n;
+  wave_copy_descriptors(stage->desc, n, first, 1u, end, bounce, dst, lane, [&] {
     if (lane == 0) __hip_atomic_fetch_add(waves_on_last, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   });
 }

@@ -66,7 +66,7 @@ __global__ __launch_bounds__(kWgThreads) void unpack_batch_kernel(const uint8_t*
     cnt = batch_of(wg, &first);
     raw = fetch(first, cnt);  // in flight while this batch is copied
     __syncthreads();          // the stage is complete; every wavefront has left the stage written two batches ago
-    wave_copy_descriptors(staged[stage], cnt_now, wave, kWavesPerWg, bounce, dst, lane, [] {});
+    wave_copy_descriptors(staged[stage], cnt_now, wave, kWavesPerWg, cnt_now, bounce, dst, lane, [] {});
   }
 }
 

@@ -299,8 +299,8 @@ struct FragmentRounds {
   }
 };
 
-// Copies descriptors first, first + stride, ... < n of a descriptor list staged in LDS with the calling
-// wavefront; neighbours in the list decide which destination lines are shared.  One round (at most 4 KiB) is in
+// Copies descriptors first, first + stride, ... < end of a descriptor list of n staged in LDS with the calling
+// wavefront; neighbours in the list (whoever copies them) decide which destination lines are shared.  One round (at most 4 KiB) is in
 // flight per wavefront: keeping a second register set to overlap the next round's loads with this round's
 // stores measured slower, because fewer wavefronts then fit on a compute unit.  `bounce` and `dst` must be
 // wave-uniform.
@@ -308,8 +308,9 @@ struct FragmentRounds {
 // once if it has none): a caller that feeds the wavefront can use it to start fetching more work.
 template <typename OnLastFragment>
 __device__ __forceinline__ void wave_copy_descriptors(const tcpxuLoadMeta* descs, uint32_t n, uint32_t first,
-                                                      uint32_t stride, const uint8_t* bounce, uint8_t* dst,
-                                                      uint32_t lane, OnLastFragment&& on_last_fragment) {
+                                                      uint32_t stride, uint32_t end, const uint8_t* bounce,
+                                                      uint8_t* dst, uint32_t lane,
+                                                      OnLastFragment&& on_last_fragment) {
   // Everything that describes a fragment is wave-uniform; saying so keeps it in scalar registers and leaves
   // the vector registers to the payload in flight.
   auto uniform = [](uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(v)); };
@@ -318,7 +319,8 @@ __device__ __forceinline__ void wave_copy_descriptors(const tcpxuLoadMeta* descs
   };
   const uint64_t dst_addr = reinterpret_cast<uint64_t>(dst);
   uint32_t j = uniform(first);
-  if (j >= n) on_last_fragment();
+  end = uniform(end);
+  if (j >= end) on_last_fragment();
   FragmentRounds fr;
   // Next round of this wavefront's work, or false when there is none.  `prev` is the round before it.
   auto produce = [&](CopyRound& out, const CopyRound& prev) -> bool {
@@ -326,10 +328,10 @@ __device__ __forceinline__ void wave_copy_descriptors(const tcpxuLoadMeta* descs
       out = fr.next_round(prev);
       return true;
     }
-    while (j < n) {
+    while (j < end) {
       const uint32_t cur = j;
       j += stride;
-      if (j >= n) on_last_fragment();
+      if (j >= end) on_last_fragment();
       const tcpxuLoadMeta d = descs[cur];
       const uint32_t len = uniform(d.len);
       if (len == 0) continue;
