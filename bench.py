@@ -31,9 +31,9 @@ import numpy as np
 import __graft_entry__ as graft
 
 # HBM bytes moved per algorithmic byte (2 x fragment bytes) by unpack_engine_kernel on the headline workload:
-# hardware counters FETCH_SIZE (x1.99977, its reading for a copy kernel of known size) and WRITE_SIZE (x1.0),
-# 9071932 KiB + 9120371 KiB against 2 x 9011200 KiB over one launch of 1100 steps.
-TRAFFIC_PER_ALGORITHMIC_BYTE = 1.0094
+# hardware counters FETCH_SIZE (x1.99985, its reading for a copy kernel of known size) and WRITE_SIZE (x1.0),
+# 9122132 KiB + 9120374 KiB against 2 x 9011200 KiB over one launch of 1100 steps.
+TRAFFIC_PER_ALGORITHMIC_BYTE = 1.0122
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 CHUNK_CONFIG = 2
 
@@ -261,7 +261,7 @@ def main():
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "traffic": round(2.0 * launch_payload * TRAFFIC_PER_ALGORITHMIC_BYTE),
             "traffic_source": "FETCH_SIZE and WRITE_SIZE of this kernel on this workload (two rocprofv3 --pmc runs, scaled by "
-            "the same counters on the plain copy kernel: x1.99977 and x1.0) came to %.4f x the algorithmic bytes; "
+            "the same counters on the plain copy kernel: x1.99985 and x1.0) came to %.4f x the algorithmic bytes; "
             "that ratio times bytes_per_launch" % TRAFFIC_PER_ALGORITHMIC_BYTE,
             "bytes_per_launch": 2.0 * launch_payload,
             "steps_per_launch": args.warmup + args.steps,
@@ -349,8 +349,8 @@ def main():
         torch.cuda.synchronize()
         pkg.check(hip.tcpxuCopyKernelTimed(dev, scratch.data_ptr() + n_copy, scratch.data_ptr(), n_copy, 3, 20, ctypes.byref(us)), "copy timed")
         result["plain_copy_kernel"] = {"bytes": n_copy, "launch_us": round(us.value, 2), "rw_GBps": round(2 * n_copy / us.value / 1e3, 1)}
-        # Each half of that copy on its own (loads only, stores only, same accesses), over 2 GiB: a copy spends
-        # 1/read + 1/write per byte, so its read+write rate cannot pass 2 / (1/read + 1/write).
+        # Each half of that copy on its own (loads only, stores only, same accesses), over 2 GiB: a copy that spends
+        # 1/read + 1/write per byte moves 2 / (1/read + 1/write) bytes of read + write per second.
         pkg.check(hip.tcpxuCopyKernelTimed(dev, None, scratch.data_ptr(), 2 * n_copy, 3, 20, ctypes.byref(us)), "read timed")
         read_gbps = 2 * n_copy / us.value / 1e3
         pkg.check(hip.tcpxuCopyKernelTimed(dev, scratch.data_ptr(), None, 2 * n_copy, 3, 20, ctypes.byref(us)), "fill timed")
@@ -359,8 +359,8 @@ def main():
             "read_only_GBps": round(read_gbps, 1),
             "write_only_GBps": round(write_gbps, 1),
             "copy_bound_rw_GBps": round(2.0 / (1.0 / read_gbps + 1.0 / write_gbps), 1),
-            "note": "plain kernels over 2 GiB with the unpack kernel's load and store instructions; the bound is what a "
-            "copy made of these two halves could reach at best on this box, against the 8000 GB/s of the roofline",
+            "note": "plain kernels over 2 GiB with the unpack kernel's load and store instructions; copy_bound is what a "
+            "plain copy made of these two halves comes to (1/read + 1/write per byte), against the roofline's 8000 GB/s",
         }
         del scratch
 
