@@ -114,7 +114,8 @@ typedef struct tcpxuEngineConfig {
   uint32_t workgroups;      /* persistent grid size, 0 = fill the GPU */
   uint32_t descs_per_ticket;/* descriptors one workgroup takes at a time (1..64); 0 = chosen per submission from
                                the backlog of descriptors not yet unpacked: 8 when the engine is idle (lowest
-                               latency) up to 32 when every workgroup has work queued (highest throughput) */
+                               latency) up to 32 when every workgroup has work queued (highest throughput); a
+                               submission of at most 32 descriptors stays whole once 8 or more are in flight */
   uint32_t spin_limit;      /* the kernel leaves by itself after this many consecutive empty polls of the ring
                                (about 1.2 us each) and is launched again by the next submission, so that a
                                device-wide synchronize never waits on an idle engine; 0 = default (400, about

@@ -55,9 +55,22 @@ constexpr uint32_t kMaxDescsPerTicket = 64;
 // all submissions not yet completed, counting each in full until it completes (how far the slots in flight have
 // got depends on the ticket size itself and would feed back).  The steps are where throughput measured at 1 to
 // 64 slots of 4 MiB in flight changed hands between sizes; 8 is one fragment per copy wavefront.
+// (Descriptors per worker workgroup below 13, 18, 30, 75; written without the division, which the leader would pay
+// for on every submission.  backlog <= 2^20 and workers < 2^16 keep the products in 32 bits.)
 __device__ __forceinline__ uint32_t ticket_size_for(uint32_t backlog, uint32_t workers) {
-  const uint32_t per_worker = backlog / workers;
-  return per_worker < 13 ? 8u : per_worker < 18 ? 12u : per_worker < 30 ? 16u : per_worker < 75 ? 24u : 32u;
+  return backlog < 13u * workers ? 8u : backlog < 18u * workers ? 12u : backlog < 30u * workers ? 16u
+                                                          : backlog < 75u * workers ? 24u : 32u;
+}
+// Ticket size for one submission of n descriptors when `in_flight` submissions (this one included) are not yet
+// completed; each is taken to be as long as this one.  A small submission among many stays whole: with 8 or
+// more in flight the parallelism is in the submissions, and a submission that is one ticket costs the leader
+// one store instead of a pass of its loop.  (64 KiB requests of 16 fragments, p50 publish -> done: 8.7 -> 9.1 us
+// at 8 in flight, 17.5 -> 9.3 us at 32, where the leader's loop had become the queue.)
+constexpr uint32_t kManyInFlight = 8, kSmallSubmission = 32;
+__device__ __forceinline__ uint32_t ticket_size_for_submission(uint32_t in_flight, uint32_t n, uint32_t workers) {
+  if (in_flight >= kManyInFlight && n <= kSmallSubmission) return kSmallSubmission;
+  const uint64_t all = static_cast<uint64_t>(in_flight) * n;
+  return ticket_size_for(all > (1u << 20) ? (1u << 20) : static_cast<uint32_t>(all), workers);
 }
 constexpr uint32_t kMaxDescsPerSubmission = 1u << 20;
 constexpr uint32_t kStopReplicas = 64;
@@ -168,9 +181,48 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
       return lane_value(i % 3 == 0 ? sect.x : i % 3 == 1 ? sect.y : sect.z, src);
     };
 
+    // Sixteen at a stroke.  A submission that fits one ticket becomes that ticket almost unchanged -- the two
+    // records share their layout up to the last sector -- so the four lanes that hold an entry's sectors write
+    // its ticket themselves: the leading run of such entries costs one store instruction, not a pass of the
+    // loop below each (which took about 0.6 us per entry and capped a storm of small requests at 1.6 M/s).
     uint32_t consumed = 0;
+    if ((ok_mask & 0xFull) == 0xFull) {  // entry s is there
+      const uint32_t n = bcast(sect.y, lane | 3u);  // payload word 10 sits in .y of sector 3
+      const bool all_sectors = ((ok_mask >> (4 * k_of_lane)) & 0xFull) == 0xFull;
+      const bool small = all_sectors && n - 1u < kSmallSubmission;  // 1 .. kSmallSubmission descriptors
+      if ((__ballot(small) & 1ull) != 0) {
+        const uint32_t done_now = bcast(aux, k_of_lane);
+        const uint32_t target_prev = bcast(aux, kPollEntries + k_of_lane);
+        const uint32_t in_flight = static_cast<uint32_t>(s + k_of_lane) - jobs_completed + 1u;
+        const uint32_t per_ticket =
+            fixed_per_ticket != 0 ? fixed_per_ticket : ticket_size_for_submission(in_flight, n, gridDim.x - 1);
+        const bool one_ticket = small && n <= per_ticket && done_now == target_prev;
+        const uint64_t not_fast = ~__ballot(one_ticket);
+        uint32_t run = not_fast == 0 ? kPollEntries : static_cast<uint32_t>(__builtin_ctzll(not_fast)) >> 2;
+        const uint32_t room = kTicketRing - (static_cast<uint32_t>(tickets_out) - tickets_done);
+        run = std::min(run, room);
+        if (run != 0) {
+          if (k_of_lane < run) {
+            const uint32_t sector = lane & 3u;
+            const uint64_t t = tickets_out + k_of_lane;
+            const uint32_t stamp = static_cast<uint32_t>(t + 1);
+            const uint32_t slot = static_cast<uint32_t>(s + k_of_lane) & ring_mask;
+            const uint32_t target = target_prev + 1u;
+            u32x4 v{sect.x, sect.y, sect.z, stamp};
+            if (sector == 3) {
+              v.y = n | (slot << 8);
+              v.z = target;
+              sys_store(&job_target[slot], target);
+            }
+            store_vec_sys(reinterpret_cast<uint8_t*>(&st->tickets[t & (kTicketRing - 1)]) + 16 * sector, v);
+          }
+          tickets_out += run;
+          consumed = run;
+        }
+      }
+    }
 #pragma unroll 1
-    for (uint32_t k = 0; k < kPollEntries; ++k) {
+    for (uint32_t k = consumed; k < kPollEntries; ++k) {
       if (((ok_mask >> (4 * k)) & 0xFull) != 0xFull) break;
       const uint32_t fl = 4 * k;  // first lane of entry k
       const uint32_t n = payload_of(fl, 10);
@@ -185,8 +237,8 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
       } else {
         // Submissions not yet completed, this one included, taken to be as long as this one.
         const uint32_t in_flight = static_cast<uint32_t>(s + k) - jobs_completed + 1u;
-        const uint32_t backlog = in_flight > (1u << 20) / n ? (1u << 20) : in_flight * n;
-        const uint32_t per_ticket = fixed_per_ticket != 0 ? fixed_per_ticket : ticket_size_for(backlog, gridDim.x - 1);
+        const uint32_t per_ticket =
+            fixed_per_ticket != 0 ? fixed_per_ticket : ticket_size_for_submission(in_flight, n, gridDim.x - 1);
         const uint32_t nt = (n + per_ticket - 1) / per_ticket;
         const uint32_t slot = static_cast<uint32_t>(s + k) & ring_mask;
         const uint32_t done_now = lane_value(aux, k);
@@ -535,8 +587,8 @@ int tcpxuEngineCreate(int device, const tcpxuEngineConfig* config, tcpxuEngine**
     if (v && *v) per_cu = std::min(std::max(static_cast<uint32_t>(atoi(v)), 1u), static_cast<uint32_t>(std::max(max_active, 1)));
     cfg.workgroups = cus * per_cu + 1;
   }
-  if (cfg.workgroups < 2) {
-    set_error("an engine needs the leader workgroup and at least one worker");
+  if (cfg.workgroups < 2 || cfg.workgroups > (1u << 16)) {
+    set_error("an engine needs the leader workgroup and 1 to 65535 workers");
     return TCPXU_INVALID_ARGUMENT;
   }
 
