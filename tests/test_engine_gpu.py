@@ -357,3 +357,54 @@ def test_engine_bursts_around_the_idle_exit(pkg, hip, oracle):
     e.destroy()
     m.free()
     assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
+
+
+@pytest.mark.parametrize("depth", [3, 16, 128])
+def test_engine_storm_of_mixed_small_submissions(pkg, hip, oracle, depth):
+    """Thousands of submissions of 0 to 300 ragged fragments in random order, `depth` of them in flight: runs of
+    submissions that the leader turns into tickets sixteen at a time are broken at every position by empty ones,
+    by ones just over the one-ticket limit and by ones that need many tickets; each submission owns a stretch of
+    the destination and every byte must be the oracle's."""
+    import torch
+
+    rng = np.random.default_rng(0x570A + depth)
+    pool = np.random.default_rng(0xD00D).integers(0, 256, size=8 << 20, dtype=np.uint8)
+    sizes = rng.choice([0, 1, 2, 7, 8, 9, 15, 16, 17, 31, 32, 33, 40, 64, 65, 300], size=3000,
+                       p=[.05, .1, .05, .05, .1, .05, .05, .2, .05, .05, .1, .03, .03, .03, .03, .03])
+    rows, subs, dst_off = [], [], 0
+    for n in sizes:
+        first = len(rows)
+        base = dst_off
+        for _ in range(int(n)):
+            ln = int(rng.integers(1, 4097)) if rng.random() < 0.5 else 4096
+            page = int(rng.integers(0, len(pool) >> 12))
+            so = (page << 12) + int(rng.integers(0, 4096 - ln + 1))
+            rows.append((so, ln, dst_off - base))
+            dst_off += ln
+        subs.append((first, int(n), base))
+        dst_off += int(rng.integers(0, 40))  # a gap that must keep the sentinel
+    descs = make_descs(rows)
+    total = dst_off + 64
+    expect = np.full(GUARD + total + GUARD, SENTINEL, dtype=np.uint8)
+    absolute = descs.copy()
+    for first, n, base in subs:
+        absolute["dst_off"][first : first + n] += base
+    expect[:] = oracle_expected(oracle, pool, absolute, total, 0)
+    pool_d = torch.from_numpy(pool).to("cuda:0")
+    dst_d = torch.full((expect.nbytes,), SENTINEL, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    items = (pkg.StreamItem * len(subs))()
+    for i, (first, n, base) in enumerate(subs):
+        items[i].bounce_base = pool_d.data_ptr()
+        items[i].dst_base = dst_d.data_ptr() + GUARD + base
+        items[i].descs_host = descs.ctypes.data + 16 * first
+        items[i].n_descs = n
+    e = Engine(pkg, hip)
+    print("engine storm case: depth=%d submissions=%d descriptors=%d" % (depth, len(subs), len(descs)), flush=True)
+    wall, kern = ctypes.c_double(), ctypes.c_double()
+    lat = (ctypes.c_double * len(subs))()
+    pkg.check(hip.tcpxuEngineRunTimed(e.h, items, len(subs), 0, depth, 20000, ctypes.byref(wall), ctypes.byref(kern), lat), "tcpxuEngineRunTimed")
+    assert e.completed() == len(subs) and min(lat) > 0
+    e.destroy()
+    got = dst_d.cpu().numpy()
+    assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
