@@ -31,8 +31,8 @@ import numpy as np
 import __graft_entry__ as graft
 
 # HBM bytes moved per algorithmic byte (2 x fragment bytes) by unpack_engine_kernel on the headline workload:
-# hardware counters FETCH_SIZE (x1.99985, its reading for a copy kernel of known size) and WRITE_SIZE (x1.0),
-# 9122132 KiB + 9120374 KiB against 2 x 9011200 KiB over one launch of 1100 steps.
+# hardware counters FETCH_SIZE (x1.99983, its reading for a copy kernel of known size) and WRITE_SIZE (x1.0),
+# 9121939 KiB + 9120367 KiB against 2 x 9011200 KiB over one launch of 1100 steps.
 TRAFFIC_PER_ALGORITHMIC_BYTE = 1.0122
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 CHUNK_CONFIG = 2
@@ -261,7 +261,7 @@ def main():
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "traffic": round(2.0 * launch_payload * TRAFFIC_PER_ALGORITHMIC_BYTE),
             "traffic_source": "FETCH_SIZE and WRITE_SIZE of this kernel on this workload (two rocprofv3 --pmc runs, scaled by "
-            "the same counters on the plain copy kernel: x1.99985 and x1.0) came to %.4f x the algorithmic bytes; "
+            "the same counters on the plain copy kernel: x1.99983 and x1.0) came to %.4f x the algorithmic bytes; "
             "that ratio times bytes_per_launch" % TRAFFIC_PER_ALGORITHMIC_BYTE,
             "bytes_per_launch": 2.0 * launch_payload,
             "steps_per_launch": args.warmup + args.steps,
