@@ -87,7 +87,9 @@ struct alignas(64) Record {
 constexpr int kPayloadWords = 12;
 __host__ __device__ constexpr int payload_slot(int i) { return (i / 3) * 4 + (i % 3); }
 // Submission payload: 0-1 bounce, 2-3 dst, 4-5 descs, 6-7 done_flag, 8-9 done_value, 10 n_descs, 11 unused.
-// Ticket payload:     0-1 bounce, 2-3 dst, 4-5 descs, 6-7 done_flag, 8-9 done_value, 10 n | job << 8, 11 target.
+// Ticket payload:     0-1 bounce, 2-3 dst, 4-5 descs, 6-7 done_flag, 8-9 done_value, 10 n | job << 8 | only << 31,
+//                     11 target.  `only`: the submission's only ticket (the job slot index is below 2^16).
+constexpr uint32_t kOnlyTicket = 1u << 31;
 
 struct HostCtl {  // mapped host memory
   alignas(64) uint64_t tail;       // host -> GPU: submissions published so far
@@ -210,7 +212,7 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
             const uint32_t target = target_prev + 1u;
             u32x4 v{sect.x, sect.y, sect.z, stamp};
             if (sector == 3) {
-              v.y = n | (slot << 8);
+              v.y = n | (slot << 8) | kOnlyTicket;
               v.z = target;
               sys_store(&job_target[slot], target);
             }
@@ -264,7 +266,7 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
           u32x4 v{bounce_lo, bounce_hi, dst_lo, stamp};
           if (sector == 1) v = u32x4{dst_hi, static_cast<uint32_t>(d), static_cast<uint32_t>(d >> 32), stamp};
           if (sector == 2) v = u32x4{flag_lo, flag_hi, val_lo, stamp};
-          if (sector == 3) v = u32x4{val_hi, count | (slot << 8), target, stamp};
+          if (sector == 3) v = u32x4{val_hi, count | (slot << 8) | (nt == 1 ? kOnlyTicket : 0u), target, stamp};
           store_vec_sys(reinterpret_cast<uint8_t*>(&st->tickets[t & (kTicketRing - 1)]) + 16 * sector, v);
         }
         tickets_out += nt;
@@ -380,14 +382,23 @@ __device__ uint32_t try_fetch_ticket(DevState* st, const uint32_t* stop_word, ui
 // completion word.
 __device__ void retire_ticket(DevState* st, uint32_t* jobs_done, const Stage* stage, uint32_t lane) {
   if (lane == 0) {
-    const uint32_t job = stage->payload[10] >> 8;
+    const uint32_t job = (stage->payload[10] & ~kOnlyTicket) >> 8;
     const uint32_t target = stage->payload[11];
+    const uint64_t done_flag = (static_cast<uint64_t>(stage->payload[7]) << 32) | stage->payload[6];
+    const uint64_t done_value = (static_cast<uint64_t>(stage->payload[9]) << 32) | stage->payload[8];
+    if ((stage->payload[10] & kOnlyTicket) != 0) {
+      // The submission's only ticket completes it: tell the caller first, count afterwards (nobody waits for the
+      // counts' round trips; the leader reads them when it wants the job slot again).
+      sys_store(reinterpret_cast<uint64_t*>(done_flag), done_value);
+      __hip_atomic_fetch_add(&jobs_done[job], 1u, __ATOMIC_RELAXED, SYS);
+      __hip_atomic_fetch_add(&st->tickets_done, 1ull, __ATOMIC_RELAXED, SYS);
+      __hip_atomic_fetch_add(&st->jobs_completed, 1ull, __ATOMIC_RELAXED, SYS);
+      return;
+    }
     const uint32_t count = __hip_atomic_fetch_add(&jobs_done[job], 1u, __ATOMIC_RELAXED, SYS) + 1u;
     __hip_atomic_fetch_add(&st->tickets_done, 1ull, __ATOMIC_RELAXED, SYS);
     if (count == target) {
       // Every other ticket's payload was in memory before it was counted, and so is this one's.
-      const uint64_t done_flag = (static_cast<uint64_t>(stage->payload[7]) << 32) | stage->payload[6];
-      const uint64_t done_value = (static_cast<uint64_t>(stage->payload[9]) << 32) | stage->payload[8];
       sys_store(reinterpret_cast<uint64_t*>(done_flag), done_value);
       __hip_atomic_fetch_add(&st->jobs_completed, 1ull, __ATOMIC_RELAXED, SYS);
     }
