@@ -97,6 +97,50 @@ def plugin_path(pkg, hip, torch, workloads, pool):
     }
 
 
+def other_configs(pkg, torch, run):
+    """The other workloads of the measurement contract through the same engine, 64 slots in flight, sources spread
+    over at least 1 GiB where the workload's own pool would fit the Infinity Cache.  Their bytes are checked by the
+    GPU tests; here they are only timed."""
+    out = {}
+    for cfg, passes, pool_copies, note in (
+        (4, 120, 4, "bulk: one 256 MiB message of 65536 page-aligned 4 KiB fragments from a 1 GiB pool, as 64 requests of 4 MiB"),
+        (5, 512, 4, "adversarial: 32 MiB, fragment lengths uniform in 1..4096, 10% empty descriptors, destination offset by 3 bytes"),
+        (1, 2048, 1, "one 1 MiB message of 256 page-aligned fragments from a 16 MiB pool: cache-resident by construction"),
+    ):
+        wl = pkg.Workload(cfg, seed=0xC0FFEE00 + cfg)
+        info = wl.info
+        pool_bytes, dst_bytes = int(info.pool_bytes), int(info.dst_bytes)
+        pool_d = torch.empty(pool_copies * pool_bytes, dtype=torch.uint8, device="cuda:0").random_(0, 256)
+        stride = (dst_bytes + int(info.dst_misalign) + 4095) // 4096 * 4096
+        n_dst = max(2, min(passes, (512 << 20) // stride))
+        dst_d = torch.empty(n_dst * stride + 512, dtype=torch.uint8, device="cuda:0")
+        torch.cuda.synchronize()
+        descs = np.ascontiguousarray(wl.descs)
+        reqs = [(int(r["first_desc"]), int(r["n_descs"])) for r in wl.requests]
+        assert int((descs["dst_off"] + descs["len"]).max()) <= dst_bytes and int((descs["src_off"].astype(np.int64) + descs["len"]).max()) <= pool_bytes
+        items = (pkg.StreamItem * (passes * len(reqs)))()
+        i = 0
+        for ps in range(passes):
+            for first, n in reqs:
+                items[i].bounce_base = pool_d.data_ptr() + (ps % pool_copies) * pool_bytes
+                # descriptor offsets count from the start of the message, whichever request they belong to
+                items[i].dst_base = dst_d.data_ptr() + 256 + (ps % n_dst) * stride + int(info.dst_misalign)
+                items[i].descs_host = descs.ctypes.data + 16 * first
+                items[i].n_descs = n
+                i += 1
+        wall_us, kernel_us, _ = run(items, 64, warmup_items=len(reqs))
+        payload = float(info.payload_bytes) * (passes - 1)
+        out["config_%d" % cfg] = {
+            "what": note,
+            "requests_per_pass": len(reqs),
+            "descriptors_per_pass": int(info.n_descs),
+            "payload_GBps": round(payload / (wall_us * 1e-6) / 1e9, 1),
+            "rw_frac_of_hbm_peak": round(2.0 * payload / (wall_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+        }
+        del pool_d, dst_d
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -363,6 +407,8 @@ def main():
             "plain copy made of these two halves comes to (1/read + 1/write per byte), against the roofline's 8000 GB/s",
         }
         del scratch
+
+        result["other_configs"] = other_configs(pkg, torch, run)
 
     pkg.check(hip.tcpxuEngineDestroy(engine), "tcpxuEngineDestroy")
 
