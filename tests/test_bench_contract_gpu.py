@@ -45,3 +45,7 @@ def test_bench_extras_report_latency_and_the_storm_sweep():
     assert [x["descriptors_in_flight"] for x in sweep] == [64, 128, 256, 512, 1024, 2048] and r["storm_64KiB"]["requests"] == 2048
     assert all(x["requests_per_s"] > 0 and 0 < x["p50_us"] <= x["p99_us"] for x in sweep)
     assert r["single_comm"]["value"] > 0 and r["plugin_path"]["payload_GBps"] > 0 and r["plain_copy_kernel"]["rw_GBps"] > 0
+    assert sorted(r["other_configs"]) == ["config_1", "config_4", "config_5"]
+    assert all(v["payload_GBps"] > 0 for v in r["other_configs"].values())
+    yard = r["hbm_yardsticks"]
+    assert yard["read_only_GBps"] > 0 and yard["write_only_GBps"] > 0 and yard["copy_bound_rw_GBps"] > 0
