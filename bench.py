@@ -97,6 +97,42 @@ def plugin_path(pkg, hip, torch, workloads, pool):
     }
 
 
+def batch_kernel_line(pkg, hip, torch, dev, chunks=48, pools=15, warmup=3, iters=20):
+    """tcpxuUnpackBatch on `chunks` chunks of the headline workload as ONE descriptor list and one launch: chunk c
+    reads copy c % pools of the 256 MiB pool (descriptor offsets are 32-bit: 15 copies stay below 4 GiB) and writes
+    its own 8 MiB of the destination, so a launch moves chunks x 8 MiB each way with nothing read or written twice."""
+    wls = [pkg.Workload(CHUNK_CONFIG, seed=0xC0FFEE02 + 7919 * i) for i in range(chunks)]
+    info0 = wls[0].info
+    pool_bytes, chunk_bytes = int(info0.pool_bytes), int(info0.payload_bytes)
+    parts = []
+    for c, wl in enumerate(wls):
+        d = np.array(wl.descs, copy=True)
+        d["src_off"] += np.uint32((c % pools) * pool_bytes)
+        d["dst_off"] += np.uint64(c * chunk_bytes)
+        parts.append(d)
+    descs = np.ascontiguousarray(np.concatenate(parts))
+    assert int(descs["src_off"].astype(np.int64).max()) + 4096 <= pools * pool_bytes <= 1 << 32
+    pool_d = torch.empty(pools * pool_bytes, dtype=torch.uint8, device="cuda:0").random_(0, 256)
+    dst_d = torch.empty(chunks * chunk_bytes + 512, dtype=torch.uint8, device="cuda:0")
+    descs_d = torch.from_numpy(descs.view(np.uint8)).to("cuda:0")
+    torch.cuda.synchronize()
+    us = ctypes.c_double()
+    pkg.check(
+        hip.tcpxuUnpackBatchTimed(dev, pool_d.data_ptr(), dst_d.data_ptr() + 256, descs_d.data_ptr(), len(descs), warmup, iters, ctypes.byref(us)),
+        "tcpxuUnpackBatchTimed",
+    )
+    payload = float(descs["len"].sum())
+    return {
+        "kernel": "unpack_batch_kernel",
+        "workload": "%d chunks of 8 MiB in one launch, %d descriptors, sources in %d copies of the 256 MiB pool" % (chunks, len(descs), pools),
+        "launches": warmup + iters,
+        "bytes_per_launch": 2.0 * payload,
+        "launch_us": round(us.value, 2),
+        "rw_GBps": round(2.0 * payload / us.value / 1e3, 1),
+        "frac": round(2.0 * payload / us.value / 1e3 / HBM_PEAK_GBPS, 4),
+    }
+
+
 def other_configs(pkg, torch, run):
     """The other workloads of the measurement contract through the same engine, 64 slots in flight, sources spread
     over at least 1 GiB where the workload's own pool would fit the Infinity Cache.  Their bytes are checked by the
@@ -166,6 +202,12 @@ def main():
         help="run only the plain copy kernel on MIB mebibytes (10 launches) and exit: a kernel of known traffic "
         "against which hardware counters (FETCH_SIZE, WRITE_SIZE) are scaled",
     )
+    ap.add_argument(
+        "--batch-kernel",
+        action="store_true",
+        help="run only the launch-per-batch kernel on 48 chunks of the headline workload in one launch (384 MiB of "
+        "payload, 15 copies of the pool) and exit: what a kernel trace of unpack_batch_kernel should see",
+    )
     args = ap.parse_args()
     if not 1 <= args.comms <= 4 or not 1 <= args.depth <= 16 or not 1 <= args.pools <= 16:
         sys.exit("bench.py: --comms must be 1..4, --depth 1..16, --pools 1..16")
@@ -187,6 +229,9 @@ def main():
         us = ctypes.c_double()
         pkg.check(hip.tcpxuCopyKernelTimed(dev, b.data_ptr(), a.data_ptr(), n, 0, 10, ctypes.byref(us)), "tcpxuCopyKernelTimed")
         print(json.dumps({"kernel": "copy_kernel", "launches": 10, "bytes_read_per_launch": n, "bytes_written_per_launch": n, "launch_us": round(us.value, 2)}))
+        return
+    if args.batch_kernel:
+        print(json.dumps(batch_kernel_line(pkg, hip, torch, dev)))
         return
     name = ctypes.create_string_buffer(256)
     cus = ctypes.c_int()
@@ -409,6 +454,7 @@ def main():
         del scratch
 
         result["other_configs"] = other_configs(pkg, torch, run)
+        result["launch_per_batch_384MiB"] = batch_kernel_line(pkg, hip, torch, dev)
 
     pkg.check(hip.tcpxuEngineDestroy(engine), "tcpxuEngineDestroy")
 
