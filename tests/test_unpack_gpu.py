@@ -184,3 +184,37 @@ def test_yardstick_kernels_copy_read_fill(pkg, hip):
     assert bool((dst[n:] == SENTINEL).all())
     assert hip.tcpxuCopyKernelTimed(0, None, None, n, 1, 3, ctypes.byref(us)) == pkg.INVALID_ARGUMENT
     assert hip.tcpxuCopyKernelTimed(0, dst.data_ptr(), src.data_ptr(), n + 8, 1, 3, ctypes.byref(us)) == pkg.INVALID_ARGUMENT
+
+
+def test_batch_launches_replayed_from_a_hip_graph(pkg, hip, oracle):
+    """A launch-bound loop of small batches (32 requests of 16 fragments, one tcpxuUnpackBatch each) captured once
+    into a HIP graph on a caller's stream and replayed: every replay, with the pool refilled and the destination
+    reset by ordinary eager work in between, must give the oracle's bytes for the pool of that replay."""
+    import torch
+
+    wl = pkg.Workload(3, seed=0x6A9, shrink=6)
+    info = wl.info
+    reqs = [(int(r["first_desc"]), int(r["n_descs"])) for r in wl.requests][:32]
+    n_descs = reqs[-1][0] + reqs[-1][1]
+    descs = np.ascontiguousarray(wl.descs[:n_descs])
+    dst_bytes = int((descs["dst_off"] + descs["len"]).max())
+    pool = np.empty(info.pool_bytes, dtype=np.uint8)
+    wl.fill_window(0, pool)
+    g = GpuBuffers(pool, descs, dst_bytes, 0)
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    print("graph case: %d launches, %d descriptors" % (len(reqs), n_descs), flush=True)
+    with torch.cuda.graph(graph, stream=stream):
+        s = torch.cuda.current_stream().cuda_stream
+        for first, n in reqs:
+            pkg.check(hip.tcpxuUnpackBatch(0, g.pool.data_ptr(), g.dst_base, g.descs.data_ptr() + 16 * first, n, ctypes.c_void_p(s)), "tcpxuUnpackBatch")
+    for replay in range(3):
+        if replay:
+            pool = np.roll(pool, 4099 * replay) ^ np.uint8(replay)
+            g.pool.copy_(torch.from_numpy(pool))
+        g.reset()
+        graph.replay()
+        torch.cuda.synchronize()
+        expect = oracle_expected(oracle, pool, descs, dst_bytes, 0)
+        got = g.result()
+        assert first_difference(got, expect) is None, "replay %d, first (index, got, want, count): %r" % (replay, first_difference(got, expect))
