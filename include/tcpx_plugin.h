@@ -121,6 +121,11 @@ typedef struct tcpxDeviceOps {
   int (*engine_submit)(tcpxuEngine* engine, const void* bounce_base, void* dst_base, const void* descs_dev,
                        uint32_t n_descs, void* done_flag_dev, uint64_t done_value);
   const char* (*last_error)(void);
+  /* Optional (may be NULL, and the allocation may fail): device memory that the host can write, for a second
+   * copy of the descriptors of small requests (tcpxuVisibleAlloc / Free / Flush, include/tcpx_unpack_hip.h). */
+  int (*visible_alloc)(int device, size_t bytes, void** host_ptr, void** dev_ptr);
+  int (*visible_free)(int device, void* host_ptr);
+  void (*visible_flush)(void);
 } tcpxDeviceOps;
 
 /* Installs `ops` in place of the HIP layer (NULL restores the default binding).  For host-logic tests only;

@@ -77,6 +77,20 @@ int tcpxuDeviceSynchronize(int device);
 int tcpxuMappedAlloc(int device, size_t bytes, void** host_ptr, void** dev_ptr);
 int tcpxuMappedFree(int device, void* host_ptr);
 
+/* Allocates `bytes` (at most 64 MiB) of DEVICE memory that the host can write through the PCIe BAR, for the few
+ * bytes per request that the GPU should not have to fetch over PCIe itself: a caller copies the descriptors of a
+ * small request here (in addition to the mapped slot above), calls tcpxuVisibleFlush, and only then submits the
+ * request with this copy's device address as `descs`.  The copy is a posted write that PCIe delivers before the
+ * completion of any later read by the GPU of host memory written after the flush, so a GPU that has seen the
+ * submission finds the descriptors in its own memory (a lone request of 1..16 descriptors completes 0.7-1.3 us
+ * sooner).  Write-combined for the host: write whole records, never read.  TCPXU_INVALID_USAGE if the device
+ * does not expose its memory to the host (no large BAR) or TCPXU_VISIBLE_DEVICE_MEMORY=0; callers then simply go
+ * without.  Freed blocks are kept for later allocations and are not returned to the driver.  No counterpart in
+ * the reference, whose consumer (NCCL's kernel) always reads the mapped slot. */
+int tcpxuVisibleAlloc(int device, size_t bytes, void** host_ptr, void** dev_ptr);
+int tcpxuVisibleFree(int device, void* host_ptr);
+void tcpxuVisibleFlush(void); /* orders the host's writes to such memory before its later stores (sfence) */
+
 /* ---- (3) launch-per-batch unpack --------------------------------------------------------------------- */
 
 /* Scatter-gathers `n_descs` descriptors with one kernel launch on `stream` (a hipStream_t, NULL = the

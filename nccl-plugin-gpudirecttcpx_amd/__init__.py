@@ -114,6 +114,12 @@ _HIP_PROTOTYPES = {
         [ctypes.c_int, ctypes.c_size_t, ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_void_p)],
     ),
     "tcpxuMappedFree": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p]),
+    "tcpxuVisibleAlloc": (
+        ctypes.c_int,
+        [ctypes.c_int, ctypes.c_size_t, ctypes.POINTER(ctypes.c_void_p), ctypes.POINTER(ctypes.c_void_p)],
+    ),
+    "tcpxuVisibleFree": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p]),
+    "tcpxuVisibleFlush": (None, []),
     "tcpxuUnpackBatch": (
         ctypes.c_int,
         [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p],

@@ -559,6 +559,10 @@ struct tcpxuEngine {
   // hipHostFree waits for every stream of the device, so nothing may be freed while the kernel runs.
   void* stream_host = nullptr;
   void* stream_dev = nullptr;
+  // Device memory the host can write: a copy of the descriptors of small stream items (kStageDescs each), or null.
+  void* stage_host = nullptr;
+  void* stage_dev = nullptr;
+  bool stage_tried = false;
   std::mutex mu;
 };
 
@@ -724,6 +728,7 @@ int tcpxuEngineDestroy(tcpxuEngine* e) {
   if (e->st) (void)hipFree(e->st);
   if (e->ctl) (void)hipHostFree(e->ctl);
   if (e->stream_host) (void)hipHostFree(e->stream_host);
+  if (e->stage_host) (void)tcpxuVisibleFree(e->device, e->stage_host);
   delete e;
   return TCPXU_SUCCESS;
 }
@@ -803,6 +808,11 @@ int tcpxuEngineRunning(tcpxuEngine* e, int* running) {
   return TCPXU_SUCCESS;
 }
 
+// Descriptors of a stream item that are also copied into host-visible device memory, and the room per slot.
+constexpr uint32_t kStageDescs = 16;
+constexpr size_t kStageBytes = kStageDescs * sizeof(tcpxuLoadMeta);
+constexpr uint64_t kStageInFlight = 16;
+
 int tcpxuEngineStream(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_items, uint32_t depth,
                       uint32_t stall_timeout_ms, double* wall_us, double* latency_us) {
   return tcpxuEngineStreamWarm(e, items, n_items, 0, depth, stall_timeout_ms, wall_us, latency_us);
@@ -826,6 +836,12 @@ int tcpxuEngineStreamWarm(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t
   if (!e->stream_host)
     TCPXU_TRY(tcpxuMappedAlloc(e->device, flags_bytes + slot_bytes * TCPXU_STREAM_MAX_DEPTH, &e->stream_host,
                                &e->stream_dev));
+  if (!e->stage_tried) {
+    // Optional: without it every item's descriptors are read from the mapped slot.
+    e->stage_tried = true;
+    if (tcpxuVisibleAlloc(e->device, kStageBytes * TCPXU_STREAM_MAX_DEPTH, &e->stage_host, &e->stage_dev) != TCPXU_SUCCESS)
+      e->stage_host = e->stage_dev = nullptr;
+  }
   uint8_t* hb = static_cast<uint8_t*>(e->stream_host);
   uint8_t* db = static_cast<uint8_t*>(e->stream_dev);
   memset(hb, 0, flags_bytes);
@@ -860,6 +876,14 @@ int tcpxuEngineStreamWarm(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t
       published[slot] = clock::now();
       if (next_submit == warmup_items) t_begin = published[slot];
       const void* descs_dev = db + flags_bytes + slot_bytes * slot;
+      if (e->stage_host && it.n_descs != 0 && it.n_descs <= kStageDescs && next_submit - next_done < kStageInFlight) {
+        // A small request with few ahead of it: its descriptors also go into the GPU's own memory, ahead of the
+        // submission.  (With many in flight the request waits in queues anyway, and the write through the BAR with
+        // its flush, about 0.2 us of host time, would cap the rate at which one thread can publish.)
+        memcpy(static_cast<uint8_t*>(e->stage_host) + kStageBytes * slot, it.descs_host, sizeof(tcpxuLoadMeta) * it.n_descs);
+        tcpxuVisibleFlush();
+        descs_dev = static_cast<uint8_t*>(e->stage_dev) + kStageBytes * slot;
+      }
       rc = tcpxuEngineSubmit(e, it.bounce_base, it.dst_base, descs_dev, it.n_descs,
                              db + flag_stride * slot, next_submit + 1);
       if (rc == kTcpxuInProgress) {

@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <vector>
 
 #include "hip_common.h"
@@ -275,6 +276,69 @@ int tcpxuMappedFree(int device, void* host_ptr) {
   TCPXU_HIP(hipHostFree(host_ptr));
   return TCPXU_SUCCESS;
 }
+
+// ---- device memory that the host can write ------------------------------------------------------------------------
+// Fine-grained device memory is mapped for the host through the PCIe BAR where the whole of device memory is
+// exposed (large BAR).  Blocks are small and few, and they are handed back to a pool, never to the driver:
+// memory with non-default caching is not returned while the process lives.
+namespace {
+struct VisibleBlock {
+  void* ptr;
+  size_t bytes;
+  int device;
+  bool in_use;
+};
+std::mutex g_visible_mu;
+std::vector<VisibleBlock> g_visible;
+}  // namespace
+
+int tcpxuVisibleAlloc(int device, size_t bytes, void** host_ptr, void** dev_ptr) {
+  if (!host_ptr || !dev_ptr || bytes == 0 || bytes > (64u << 20)) return TCPXU_INVALID_ARGUMENT;
+  const char* sw = getenv("TCPXU_VISIBLE_DEVICE_MEMORY");
+  if (sw && *sw == '0') {
+    set_error("host-visible device memory is switched off (TCPXU_VISIBLE_DEVICE_MEMORY=0)");
+    return TCPXU_INVALID_USAGE;
+  }
+  TCPXU_TRY(use_device(device));
+  int large_bar = 0;
+  if (hipDeviceGetAttribute(&large_bar, hipDeviceAttributeIsLargeBar, device) != hipSuccess || !large_bar) {
+    set_error("device %d does not expose its memory to the host (no large BAR)", device);
+    return TCPXU_INVALID_USAGE;
+  }
+  bytes = (bytes + 4095) / 4096 * 4096;
+  std::lock_guard<std::mutex> lock(g_visible_mu);
+  void* p = nullptr;
+  for (auto& b : g_visible) {
+    if (!b.in_use && b.device == device && b.bytes == bytes) {
+      b.in_use = true;
+      p = b.ptr;
+      break;
+    }
+  }
+  if (!p) {
+    TCPXU_HIP(hipExtMallocWithFlags(&p, bytes, hipDeviceMallocFinegrained));
+    g_visible.push_back(VisibleBlock{p, bytes, device, true});
+  }
+  memset(p, 0, bytes);  // the first host access: through the BAR, write-combined
+  __builtin_ia32_sfence();
+  *host_ptr = p;
+  *dev_ptr = p;
+  return TCPXU_SUCCESS;
+}
+
+int tcpxuVisibleFree(int device, void* host_ptr) {
+  std::lock_guard<std::mutex> lock(g_visible_mu);
+  for (auto& b : g_visible) {
+    if (b.ptr == host_ptr && b.device == device && b.in_use) {
+      b.in_use = false;
+      return TCPXU_SUCCESS;
+    }
+  }
+  set_error("not a block of tcpxuVisibleAlloc on device %d", device);
+  return TCPXU_INVALID_ARGUMENT;
+}
+
+void tcpxuVisibleFlush(void) { __builtin_ia32_sfence(); }
 
 static int launch_batch(int device, const void* bounce_base, void* dst_base, const tcpxuLoadMeta* descs,
                         uint64_t n_descs, hipStream_t stream) {

@@ -54,6 +54,9 @@ const tcpxDeviceOps* default_device_ops() {
   ok &= bind(&g_hip_ops.engine_destroy, "tcpxuEngineDestroy");
   ok &= bind(&g_hip_ops.engine_submit, "tcpxuEngineSubmit");
   ok &= bind(&g_hip_ops.last_error, "tcpxuLastError");
+  ok &= bind(&g_hip_ops.visible_alloc, "tcpxuVisibleAlloc");
+  ok &= bind(&g_hip_ops.visible_free, "tcpxuVisibleFree");
+  ok &= bind(&g_hip_ops.visible_flush, "tcpxuVisibleFlush");
   if (!ok) {
     dlclose(g_hip_lib);
     g_hip_lib = nullptr;

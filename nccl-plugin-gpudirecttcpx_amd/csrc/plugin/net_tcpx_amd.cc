@@ -473,6 +473,7 @@ ncclResult_t tcpxFinalize(void) {
     for (QueueBlock& b : ds->free_blocks) {
       g.ops->mapped_free(d, b.meta);
       g.ops->device_free(d, b.dev_handle);
+      if (b.stage && g.ops->visible_free) g.ops->visible_free(d, b.stage);
     }
     ds->free_blocks.clear();
     if (ds->arena) g.ops->arena_destroy(d, ds->arena);
@@ -717,8 +718,18 @@ ncclResult_t tcpxTest(void* request, int* done, int* size) {
         std::atomic_thread_fence(std::memory_order_release);
         q->meta->done[r->slot.idx].value = 0;
         r->done_value = ++comm->done_seq;
-        const int rc = g.ops->engine_submit(comm->device->engine, comm->device->arena, r->data,
-                                            q->meta_dev->nccl.mem[r->slot.idx], static_cast<uint32_t>(r->slot.cnt_cache),
+        // The descriptors the engine reads: the mapped slot, or -- for a small request, of which a comm has at
+        // most 16 in flight -- a second copy in the GPU's own memory, written through the BAR ahead of the
+        // submission, which saves the GPU a PCIe round trip before it can start copying.
+        const void* descs_dev = q->meta_dev->nccl.mem[r->slot.idx];
+        if (q->stage && r->slot.cnt_cache <= kStagedDescs) {
+          union loadMeta* copy = q->stage + r->slot.idx * kStagedDescs;
+          memcpy(copy, r->slot.mem, sizeof(union loadMeta) * r->slot.cnt_cache);
+          g.ops->visible_flush();
+          descs_dev = q->stage_dev + r->slot.idx * kStagedDescs;
+        }
+        const int rc = g.ops->engine_submit(comm->device->engine, comm->device->arena, r->data, descs_dev,
+                                            static_cast<uint32_t>(r->slot.cnt_cache),
                                             &q->meta_dev->done[r->slot.idx].value, r->done_value);
         if (rc == TCPXU_IN_PROGRESS) {  // submission ring full: try again at the next poll
           --comm->done_seq;

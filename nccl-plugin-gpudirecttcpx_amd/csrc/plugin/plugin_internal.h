@@ -120,6 +120,8 @@ struct UnpackQueue {  // struct tcpxNetDeviceQueue, src/devcomm/unpack_defs1.h:5
   QueueMeta* meta = nullptr;      // host address
   QueueMeta* meta_dev = nullptr;  // device alias
   struct unpackNetDeviceHandle* dev_handle = nullptr;  // device memory
+  union loadMeta* stage = nullptr;      // see QueueBlock
+  union loadMeta* stage_dev = nullptr;
   uint64_t head = 0, tail = 0;
   int dev = 0;
   QueueRecord record;
@@ -281,7 +283,12 @@ struct QueueBlock {  // mapped metadata + device handle, recycled between comms 
   QueueMeta* meta;
   QueueMeta* meta_dev;
   struct unpackNetDeviceHandle* dev_handle;
+  // Device memory the host can write, kQueueDepth x kStagedDescs descriptors, or null: where the descriptors of a
+  // small request are copied to as well, so that the GPU need not fetch them over PCIe.
+  union loadMeta* stage;
+  union loadMeta* stage_dev;
 };
+constexpr uint32_t kStagedDescs = 16;
 
 struct DeviceState {
   int dev = 0;

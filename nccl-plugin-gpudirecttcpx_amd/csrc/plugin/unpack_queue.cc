@@ -28,13 +28,21 @@ ncclResult_t unpack_queue_new(int dev, bool passive, UnpackQueue** queue) {
       delete q;
       return rc;
     }
+    void *sh = nullptr, *sd = nullptr;
+    if (!g.ops->visible_alloc || !g.ops->visible_flush ||
+        g.ops->visible_alloc(dev, sizeof(union loadMeta) * kStagedDescs * kQueueDepth, &sh, &sd) != TCPXU_SUCCESS) {
+      sh = sd = nullptr;  // optional: every request's descriptors are then read from the mapped slot
+    }
     blk = QueueBlock{static_cast<QueueMeta*>(h), static_cast<QueueMeta*>(d),
-                     static_cast<struct unpackNetDeviceHandle*>(dh)};
+                     static_cast<struct unpackNetDeviceHandle*>(dh), static_cast<union loadMeta*>(sh),
+                     static_cast<union loadMeta*>(sd)};
   }
   memset(blk.meta, 0, sizeof(QueueMeta));
   q->meta = blk.meta;
   q->meta_dev = blk.meta_dev;
   q->dev_handle = blk.dev_handle;
+  q->stage = blk.stage;
+  q->stage_dev = blk.stage_dev;
   // Device-side handle {meta, bounce_buf, head}; head starts at -1 because NCCL's consumer increments it before
   // it copies (src/devcomm/nccl/unpack1.cu:54-63).  Only the receiving side knows a bounce buffer.
   struct unpackNetDeviceHandle hd;
@@ -56,7 +64,7 @@ void unpack_queue_free(UnpackQueue* q) {
   // stream of the device when it frees), so the block goes back to the device's pool; tcpxFinalize releases it.
   DeviceState* ds = &g.devices[q->dev];
   std::lock_guard<std::mutex> lock(ds->mu);
-  ds->free_blocks.push_back(QueueBlock{q->meta, q->meta_dev, q->dev_handle});
+  ds->free_blocks.push_back(QueueBlock{q->meta, q->meta_dev, q->dev_handle, q->stage, q->stage_dev});
   delete q;
 }
 

@@ -40,6 +40,13 @@ static int g_n_pending = 0;
 static int g_hold = 0;
 static int g_ring_full = 0;
 static uint64_t g_submitted = 0, g_mapped_live = 0, g_device_live = 0, g_arenas_live = 0, g_engine_starts = 0;
+/* "Device memory that the host can write": host memory here; the blocks are remembered so that a submission whose
+ * descriptors lie in one can be counted. */
+#define EMU_MAX_VISIBLE 256
+static struct { uint8_t* p; size_t bytes; } g_visible[EMU_MAX_VISIBLE];
+static uint64_t g_visible_live = 0, g_staged_submits = 0, g_visible_flushes = 0;
+static int g_visible_off = 0;
+static int in_visible(const void* p);
 
 static void run_job(const emu_job* j) {
   if (j->n) tcpx_oracle_unpack((uint8_t*)j->dst, (const uint8_t*)j->bounce, (const tcpx_oracle_desc*)j->descs, j->n);
@@ -49,6 +56,7 @@ static void run_job(const emu_job* j) {
 /* ---- test controls -------------------------------------------------------------------------------------------- */
 void emu_set_hold(int hold) { g_hold = hold; }
 void emu_set_ring_full(int full) { g_ring_full = full; }
+void emu_set_visible_off(int off) { g_visible_off = off; } /* allocations of host-visible device memory fail */
 int emu_pending(void) { return g_n_pending; }
 int emu_release(int n) { /* completes the n oldest held submissions; returns how many were completed */
   int done = 0;
@@ -67,6 +75,9 @@ uint64_t emu_counter(int which) {
     case 2: return g_device_live;
     case 3: return g_arenas_live;
     case 4: return g_engine_starts;
+    case 5: return g_visible_live;
+    case 6: return g_staged_submits;
+    case 7: return g_visible_flushes;
     default: return 0;
   }
 }
@@ -109,6 +120,7 @@ static int emu_engine_submit(tcpxuEngine* e, const void* bounce, void* dst, cons
   if (!e->started) return 5;
   if (g_ring_full) return TCPXU_IN_PROGRESS;
   ++g_submitted;
+  if (in_visible(descs)) ++g_staged_submits;
   emu_job j = {bounce, dst, descs, n, (uint64_t*)flag, value};
   if (g_hold) {
     if (g_n_pending >= EMU_MAX_PENDING) return TCPXU_IN_PROGRESS;
@@ -119,10 +131,44 @@ static int emu_engine_submit(tcpxuEngine* e, const void* bounce, void* dst, cons
   return 0;
 }
 static const char* emu_last_error(void) { return "emulated device"; }
+static int emu_visible_alloc(int dev, size_t bytes, void** host_ptr, void** dev_ptr) {
+  (void)dev;
+  if (g_visible_off) return TCPXU_INVALID_USAGE;
+  for (int i = 0; i < EMU_MAX_VISIBLE; ++i) {
+    if (!g_visible[i].p) {
+      g_visible[i].p = (uint8_t*)calloc(1, bytes);
+      if (!g_visible[i].p) return TCPXU_SYSTEM_ERROR;
+      g_visible[i].bytes = bytes;
+      ++g_visible_live;
+      *host_ptr = *dev_ptr = g_visible[i].p;
+      return 0;
+    }
+  }
+  return TCPXU_SYSTEM_ERROR;
+}
+static int emu_visible_free(int dev, void* host_ptr) {
+  (void)dev;
+  for (int i = 0; i < EMU_MAX_VISIBLE; ++i) {
+    if (g_visible[i].p && g_visible[i].p == host_ptr) {
+      free(g_visible[i].p);
+      g_visible[i].p = NULL;
+      --g_visible_live;
+      return 0;
+    }
+  }
+  return TCPXU_INVALID_ARGUMENT;
+}
+static void emu_visible_flush(void) { ++g_visible_flushes; }
+static int in_visible(const void* p) {
+  for (int i = 0; i < EMU_MAX_VISIBLE; ++i)
+    if (g_visible[i].p && (const uint8_t*)p >= g_visible[i].p && (const uint8_t*)p < g_visible[i].p + g_visible[i].bytes) return 1;
+  return 0;
+}
 
 static const tcpxDeviceOps g_ops = {
     emu_device_count, emu_arena_create,  emu_arena_destroy, emu_mapped_alloc,  emu_mapped_free,
     emu_device_alloc, emu_device_free,   emu_copy_to_device, emu_engine_create, emu_engine_start,
     emu_engine_stop,  emu_engine_destroy, emu_engine_submit, emu_last_error,
+    emu_visible_alloc, emu_visible_free, emu_visible_flush,
 };
 const tcpxDeviceOps* emu_ops(void) { return &g_ops; }

@@ -13,7 +13,9 @@ EMU_LIB = os.path.join(EMU_DIR, "libemu.so")
 def build_emu():
     src = os.path.join(EMU_DIR, "emu_device_ops.c")
     oracle_src = os.path.join(ROOT, "oracle", "tcpx_oracle.c")
-    if os.path.exists(EMU_LIB) and os.path.getmtime(EMU_LIB) >= max(os.path.getmtime(src), os.path.getmtime(oracle_src)):
+    inc = os.path.join(ROOT, "include")
+    deps = [src, oracle_src] + [os.path.join(inc, f) for f in os.listdir(inc) if f.endswith(".h")]  # the ops table lives in a header
+    if os.path.exists(EMU_LIB) and os.path.getmtime(EMU_LIB) >= max(os.path.getmtime(d) for d in deps):
         return
     subprocess.check_call(
         ["gcc", "-O1", "-g", "-fPIC", "-shared", "-Wall", "-I" + os.path.join(ROOT, "include"), "-o", EMU_LIB, src, oracle_src, "-pthread"]
@@ -29,6 +31,7 @@ def load_emu():
     lib.emu_pending.restype = ctypes.c_int
     lib.emu_set_hold.argtypes = [ctypes.c_int]
     lib.emu_set_ring_full.argtypes = [ctypes.c_int]
+    lib.emu_set_visible_off.argtypes = [ctypes.c_int]
     lib.emu_counter.restype = ctypes.c_uint64
     lib.emu_counter.argtypes = [ctypes.c_int]
     return lib

@@ -44,6 +44,7 @@ def env(pkg):
     yield e
     assert lib.tcpxFinalize() == 0
     assert emu.emu_counter(1) == 0 and emu.emu_counter(2) == 0 and emu.emu_counter(3) == 0, "finalize leaked"
+    assert emu.emu_counter(5) == 0, "finalize leaked host-visible device memory"
     lib.tcpxSetFailStopForTesting(1)
     assert lib.tcpxSetDeviceOpsForTesting(None) == 0
 
@@ -135,6 +136,35 @@ def test_native_driver_gives_the_same_bytes(env, comm, config, shrink):
     assert head == tail == len(wl.requests)
     assert env.lib.tcpxSynthRunRequests(comm.comm, None, None, 0, ptr, 64, 8, 1000, None, None) == INVALID_ARGUMENT
     assert env.lib.tcpxSynthRunRequests(comm.comm, ptr, ptr, 0, ptr, 64, 17, 1000, None, None) == INVALID_ARGUMENT
+
+
+def test_small_requests_hand_over_a_second_copy_of_their_descriptors(env, comm):
+    """A request of at most 16 descriptors is submitted with its descriptors in host-visible device memory (copied
+    there and flushed before the submission); a longer one with the mapped slot.  Either way the bytes are right,
+    and a comm whose device offers no such memory works the same."""
+    wl = env.pkg.Workload(3, seed=0x57A6, shrink=6)  # requests of 16 fragments
+    big = env.pkg.Workload(2, seed=0x57A7, shrink=2)  # requests of hundreds
+    for workload, staged in ((wl, True), (big, False)):
+        pool = fill_arena(env, workload)
+        buf, ptr = host_buffer(int(workload.info.dst_bytes))
+        before = [env.emu.emu_counter(i) for i in (0, 6, 7)]
+        env.driver.run_workload(comm, workload, ptr, n_flows=4, window=8)
+        after = [env.emu.emu_counter(i) for i in (0, 6, 7)]
+        assert np.array_equal(buf, expected_bytes(pool, workload.frags, workload.requests, int(workload.info.dst_bytes)))
+        submitted, in_visible, flushes = (a - b for a, b in zip(after, before))
+        assert submitted == len(workload.requests)
+        assert (in_visible, flushes) == ((submitted, submitted) if staged else (0, 0))
+    env.emu.emu_set_visible_off(1)
+    try:
+        c2 = env.driver.RecvComm(0)
+        pool = fill_arena(env, wl)
+        buf, ptr = host_buffer(int(wl.info.dst_bytes))
+        # (a comm that takes a recycled queue block keeps that block's copy area; a new block gets none)
+        env.driver.run_workload(c2, wl, ptr, n_flows=4, window=8)
+        assert np.array_equal(buf, expected_bytes(pool, wl.frags, wl.requests, int(wl.info.dst_bytes)))
+        c2.close()
+    finally:
+        env.emu.emu_set_visible_off(0)
 
 
 def test_partial_recvmsg_and_window_one(env, comm):

@@ -218,3 +218,34 @@ def test_batch_launches_replayed_from_a_hip_graph(pkg, hip, oracle):
         expect = oracle_expected(oracle, pool, descs, dst_bytes, 0)
         got = g.result()
         assert first_difference(got, expect) is None, "replay %d, first (index, got, want, count): %r" % (replay, first_difference(got, expect))
+
+
+def test_descriptors_in_host_visible_device_memory(pkg, hip, oracle):
+    """tcpxuVisibleAlloc: the host writes descriptors straight into device memory (through the BAR), flushes, and
+    a kernel launched afterwards reads them there; a freed block is handed out again; bad arguments are refused."""
+    wl = pkg.Workload(5, seed=0x715, shrink=5)
+    pool = np.empty(wl.info.pool_bytes, dtype=np.uint8)
+    wl.fill_window(0, pool)
+    descs = np.ascontiguousarray(wl.descs)
+    g = GpuBuffers(pool, descs[:0], wl.info.dst_bytes, wl.info.dst_misalign)
+    host, dev = ctypes.c_void_p(), ctypes.c_void_p()
+    rc = hip.tcpxuVisibleAlloc(0, descs.nbytes, ctypes.byref(host), ctypes.byref(dev))
+    if rc == pkg.INVALID_USAGE:
+        pytest.skip("this device does not expose its memory to the host: " + hip.tcpxuLastError().decode())
+    pkg.check(rc, "tcpxuVisibleAlloc")
+    print("visible-memory case: %d descriptors" % len(descs), flush=True)
+    ctypes.memmove(host.value, descs.ctypes.data, descs.nbytes)
+    hip.tcpxuVisibleFlush()
+    pkg.check(hip.tcpxuUnpackBatch(0, g.pool.data_ptr(), g.dst_base, dev, len(descs), None), "tcpxuUnpackBatch")
+    pkg.check(hip.tcpxuDeviceSynchronize(0), "sync")
+    expect = oracle_expected(oracle, pool, descs, wl.info.dst_bytes, wl.info.dst_misalign)
+    got = g.result()
+    assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
+    pkg.check(hip.tcpxuVisibleFree(0, host), "tcpxuVisibleFree")
+    assert hip.tcpxuVisibleFree(0, host) == pkg.INVALID_ARGUMENT  # not handed out any more
+    again_h, again_d = ctypes.c_void_p(), ctypes.c_void_p()
+    pkg.check(hip.tcpxuVisibleAlloc(0, descs.nbytes, ctypes.byref(again_h), ctypes.byref(again_d)), "tcpxuVisibleAlloc")
+    assert again_h.value == host.value  # blocks are kept and reused, not returned to the driver
+    pkg.check(hip.tcpxuVisibleFree(0, again_h), "tcpxuVisibleFree")
+    assert hip.tcpxuVisibleAlloc(0, 0, ctypes.byref(host), ctypes.byref(dev)) == pkg.INVALID_ARGUMENT
+    assert hip.tcpxuVisibleAlloc(0, 65 << 20, ctypes.byref(host), ctypes.byref(dev)) == pkg.INVALID_ARGUMENT
