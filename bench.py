@@ -359,6 +359,11 @@ def main():
         "parity_ok": parity_ok,
         "timed_region_s": round(t1 - t0, 4),
     }
+    if args.steps < 500:
+        # A step is 3 us of GPU work and a request's way through the engine about 10 us: a short run measures the
+        # filling and draining of the queues, not the rate.
+        result["note"] = "only %d steps (%.0f MiB): dominated by pipeline fill and drain; the default is 4000 steps" % (
+            args.steps, args.steps * chunk_bytes / 2**20)
 
     if args.comms > 1 and not args.one_launch:
         # The same steps with one comm only: 16 slots (at most 64 MiB) in flight, a launch of its own.
