@@ -31,8 +31,8 @@ import numpy as np
 import __graft_entry__ as graft
 
 # HBM bytes moved per algorithmic byte (2 x fragment bytes) by unpack_engine_kernel on the headline workload:
-# hardware counters FETCH_SIZE (x1.99983, its reading for a copy kernel of known size) and WRITE_SIZE (x1.0),
-# 9121939 KiB + 9120367 KiB against 2 x 9011200 KiB over one launch of 1100 steps.
+# hardware counters FETCH_SIZE (x1.99986, its reading for a copy kernel of known size) and WRITE_SIZE (x1.0),
+# 9387077 KiB + 9385673 KiB against 2 x 9273344 KiB over one launch of 1132 steps.
 TRAFFIC_PER_ALGORITHMIC_BYTE = 1.0122
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 CHUNK_CONFIG = 2
@@ -278,36 +278,50 @@ def main():
     eff = pkg.EngineConfig()
     pkg.check(hip.tcpxuEngineGetConfig(engine, ctypes.byref(eff)), "tcpxuEngineGetConfig")
 
-    def run(items, depth, warmup_items=0, want_latency=False):
+    def run(items, depth, warmup_items=0, want_latency=False, timed_items=None):
+        """One launch of the engine over `items`.  With `timed_items`, the wall time is that of the timed items
+        from completion to completion (the items after them only keep the queues full); otherwise from the publish
+        of item `warmup_items` to the last completion."""
         wall, kern = ctypes.c_double(), ctypes.c_double()
         lat = (ctypes.c_double * len(items))() if want_latency else None
-        rc = hip.tcpxuEngineRunTimed(
-            engine, items, len(items), warmup_items, depth, 20000, ctypes.byref(wall), ctypes.byref(kern), lat
-        )
+        if timed_items is None:
+            rc = hip.tcpxuEngineRunTimed(
+                engine, items, len(items), warmup_items, depth, 20000, ctypes.byref(wall), ctypes.byref(kern), lat
+            )
+        else:
+            rc = hip.tcpxuEngineRunWindow(
+                engine, items, len(items), warmup_items, timed_items, depth, 20000, ctypes.byref(wall), ctypes.byref(kern), lat
+            )
         pkg.check(rc, "tcpxuEngineRunTimed")
         return wall.value, kern.value, (np.asarray(lat[:]) if want_latency else None)
 
     # ---- W warm-up steps, then exactly K timed steps, all inside ONE launch of the persistent kernel -------
-    # `value` is timed by the host over the K steps only (publish of the first timed slot -> last completion);
-    # the roofline is the kernel's: all W+K steps' bytes over the launch's duration from HIP events, which is
-    # also what a kernel trace of this command shows for the launch.
-    all_items = item_array(0, args.warmup + args.steps)
+    # `value` is timed by the host over the K steps only; the roofline is the kernel's: the bytes of every step
+    # in the launch over the launch's duration from HIP events, which is also what a kernel trace of this command
+    # shows for the launch.
+    # A tail of untimed steps (one queue's worth) follows the timed ones, so that the last timed steps finish in a
+    # full pipeline like the others; the K timed steps are clocked from the completion of the last warm-up step to
+    # the completion of the last timed step.
+    tail_steps = (args.comms * args.depth + slots_per_step - 1) // slots_per_step
+    all_items = item_array(0, args.warmup + args.steps + tail_steps)
     # An untimed launch first: brings the clocks up from idle and touches every page once.
     if not args.one_launch:
         run(item_array(0, max(args.warmup, 1)), args.comms * args.depth)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    wall_us, kernel_us, _ = run(all_items, args.comms * args.depth, warmup_items=args.warmup * slots_per_step)
+    wall_us, kernel_us, _ = run(
+        all_items, args.comms * args.depth, warmup_items=args.warmup * slots_per_step, timed_items=args.steps * slots_per_step
+    )
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     payload = float(sum(workloads[(args.warmup + s) % args.chunks].info.payload_bytes for s in range(args.steps)))
-    launch_payload = float(sum(workloads[s % args.chunks].info.payload_bytes for s in range(args.warmup + args.steps)))
+    launch_payload = float(sum(workloads[s % args.chunks].info.payload_bytes for s in range(args.warmup + args.steps + tail_steps)))
     value_gbps = payload / (wall_us * 1e-6) / 1e9
     achieved = 2.0 * launch_payload / (kernel_us * 1e-6) / 1e9
 
     # ---- parity spot check: the last chunk written must equal the oracle's bytes ---------------------------
     oracle = graft.load_oracle()
-    last = (args.warmup + args.steps - 1) % args.chunks
+    last = (args.warmup + args.steps + tail_steps - 1) % args.chunks
     expect = np.full(chunk_bytes, 0xA5, dtype=np.uint8)
     graft.oracle_unpack(oracle, expect, pool, np.ascontiguousarray(workloads[last].descs))
     got = dst_d[256 + last * chunk_bytes : 256 + (last + 1) * chunk_bytes].cpu().numpy()
@@ -350,10 +364,10 @@ def main():
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "traffic": round(2.0 * launch_payload * TRAFFIC_PER_ALGORITHMIC_BYTE),
             "traffic_source": "FETCH_SIZE and WRITE_SIZE of this kernel on this workload (two rocprofv3 --pmc runs, scaled by "
-            "the same counters on the plain copy kernel: x1.99983 and x1.0) came to %.4f x the algorithmic bytes; "
+            "the same counters on the plain copy kernel: x1.99986 and x1.0) came to %.4f x the algorithmic bytes; "
             "that ratio times bytes_per_launch" % TRAFFIC_PER_ALGORITHMIC_BYTE,
             "bytes_per_launch": 2.0 * launch_payload,
-            "steps_per_launch": args.warmup + args.steps,
+            "steps_per_launch": args.warmup + args.steps + tail_steps,
             "launch_us": round(kernel_us, 1),
         },
         "parity_ok": parity_ok,
@@ -367,7 +381,7 @@ def main():
 
     if args.comms > 1 and not args.one_launch:
         # The same steps with one comm only: 16 slots (at most 64 MiB) in flight, a launch of its own.
-        w1, k1, _ = run(all_items, args.depth, warmup_items=args.warmup * slots_per_step)
+        w1, k1, _ = run(all_items, args.depth, warmup_items=args.warmup * slots_per_step, timed_items=args.steps * slots_per_step)
         result["single_comm"] = {
             "value": round(payload / (w1 * 1e-6) / 1e9, 2),
             "unit": "GB/s",

@@ -202,6 +202,15 @@ int tcpxuEngineRunTimed(tcpxuEngine* engine, const tcpxuStreamItem* items, uint6
                         uint64_t warmup_items, uint32_t depth, uint32_t stall_timeout_ms, double* wall_us,
                         double* kernel_us, double* latency_us);
 
+/* Like tcpxuEngineRunTimed, but *wall_us covers items [first_timed, first_timed + n_timed) from completion to
+ * completion: the clock starts when item first_timed - 1 is seen completed (at the first publish if first_timed
+ * is 0) and stops when item first_timed + n_timed - 1 is; items after that keep the queues full while the timed
+ * ones finish.  This is the time the engine takes for n_timed items in steady state, however few they are;
+ * *kernel_us is the whole launch as before. */
+int tcpxuEngineRunWindow(tcpxuEngine* engine, const tcpxuStreamItem* items, uint64_t n_items, uint64_t first_timed,
+                         uint64_t n_timed, uint32_t depth, uint32_t stall_timeout_ms, double* wall_us,
+                         double* kernel_us, double* latency_us);
+
 #ifdef __cplusplus
 }
 #endif

@@ -210,6 +210,21 @@ _HIP_PROTOTYPES = {
             ctypes.POINTER(ctypes.c_double),
         ],
     ),
+    "tcpxuEngineRunWindow": (
+        ctypes.c_int,
+        [
+            ctypes.c_void_p,
+            ctypes.POINTER(StreamItem),
+            ctypes.c_uint64,
+            ctypes.c_uint64,
+            ctypes.c_uint64,
+            ctypes.c_uint32,
+            ctypes.c_uint32,
+            ctypes.POINTER(ctypes.c_double),
+            ctypes.POINTER(ctypes.c_double),
+            ctypes.POINTER(ctypes.c_double),
+        ],
+    ),
 }
 
 _SYNTH_PROTOTYPES = {

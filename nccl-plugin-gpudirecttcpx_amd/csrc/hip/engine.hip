@@ -818,9 +818,17 @@ int tcpxuEngineStream(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_i
   return tcpxuEngineStreamWarm(e, items, n_items, 0, depth, stall_timeout_ms, wall_us, latency_us);
 }
 
-int tcpxuEngineStreamWarm(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_items, uint64_t warmup_items,
-                          uint32_t depth, uint32_t stall_timeout_ms, double* wall_us, double* latency_us) {
+// The streaming loop.  The clock runs over items [first_timed, first_timed + n_timed): it stops when the last of
+// them is seen completed, and starts either at the publish of the first of them (`from_completion` false) or when
+// the item before them is seen completed (true: completion to completion, the time the engine takes for n_timed
+// items in a queue that was full before and, if more items follow, stays full after).
+static int stream_items(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_items, uint64_t first_timed,
+                        uint64_t n_timed, bool from_completion, uint32_t depth, uint32_t stall_timeout_ms,
+                        double* wall_us, double* latency_us) {
   if (!e || !items || !wall_us || depth == 0 || depth > TCPXU_STREAM_MAX_DEPTH) return TCPXU_INVALID_ARGUMENT;
+  if (first_timed > n_items || n_timed > n_items - first_timed) return TCPXU_INVALID_ARGUMENT;
+  const uint64_t warmup_items = first_timed;
+  const uint64_t last_timed = first_timed + n_timed;  // one past
   for (uint64_t i = 0; i < n_items; ++i) {
     if (items[i].n_descs > TCPXU_SLOT_PAGES) {
       set_error("stream item %llu has %u descriptors, a slot holds %d", static_cast<unsigned long long>(i),
@@ -862,8 +870,9 @@ int tcpxuEngineStreamWarm(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t
       const auto now = clock::now();
       if (latency_us)
         latency_us[next_done] = std::chrono::duration<double, std::micro>(now - published[slot]).count();
-      t_end = now;
       ++next_done;
+      if (from_completion && next_done == warmup_items) t_begin = now;
+      if (next_done <= last_timed) t_end = now;
       progress = true;
     }
     // Publish while a slot is free.
@@ -874,7 +883,7 @@ int tcpxuEngineStreamWarm(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t
       if (it.n_descs)
         memcpy(slot_host, it.descs_host, sizeof(tcpxuLoadMeta) * it.n_descs);
       published[slot] = clock::now();
-      if (next_submit == warmup_items) t_begin = published[slot];
+      if (next_submit == warmup_items && (!from_completion || warmup_items == 0)) t_begin = published[slot];
       const void* descs_dev = db + flags_bytes + slot_bytes * slot;
       if (e->stage_host && it.n_descs != 0 && it.n_descs <= kStageDescs && next_submit - next_done < kStageInFlight) {
         // A small request with few ahead of it: its descriptors also go into the GPU's own memory, ahead of the
@@ -910,6 +919,13 @@ int tcpxuEngineStreamWarm(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t
   return rc;
 }
 
+int tcpxuEngineStreamWarm(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_items, uint64_t warmup_items,
+                          uint32_t depth, uint32_t stall_timeout_ms, double* wall_us, double* latency_us) {
+  if (warmup_items > n_items) return TCPXU_INVALID_ARGUMENT;
+  return stream_items(e, items, n_items, warmup_items, n_items - warmup_items, false, depth, stall_timeout_ms, wall_us,
+                      latency_us);
+}
+
 int tcpxuEngineRunTimed(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_items, uint64_t warmup_items,
                         uint32_t depth, uint32_t stall_timeout_ms, double* wall_us, double* kernel_us,
                         double* latency_us) {
@@ -921,6 +937,20 @@ int tcpxuEngineRunTimed(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n
   }
   TCPXU_TRY(tcpxuEngineStart(e));
   const int rc = tcpxuEngineStreamWarm(e, items, n_items, warmup_items, depth, stall_timeout_ms, wall_us, latency_us);
+  const int rc_stop = tcpxuEngineStop(e, kernel_us);
+  return rc != TCPXU_SUCCESS ? rc : rc_stop;
+}
+
+int tcpxuEngineRunWindow(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_items, uint64_t first_timed,
+                         uint64_t n_timed, uint32_t depth, uint32_t stall_timeout_ms, double* wall_us,
+                         double* kernel_us, double* latency_us) {
+  if (!e || !kernel_us || n_timed == 0) return TCPXU_INVALID_ARGUMENT;
+  if (!e->stream_host) {
+    const size_t bytes = (64 + sizeof(tcpxuLoadMeta) * TCPXU_SLOT_PAGES) * TCPXU_STREAM_MAX_DEPTH;
+    TCPXU_TRY(tcpxuMappedAlloc(e->device, bytes, &e->stream_host, &e->stream_dev));
+  }
+  TCPXU_TRY(tcpxuEngineStart(e));
+  const int rc = stream_items(e, items, n_items, first_timed, n_timed, true, depth, stall_timeout_ms, wall_us, latency_us);
   const int rc_stop = tcpxuEngineStop(e, kernel_us);
   return rc != TCPXU_SUCCESS ? rc : rc_stop;
 }

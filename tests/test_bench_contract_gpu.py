@@ -26,7 +26,10 @@ def test_bench_prints_one_json_line_with_the_contract_fields():
     roof = r["roofline"]
     assert roof["bound"] == "hbm" and roof["peak"] == 8000.0 and roof["unit"] == "GB/s"
     assert abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-3 and roof["traffic"] >= roof["bytes_per_launch"]
-    assert abs(r["value"] * 1e9 * r["ms_per_step"] * 1e-3 * r["steps"] - roof["bytes_per_launch"] / 2 * 200 / 220) / (roof["bytes_per_launch"] / 2) < 0.02
+    # value x time of the timed steps = their payload = the launch's payload x timed steps / steps in the launch
+    assert roof["steps_per_launch"] >= 220
+    timed_payload = roof["bytes_per_launch"] / 2 * 200 / roof["steps_per_launch"]
+    assert abs(r["value"] * 1e9 * r["ms_per_step"] * 1e-3 * r["steps"] - timed_payload) / timed_payload < 0.02
     cpu = r["cpu_baseline"]
     assert cpu["kind"] == "port" and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["unit"] == "GB/s" and cpu["sample"]
     assert r["parity_ok"] is True
