@@ -408,3 +408,46 @@ def test_engine_storm_of_mixed_small_submissions(pkg, hip, oracle, depth):
     e.destroy()
     got = dst_d.cpu().numpy()
     assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
+
+
+def test_engine_run_window_times_the_middle_of_a_stream(pkg, hip, oracle):
+    """tcpxuEngineRunWindow: warm-up items, timed items and a tail in one launch; the clock covers the timed ones
+    from completion to completion, so it is shorter than the launch, and every item's bytes are the oracle's."""
+    import torch
+
+    chunks = [pkg.Workload(2, seed=0xA11 + c, shrink=2) for c in range(4)]
+    info0 = chunks[0].info
+    cb = int(info0.dst_bytes)
+    pool = np.empty(info0.pool_bytes, dtype=np.uint8)
+    chunks[0].fill_window(0, pool)
+    expect = np.full(GUARD + len(chunks) * cb + GUARD, SENTINEL, dtype=np.uint8)
+    for c, wl in enumerate(chunks):
+        expect[GUARD + c * cb : GUARD + (c + 1) * cb] = oracle_expected(oracle, pool, wl.descs, cb, 0)[GUARD : GUARD + cb]
+    pool_d = torch.from_numpy(pool).to("cuda:0")
+    dst_d = torch.full((expect.nbytes,), SENTINEL, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    keep, flat = [], []
+    for rep in range(3):
+        for c, wl in enumerate(chunks):
+            for r in wl.requests:
+                d = np.ascontiguousarray(wl.descs[int(r["first_desc"]) : int(r["first_desc"]) + int(r["n_descs"])])
+                keep.append(d)
+                flat.append((pool_d.data_ptr(), dst_d.data_ptr() + GUARD + c * cb, d.ctypes.data, len(d)))
+    items = (pkg.StreamItem * len(flat))()
+    for i, (b, d, p, n) in enumerate(flat):
+        items[i].bounce_base, items[i].dst_base, items[i].descs_host, items[i].n_descs = b, d, p, n
+    n = len(flat)
+    e = Engine(pkg, hip)
+    print("engine window case: items=%d" % n, flush=True)
+    wall, kern = ctypes.c_double(), ctypes.c_double()
+    lat = (ctypes.c_double * n)()
+    pkg.check(hip.tcpxuEngineRunWindow(e.h, items, n, n // 4, n // 2, 8, 20000, ctypes.byref(wall), ctypes.byref(kern), lat), "tcpxuEngineRunWindow")
+    assert e.completed() == n and 0 < wall.value < kern.value and min(lat) > 0
+    first = ctypes.c_double()
+    pkg.check(hip.tcpxuEngineRunWindow(e.h, items, n, 0, n, 8, 20000, ctypes.byref(first), ctypes.byref(kern), None), "tcpxuEngineRunWindow")
+    assert wall.value < first.value <= kern.value  # the whole stream takes longer than its middle half
+    assert hip.tcpxuEngineRunWindow(e.h, items, n, n // 2, n, 8, 1000, ctypes.byref(wall), ctypes.byref(kern), None) == pkg.INVALID_ARGUMENT
+    assert hip.tcpxuEngineRunWindow(e.h, items, n, 0, 0, 8, 1000, ctypes.byref(wall), ctypes.byref(kern), None) == pkg.INVALID_ARGUMENT
+    e.destroy()
+    got = dst_d.cpu().numpy()
+    assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
