@@ -50,6 +50,6 @@ def test_bench_extras_report_latency_and_the_storm_sweep():
     assert r["single_comm"]["value"] > 0 and r["plugin_path"]["payload_GBps"] > 0 and r["plain_copy_kernel"]["rw_GBps"] > 0
     assert sorted(r["other_configs"]) == ["config_1", "config_4", "config_5"]
     assert all(v["payload_GBps"] > 0 for v in r["other_configs"].values())
-    assert r["launch_per_batch_384MiB"]["kernel"] == "unpack_batch_kernel" and r["launch_per_batch_384MiB"]["rw_GBps"] > 0
+    assert r["launch_per_batch_1GiB"]["kernel"] == "unpack_batch_kernel" and r["launch_per_batch_1GiB"]["rw_GBps"] > 0
     yard = r["hbm_yardsticks"]
     assert yard["read_only_GBps"] > 0 and yard["write_only_GBps"] > 0 and yard["copy_bound_rw_GBps"] > 0
