@@ -100,16 +100,15 @@ __device__ __forceinline__ u32x4 extract16(u32x4 a, u32x4 b, uint32_t shift) {
 // One round of a wavefront's copy work: up to 4 KiB of 16-byte vectors with a 16-byte aligned destination, the
 // edge bytes of the fragment (a head and a tail of fewer than 16 bytes where the fragment keeps its own partial
 // lines), and the shared last line (eight vectors, each assembled from up to two sources).
-// Loading and storing are separate steps so that a wavefront can issue the loads of its next round before the
-// stores of the current one: the memory counter of gfx9 retires in issue order, so waiting for the older loads
-// leaves the younger ones in flight.
+// Loading and storing are separate steps, with an explicit wait for everything in flight between them.
 //
-// Nothing in a round is predicated.  A lane whose vector index is past the round's end is clamped to the last
-// vector for the load AND for the store: it re-reads and re-writes that vector with the very same bytes, which
-// changes nothing.  A lane without an edge byte copies the fragment's byte 0 onto itself the same way, and a
-// round without a shared line repeats its vector 0 in its place.  Every round therefore issues exactly the
-// same loads and stores on every path, which lets the compiler compute exact wait counts and keep the younger
-// round in flight.
+// Only the lanes that have something to move take part in a memory instruction, and a part of the round that
+// has nothing to move is skipped by the whole wavefront: the edge bytes where the fragment shares its first and
+// last line with its neighbours, the shared line where it does not, the extra dword where the source needs no
+// shifting.  (An earlier form issued the same eight loads and six stores in every round, with idle lanes
+// repeating a neighbour's access; at an 8 MiB chunk of 4 KiB fragments the four main vectors alone ran 5 % faster
+// than that.)
+constexpr uint32_t kNoEdge = 0xFFFFFFFFu;
 struct CopyRound {
   // Wave-uniform (scalar registers):
   const uint8_t* src_vec;   // source of vector 0 of this round (any alignment)
@@ -120,9 +119,10 @@ struct CopyRound {
   uint32_t nvec;            // vectors in this round, 1..kVecPerRound
   uint32_t frag_len;
   uint32_t line_off;        // offset of the shared last line from dst_frag
-  bool share_next;          // this wavefront completes its last line out of the next fragment
+  bool share_next;          // this round completes the fragment's last line out of the next fragment
+  bool has_edge;            // this round copies edge bytes (some lane has one)
   // Per lane:
-  uint32_t edge_off;        // offset of this lane's edge byte in the fragment, 0 if it has none
+  uint32_t edge_off;        // offset of this lane's edge byte in the fragment, kNoEdge if it has none
 };
 struct CopyRegs {
   u32x4 r[kVecPerLane];
@@ -130,43 +130,30 @@ struct CopyRegs {
   uint32_t tail_dword;
   uint32_t edge_byte;
 };
+constexpr uint32_t kLineVecs = kLineBytes / 16;  // lanes that take part in the shared line
 
-// Byte offset of lane's k-th vector in a round of nvec vectors, clamped to the last one.
-__device__ __forceinline__ uint32_t round_vec_offset(uint32_t nvec, int k, uint32_t lane) {
-  const uint32_t v = static_cast<uint32_t>(k) * kWaveLanes + lane;
-  const uint32_t last = nvec - 1;
-  return (v < last ? v : last) << 4;
-}
-
-// What a lane does for the shared last line: vector (lane & 7) of the line is bytes [shift, shift+16) of
-// A:B with A = 16 bytes at src_frag + off_a and B = 16 bytes at src_next + off_b.
+// What a lane below kLineVecs does for the shared last line: vector `lane` of the line is bytes [shift, shift+16)
+// of A:B with A = 16 bytes at src_frag + off_a and B = 16 bytes at src_next + off_b.
 struct LineLane {
   uint32_t off_a, off_b, shift, dst_off;
 };
 __device__ __forceinline__ LineLane line_lane(const CopyRound& c, uint32_t lane) {
   LineLane l;
-  if (c.share_next) {  // wave-uniform
-    const uint32_t x = c.line_off + ((lane & 7u) << 4);  // this vector's offset from the fragment's start
-    const int32_t own = static_cast<int32_t>(c.frag_len) - static_cast<int32_t>(x);  // bytes still in this fragment
-    l.dst_off = x;
-    if (own >= 16) {  // entirely this fragment
-      l.off_a = x;
-      l.off_b = 0;
-      l.shift = 0;
-    } else if (own <= 0) {  // entirely the next fragment
-      l.off_a = c.frag_len - 16u;
-      l.off_b = static_cast<uint32_t>(-own);
-      l.shift = 16;
-    } else {  // the last `own` bytes of this fragment, then the first bytes of the next
-      l.off_a = c.frag_len - 16u;
-      l.off_b = 0;
-      l.shift = 16u - static_cast<uint32_t>(own);
-    }
-  } else {  // repeat vector 0 of the round
-    l.dst_off = static_cast<uint32_t>(c.dst_vec - c.dst_frag);
-    l.off_a = l.dst_off;
-    l.off_b = l.dst_off;
+  const uint32_t x = c.line_off + ((lane & (kLineVecs - 1)) << 4);  // this vector's offset from the fragment's start
+  const int32_t own = static_cast<int32_t>(c.frag_len) - static_cast<int32_t>(x);  // bytes still in this fragment
+  l.dst_off = x;
+  if (own >= 16) {  // entirely this fragment
+    l.off_a = x;
+    l.off_b = 0;
     l.shift = 0;
+  } else if (own <= 0) {  // entirely the next fragment
+    l.off_a = c.frag_len - 16u;
+    l.off_b = static_cast<uint32_t>(-own);
+    l.shift = 16;
+  } else {  // the last `own` bytes of this fragment, then the first bytes of the next
+    l.off_a = c.frag_len - 16u;
+    l.off_b = 0;
+    l.shift = 16u - static_cast<uint32_t>(own);
   }
   return l;
 }
@@ -179,40 +166,58 @@ __device__ __forceinline__ LineLane line_lane(const CopyRound& c, uint32_t lane)
 // every vector of the round) and shifts the bytes into place in registers: a vector is bytes [skew, skew+16)
 // of its own four dwords plus one more dword, and that fifth dword is the first dword of the next vector --
 // which the neighbouring lane holds.  Only the round's last vector has no neighbour; its fifth dword comes
-// from one extra 4-byte load.
+// from one extra 4-byte load by lane 0 (with skew > 0 that dword starts inside the fragment, and an aligned dword
+// never leaves the 4 KiB page it starts in; with skew 0 nothing of it is used and it is not loaded).
 __device__ __forceinline__ uint32_t load_dword_sys(const uint8_t* p) {
   return __hip_atomic_load((const TCPXU_GLOBAL uint32_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 __device__ __forceinline__ void round_load(const CopyRound& c, CopyRegs& x, uint32_t lane) {
-  const LineLane l = line_lane(c, lane);
   const uint32_t skew = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(c.src_vec)) & 3u;
   const uint8_t* base4 = c.src_vec - skew;
-  x.edge_byte = load_byte_sys(c.src_frag + c.edge_off);
+  x.edge_byte = 0;
+  x.tail_dword = 0;
+  x.line_a = u32x4{0, 0, 0, 0};
+  x.line_b = u32x4{0, 0, 0, 0};
+  if (c.has_edge) {
+    if (c.edge_off != kNoEdge) x.edge_byte = load_byte_sys(c.src_frag + c.edge_off);
+  }
 #pragma unroll
-  for (int k = 0; k < kVecPerLane; ++k) x.r[k] = load_vec_sys(base4 + round_vec_offset(c.nvec, k, lane));
-  // The dword after the last vector's four.  With skew 0 nothing of it is used, and it may lie outside the
-  // fragment (even outside the arena), so the last vector's own last dword is read instead.  With skew > 0 it
-  // starts inside the fragment, and an aligned dword never leaves the 4 KiB page it starts in.
-  x.tail_dword = load_dword_sys(base4 + ((c.nvec - 1) << 4) + (skew != 0 ? 16u : 12u));
-  x.line_a = load_vec_sys(c.src_frag + l.off_a);
-  x.line_b = load_vec_sys(c.src_next + l.off_b);
+  for (int k = 0; k < kVecPerLane; ++k) {
+    x.r[k] = u32x4{0, 0, 0, 0};
+    const uint32_t v = static_cast<uint32_t>(k) * kWaveLanes + lane;
+    if (v < c.nvec) x.r[k] = load_vec_sys(base4 + (v << 4));
+  }
+  if (skew != 0) {
+    if (lane == 0) x.tail_dword = load_dword_sys(base4 + (c.nvec << 4));
+  }
+  if (c.share_next) {
+    if (lane < kLineVecs) {
+      const LineLane l = line_lane(c, lane);
+      x.line_a = load_vec_sys(c.src_frag + l.off_a);
+      x.line_b = load_vec_sys(c.src_next + l.off_b);
+    }
+  }
 }
 
-__device__ __forceinline__ void round_store(const CopyRound& c, CopyRegs& x, uint32_t lane) {
-  // Wait for every load of the round before the first store, rather than store each vector as soon as its own
-  // load has landed (what the compiler would arrange): the round's stores then leave back to back, which
-  // measured 2-3 % faster end to end.  The registers pass through the statement so that no use of them can be
-  // scheduled before it.
+// Waits for every load of the round (and for whatever else the wavefront has in flight) rather than let each
+// vector be stored as soon as its own load has landed (what the compiler would arrange): the round's stores then
+// leave back to back, which measured 2-3 % faster end to end.  The registers pass through the statement so that no
+// use of them can be scheduled before it.
+__device__ __forceinline__ void round_wait(CopyRegs& x) {
   asm volatile("s_waitcnt vmcnt(0)"
                : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.r[2]), "+v"(x.r[3]), "+v"(x.line_a), "+v"(x.line_b),
                  "+v"(x.tail_dword), "+v"(x.edge_byte)
                :
                : "memory");
   static_assert(kVecPerLane == 4, "the statement above names the four vectors of a round");
-  const LineLane l = line_lane(c, lane);
+}
+
+// Shifts the loaded bytes into place and stores them; the round's loads must have landed (round_wait).
+__device__ __forceinline__ void round_store_loaded(const CopyRound& c, CopyRegs& x, uint32_t lane) {
   const uint32_t skew = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(c.src_vec)) & 3u;
   const uint32_t last = c.nvec - 1;
+  const uint32_t tail_dword = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(x.tail_dword), 0));
 #pragma unroll
   for (int k = 0; k < kVecPerLane; ++k) {
     // First dword of the next vector: lane+1 of this register, or lane 0 of the next register for lane 63.
@@ -223,16 +228,28 @@ __device__ __forceinline__ void round_store(const CopyRound& c, CopyRegs& x, uin
       if (lane == 63u) next0 = wrap;
     }
     const uint32_t v = static_cast<uint32_t>(k) * kWaveLanes + lane;
-    const uint32_t w4 = v < last ? next0 : x.tail_dword;  // the last vector and its clamped repeats use the tail
+    const uint32_t w4 = v < last ? next0 : tail_dword;  // the last vector uses the extra dword
     u32x4 out;
     out[0] = __builtin_amdgcn_alignbyte(x.r[k][1], x.r[k][0], skew);
     out[1] = __builtin_amdgcn_alignbyte(x.r[k][2], x.r[k][1], skew);
     out[2] = __builtin_amdgcn_alignbyte(x.r[k][3], x.r[k][2], skew);
     out[3] = __builtin_amdgcn_alignbyte(w4, x.r[k][3], skew);
-    store_vec_stream(c.dst_vec + round_vec_offset(c.nvec, k, lane), out);
+    if (v < c.nvec) store_vec_stream(c.dst_vec + (v << 4), out);
   }
-  store_vec_stream(c.dst_frag + l.dst_off, extract16(x.line_a, x.line_b, l.shift));
-  store_byte_sys(c.dst_frag + c.edge_off, static_cast<uint8_t>(x.edge_byte));
+  if (c.share_next) {
+    if (lane < kLineVecs) {
+      const LineLane l = line_lane(c, lane);
+      store_vec_stream(c.dst_frag + l.dst_off, extract16(x.line_a, x.line_b, l.shift));
+    }
+  }
+  if (c.has_edge) {
+    if (c.edge_off != kNoEdge) store_byte_sys(c.dst_frag + c.edge_off, static_cast<uint8_t>(x.edge_byte));
+  }
+}
+
+__device__ __forceinline__ void round_store(const CopyRound& c, CopyRegs& x, uint32_t lane) {
+  round_wait(x);
+  round_store_loaded(c, x, lane);
 }
 
 // A fragment too short to contain one destination-aligned vector (at most 30 bytes) is copied byte per lane,
@@ -245,52 +262,75 @@ __device__ __forceinline__ void copy_tiny_fragment(const uint8_t* src, uint8_t* 
   if (lane < len) store_byte_sys(dst + lane, static_cast<uint8_t>(load_byte_sys(src + lane)));
 }
 
-// Splits a fragment that is not tiny (all arguments wave-uniform) into rounds of 1..kVecPerRound vectors.
-// Fragments of the wire format (at most 4 KiB) have exactly one round; later rounds of a longer fragment repeat
-// the edge bytes and the shared line with the same bytes.
+// Where the vectors of a fragment that is not tiny start and end.
 //   share_prev  the fragment's first partial line is written by the owner of the previous fragment
 //   share_next  this owner completes the fragment's last line from src_next, the next fragment's source
+struct FragmentPlan {
+  uint32_t start_off;  // offset of vector 0 from the fragment's first byte
+  uint32_t end_off;    // offset of the end of the last vector (where the shared last line starts, if there is one)
+  uint32_t head, tail; // edge bytes before vector 0 and after the last vector, each fewer than 16
+  uint32_t nvec;       // vectors in all, at least 1
+};
+__device__ __forceinline__ FragmentPlan plan_fragment(uint64_t dst_addr, uint32_t len, bool share_prev, bool share_next) {
+  FragmentPlan p;
+  p.head = 0;
+  if (share_prev) {
+    p.start_off = static_cast<uint32_t>(-dst_addr) & (kLineBytes - 1);
+  } else {
+    p.head = static_cast<uint32_t>(-dst_addr) & 15u;
+    p.start_off = p.head;
+  }
+  p.tail = 0;
+  if (share_next) {
+    p.end_off = len - (static_cast<uint32_t>(dst_addr + len) & (kLineBytes - 1));
+  } else {
+    p.end_off = p.start_off + ((len - p.start_off) & ~15u);
+    p.tail = len - p.end_off;
+  }
+  p.nvec = (p.end_off - p.start_off) >> 4;
+  return p;
+}
+// The first round of a planned fragment; *nvec_left receives the vectors that remain for later rounds.
+__device__ __forceinline__ CopyRound first_round_of(const uint8_t* src, uint8_t* dst, const uint8_t* src_next,
+                                                    uint32_t len, bool share_next, uint32_t start_off,
+                                                    uint32_t end_off, uint32_t head, uint32_t tail, uint32_t nvec,
+                                                    uint32_t lane, uint32_t* nvec_left) {
+  CopyRound c;
+  c.src_frag = src;
+  c.dst_frag = dst;
+  c.src_vec = src + start_off;
+  c.dst_vec = dst + start_off;
+  c.src_next = share_next ? src_next : src;
+  c.frag_len = len;
+  c.line_off = end_off;
+  c.share_next = share_next;
+  // Lanes [0,head) carry the head, lanes [16,16+tail) the tail (both < 16 bytes); the other lanes have none.
+  c.has_edge = (head | tail) != 0;
+  c.edge_off = kNoEdge;
+  if (lane < head) c.edge_off = lane;
+  else if (lane >= 16u && lane - 16u < tail) c.edge_off = end_off + (lane - 16u);
+  c.nvec = nvec < kVecPerRound ? nvec : kVecPerRound;
+  *nvec_left = nvec - c.nvec;
+  return c;
+}
+
+// Splits a fragment that is not tiny (all arguments wave-uniform) into rounds of 1..kVecPerRound vectors.
+// Fragments of the wire format (at most 4 KiB) have exactly one round; the first round of a longer fragment
+// copies its edge bytes and its shared line.
 struct FragmentRounds {
   uint32_t nvec_left = 0;  // vectors not yet handed out
 
   __device__ __forceinline__ CopyRound first_round(const uint8_t* src, uint8_t* dst, uint32_t len, bool share_prev,
                                                    bool share_next, const uint8_t* src_next, uint32_t lane) {
-    const uintptr_t d = reinterpret_cast<uintptr_t>(dst);
-    uint32_t head = 0, start_off;  // start_off: offset of vector 0 from dst
-    if (share_prev) {
-      start_off = static_cast<uint32_t>(-d) & (kLineBytes - 1);
-    } else {
-      head = static_cast<uint32_t>(-d) & 15u;
-      start_off = head;
-    }
-    uint32_t tail = 0, end_off;  // end_off: offset of the end of the last vector from dst
-    if (share_next) {
-      end_off = len - (static_cast<uint32_t>(d + len) & (kLineBytes - 1));
-    } else {
-      end_off = start_off + ((len - start_off) & ~15u);
-      tail = len - end_off;
-    }
-    const uint32_t nvec = (end_off - start_off) >> 4;
-    CopyRound c;
-    c.src_frag = src;
-    c.dst_frag = dst;
-    c.src_vec = src + start_off;
-    c.dst_vec = dst + start_off;
-    c.src_next = share_next ? src_next : src;
-    c.frag_len = len;
-    c.line_off = end_off;
-    c.share_next = share_next;
-    // Lanes [0,head) carry the head, lanes [16,16+tail) the tail (both < 16 bytes); every other lane gets 0.
-    c.edge_off = 0;
-    if (lane < head) c.edge_off = lane;
-    else if (lane >= 16u && lane - 16u < tail) c.edge_off = end_off + (lane - 16u);
-    c.nvec = nvec < kVecPerRound ? nvec : kVecPerRound;
-    nvec_left = nvec - c.nvec;
-    return c;
+    const FragmentPlan p = plan_fragment(reinterpret_cast<uintptr_t>(dst), len, share_prev, share_next);
+    return first_round_of(src, dst, src_next, len, share_next, p.start_off, p.end_off, p.head, p.tail, p.nvec, lane,
+                          &nvec_left);
   }
   __device__ __forceinline__ bool more() const { return nvec_left != 0; }
   __device__ __forceinline__ CopyRound next_round(const CopyRound& prev) {
     CopyRound c = prev;
+    c.has_edge = false;  // the first round has copied the edge bytes and the shared line
+    c.share_next = false;
     c.src_vec = prev.src_vec + (static_cast<size_t>(prev.nvec) << 4);
     c.dst_vec = prev.dst_vec + (static_cast<size_t>(prev.nvec) << 4);
     c.nvec = nvec_left < kVecPerRound ? nvec_left : kVecPerRound;
@@ -299,39 +339,48 @@ struct FragmentRounds {
   }
 };
 
-// Copies descriptors first, first + stride, ... < end of a descriptor list of n staged in LDS with the calling
-// wavefront; neighbours in the list (whoever copies them) decide which destination lines are shared.  One round (at most 4 KiB) is in
-// flight per wavefront: keeping a second register set to overlap the next round's loads with this round's
-// stores measured slower, because fewer wavefronts then fit on a compute unit.  `bounce` and `dst` must be
-// wave-uniform.
-// `on_last_fragment()` is called exactly once, when the wavefront turns to the last descriptor of its share (at
-// once if it has none): a caller that feeds the wavefront can use it to start fetching more work.
-template <typename OnLastFragment>
-__device__ __forceinline__ void wave_copy_descriptors(const tcpxuLoadMeta* descs, uint32_t n, uint32_t first,
-                                                      uint32_t stride, uint32_t end, const uint8_t* bounce,
-                                                      uint8_t* dst, uint32_t lane,
-                                                      OnLastFragment&& on_last_fragment) {
-  // Everything that describes a fragment is wave-uniform; saying so keeps it in scalar registers and leaves
-  // the vector registers to the payload in flight.
-  auto uniform = [](uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(v)); };
-  auto uniform64 = [&](uint64_t v) {
-    return (static_cast<uint64_t>(uniform(static_cast<uint32_t>(v >> 32))) << 32) | uniform(static_cast<uint32_t>(v));
-  };
-  const uint64_t dst_addr = reinterpret_cast<uint64_t>(dst);
-  uint32_t j = uniform(first);
-  end = uniform(end);
-  if (j >= end) on_last_fragment();
+// A wavefront's position in its share of a descriptor list staged in LDS: descriptors j, j + stride, ... < end of
+// a list of n.  Neighbours in the list (whoever copies them) decide which destination lines are shared.
+// Everything that describes a fragment is wave-uniform; saying so keeps it in scalar registers and leaves the
+// vector registers to the payload in flight.  `bounce` and `dst` must be wave-uniform.
+struct ShareCursor {
+  const tcpxuLoadMeta* descs;
+  uint32_t n, j, end, stride;
+  const uint8_t* bounce;
+  uint8_t* dst;
   FragmentRounds fr;
-  // Next round of this wavefront's work, or false when there is none.  `prev` is the round before it.
-  auto produce = [&](CopyRound& out, const CopyRound& prev) -> bool {
+
+  static __device__ __forceinline__ uint32_t uniform(uint32_t v) {
+    return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(v));
+  }
+  static __device__ __forceinline__ uint64_t uniform64(uint64_t v) {
+    return (static_cast<uint64_t>(uniform(static_cast<uint32_t>(v >> 32))) << 32) | uniform(static_cast<uint32_t>(v));
+  }
+  __device__ __forceinline__ void open(const tcpxuLoadMeta* list, uint32_t count, uint32_t first, uint32_t step,
+                                       uint32_t stop, const uint8_t* bounce_base, uint8_t* dst_base) {
+    descs = list;
+    n = count;
+    j = uniform(first);
+    end = uniform(stop);
+    stride = step;
+    bounce = bounce_base;
+    dst = dst_base;
+    fr.nvec_left = 0;
+  }
+  // Next round of the share, or false when there is none.  `prev` is the round before it (read only while a
+  // fragment longer than one round is being continued).  `on_take()` runs after each descriptor has been taken
+  // off the share, with j already advanced.  Fragments too short for a round are copied here, at once.
+  template <typename OnTake>
+  __device__ __forceinline__ bool produce(CopyRound& out, const CopyRound& prev, uint32_t lane, OnTake&& on_take) {
     if (fr.more()) {
       out = fr.next_round(prev);
       return true;
     }
+    const uint64_t dst_addr = reinterpret_cast<uint64_t>(dst);
     while (j < end) {
       const uint32_t cur = j;
       j += stride;
-      if (j >= end) on_last_fragment();
+      on_take();
       const tcpxuLoadMeta d = descs[cur];
       const uint32_t len = uniform(d.len);
       if (len == 0) continue;
@@ -358,15 +407,32 @@ __device__ __forceinline__ void wave_copy_descriptors(const tcpxuLoadMeta* descs
       return true;
     }
     return false;
+  }
+};
+
+// Copies descriptors first, first + stride, ... < end of a descriptor list of n staged in LDS with the calling
+// wavefront, one round (at most 4 KiB) in flight at a time.
+// `on_last_fragment()` is called exactly once, when the wavefront turns to the last descriptor of its share (at
+// once if it has none): a caller that feeds the wavefront can use it to start fetching more work.
+template <typename OnLastFragment>
+__device__ __forceinline__ void wave_copy_descriptors(const tcpxuLoadMeta* descs, uint32_t n, uint32_t first,
+                                                      uint32_t stride, uint32_t end, const uint8_t* bounce,
+                                                      uint8_t* dst, uint32_t lane,
+                                                      OnLastFragment&& on_last_fragment) {
+  ShareCursor cursor;
+  cursor.open(descs, n, first, stride, end, bounce, dst);
+  if (cursor.j >= cursor.end) on_last_fragment();
+  auto on_take = [&] {
+    if (cursor.j >= cursor.end) on_last_fragment();
   };
   CopyRound r;
   CopyRegs x;
-  if (!produce(r, r)) return;
+  if (!cursor.produce(r, r, lane, on_take)) return;
   for (;;) {
     round_load(r, x, lane);
     round_store(r, x, lane);
     CopyRound nxt;
-    if (!produce(nxt, r)) return;
+    if (!cursor.produce(nxt, r, lane, on_take)) return;
     r = nxt;
   }
 }
