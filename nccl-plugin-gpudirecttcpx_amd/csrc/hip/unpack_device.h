@@ -124,6 +124,7 @@ struct CopyRound {
   // Per lane:
   uint32_t edge_off;        // offset of this lane's edge byte in the fragment, kNoEdge if it has none
 };
+constexpr int kDppWaveShiftLeft1 = 0x130;  // lane i receives lane i+1's value; lane 63 keeps the first operand
 struct CopyRegs {
   u32x4 r[kVecPerLane];
   u32x4 line_a, line_b;
@@ -221,8 +222,9 @@ __device__ __forceinline__ void round_store_loaded(const CopyRound& c, CopyRegs&
 #pragma unroll
   for (int k = 0; k < kVecPerLane; ++k) {
     // First dword of the next vector: lane+1 of this register, or lane 0 of the next register for lane 63.
+    // (a DPP wavefront shift: one vector instruction, no trip through the LDS crossbar)
     uint32_t next0 = static_cast<uint32_t>(
-        __builtin_amdgcn_ds_bpermute(static_cast<int>(((lane + 1u) & 63u) << 2), static_cast<int>(x.r[k][0])));
+        __builtin_amdgcn_update_dpp(0, static_cast<int>(x.r[k][0]), kDppWaveShiftLeft1, 0xF, 0xF, false));
     if (k + 1 < kVecPerLane) {
       const uint32_t wrap = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(x.r[k + 1 < kVecPerLane ? k + 1 : k][0]), 0));
       if (lane == 63u) next0 = wrap;
