@@ -170,7 +170,10 @@ void batch_geometry(int device, uint64_t n_descs, uint32_t* descs_per_wg, uint64
   dpw = std::min(std::max(dpw, 1u), kMaxDescsPerWg);
   const uint64_t batches = (n_descs + dpw - 1) / dpw;
   const uint64_t per_xcd = (batches + 7) / 8;
-  const uint64_t max_grid = cus * 16;
+  // One batch per workgroup up to 128 workgroups per compute unit; beyond that workgroups take several batches in
+  // turn.  Letting the dispatcher hand out batches balances the compute units better than a grid that just fills
+  // them and strides (1 GiB of 4 KiB fragments: 5.34 against 5.09 TB/s r+w with 16 workgroups per compute unit).
+  const uint64_t max_grid = cus * static_cast<uint64_t>(std::max(1, env_int("TCPXU_BATCH_WGS_PER_CU", 128)));
   *descs_per_wg = dpw;
   *n_batches = batches;
   *grid = static_cast<uint32_t>(std::min<uint64_t>(per_xcd * 8, std::max<uint64_t>(max_grid, 8)));
