@@ -114,6 +114,13 @@ def test_long_descriptor_beyond_one_page(pkg, hip, oracle):
     pool = seeded_pool(1 << 20, 5)
     rows = [(3, 70001, 5), (100000, 8192, 80000), (200001, 4097, 90001)]
     run_batch(pkg, hip, oracle, pool, make_descs(rows), 100000)
+    # Long fragments that continue each other in the destination with boundaries inside 128-byte lines: several
+    # rounds each, and the line at every boundary is completed by the owner of the fragment before it.
+    rows, dst = [], 7
+    for src, ln in [(11, 10001), (300002, 9000), (500003, 4097 + 4096), (700000, 300), (800005, 20000), (900001, 4096)]:
+        rows.append((src, ln, dst))
+        dst += ln
+    run_batch(pkg, hip, oracle, pool, make_descs(rows), dst + 64)
 
 
 def test_descriptors_in_mapped_host_memory(pkg, hip, oracle):
