@@ -343,12 +343,31 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
 constexpr uint32_t kCopyWaves = TCPXU_ENGINE_COPY_WAVES;
 constexpr uint32_t kEngineThreads = (kCopyWaves + 1) * kWaveLanes;
 
+// What a copy wavefront needs to know about one fragment, worked out by the fetcher: one descriptor per lane, all
+// 8..32 of a ticket at once, instead of by each copy wavefront from three descriptors per fragment.
+constexpr uint32_t kRecSkip = 0, kRecTiny = 1, kRecRounds = 2;
+struct alignas(16) RoundRec {
+  uint32_t src_lo, src_hi;     // the fragment's first byte
+  uint32_t dst_lo, dst_hi;
+  uint32_t next_lo, next_hi;   // the next fragment's first source byte (read only if the last line is shared)
+  uint32_t start_off, end_off; // FragmentPlan
+  uint32_t len;
+  uint32_t nvec;
+  uint32_t bits;               // head | tail << 8 | share_next << 16 | kind << 24
+  uint32_t pad;
+};
+static_assert(sizeof(RoundRec) == 48, "three 16-byte LDS reads");
+
 struct Stage {
   uint32_t payload[kPayloadWords];
   uint32_t go;
   uint32_t pad[3];
-  tcpxuLoadMeta desc[kMaxDescsPerTicket];
+  RoundRec rec[kMaxDescsPerTicket];
 };
+
+__device__ __forceinline__ uint32_t lane_shift(uint32_t v, uint32_t from_lane) {
+  return static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(static_cast<int>((from_lane & 63u) << 2), static_cast<int>(v)));
+}
 
 // Fetcher: look once at the slot of ticket number `ticket` (one 64-byte read, with this workgroup's stop word in
 // the same round trip).  Returns 1 and stages the ticket if it is there.  Wave-uniform.
@@ -367,13 +386,47 @@ __device__ uint32_t try_fetch_ticket(DevState* st, const uint32_t* stop_word, ui
   const uint32_t gathered = bcast(word, (pl / 3) * 4 + (pl % 3));
   if (lane < kPayloadWords) stage->payload[lane] = gathered;
   if (lane == 0) stage->go = 1;
-  const uint64_t descs_addr =
-      (static_cast<uint64_t>(bcast(word, payload_slot(5))) << 32) | bcast(word, payload_slot(4));
+  auto word64 = [&](int lo) {
+    return (static_cast<uint64_t>(bcast(word, payload_slot(lo + 1))) << 32) | bcast(word, payload_slot(lo));
+  };
+  const uint64_t bounce = word64(0), dst = word64(2), descs_addr = word64(4);
   const uint32_t n = bcast(word, payload_slot(10)) & 0xFFu;
+  // One 16-byte descriptor per lane straight from where the submission keeps them (system scope: never a cached
+  // copy); lanes past the end repeat the last one and write no record.
+  const uint32_t mine = lane < n ? lane : (n != 0 ? n - 1u : 0u);  // a ticket has at least one descriptor
+  const u32x4 d = load_vec_sys(reinterpret_cast<const uint8_t*>(descs_addr) + 16 * mine);
+  const uint32_t so = d[0], len = d[1];
+  const uint64_t doff = (static_cast<uint64_t>(d[3]) << 32) | d[2];
+  // The neighbours' descriptors decide which destination lines are shared with them.
+  const uint32_t p_len = lane_shift(len, lane - 1u), p_dlo = lane_shift(d[2], lane - 1u), p_dhi = lane_shift(d[3], lane - 1u);
+  const uint32_t q_len = lane_shift(len, lane + 1u), q_dlo = lane_shift(d[2], lane + 1u), q_dhi = lane_shift(d[3], lane + 1u);
+  const uint32_t q_so = lane_shift(so, lane + 1u);
+  const uint64_t fdst = dst + doff, fsrc = bounce + so;
+  const uint64_t p_dst = dst + ((static_cast<uint64_t>(p_dhi) << 32) | p_dlo);
+  const uint64_t q_dst = dst + ((static_cast<uint64_t>(q_dhi) << 32) | q_dlo);
+  uint32_t kind = kRecRounds;
+  if (len == 0) kind = kRecSkip;
+  else if (fragment_is_tiny(reinterpret_cast<const uint8_t*>(fdst), len)) kind = kRecTiny;
+  const bool share_prev = kind == kRecRounds && lane > 0 && shares_line(p_dst, p_len, fdst, len);
+  const bool share_next = kind == kRecRounds && lane + 1 < n && shares_line(fdst, len, q_dst, q_len);
+  FragmentPlan plan = {0, 0, 0, 0, 1};
+  if (kind == kRecRounds) plan = plan_fragment(fdst, len, share_prev, share_next);
+  const uint64_t next_src = share_next ? bounce + q_so : fsrc;
   if (lane < n) {
-    // One 16-byte descriptor per lane straight from the mapped slot (system scope: never a cached copy).
-    const u32x4 d = load_vec_sys(reinterpret_cast<const uint8_t*>(descs_addr) + 16 * lane);
-    *reinterpret_cast<u32x4*>(&stage->desc[lane]) = d;
+    RoundRec r;
+    r.src_lo = static_cast<uint32_t>(fsrc);
+    r.src_hi = static_cast<uint32_t>(fsrc >> 32);
+    r.dst_lo = static_cast<uint32_t>(fdst);
+    r.dst_hi = static_cast<uint32_t>(fdst >> 32);
+    r.next_lo = static_cast<uint32_t>(next_src);
+    r.next_hi = static_cast<uint32_t>(next_src >> 32);
+    r.start_off = plan.start_off;
+    r.end_off = plan.end_off;
+    r.len = len;
+    r.nvec = plan.nvec;
+    r.bits = plan.head | (plan.tail << 8) | (share_next ? 1u << 16 : 0u) | (kind << 24);
+    r.pad = 0;
+    stage->rec[lane] = r;
   }
   return 1;
 }
@@ -406,21 +459,62 @@ __device__ void retire_ticket(DevState* st, uint32_t* jobs_done, const Stage* st
 }
 
 // Copy wavefront `wave` of kCopyWaves: its run of consecutive fragments of the staged ticket (an eighth of the
-// ticket, rounded up).  A wavefront that writes one contiguous stretch of the destination after another measured
-// about 1 % faster end to end than fragments dealt out in turn (wave, wave + kCopyWaves, ...).
+// ticket, rounded up), one round (at most 4 KiB) in flight at a time.  A wavefront that writes one contiguous
+// stretch of the destination after another measured about 1 % faster end to end than fragments dealt out in turn
+// (wave, wave + kCopyWaves, ...).
 __device__ void copy_ticket(const Stage* stage, uint32_t wave, uint32_t lane, uint32_t* waves_on_last) {
   auto uniform = [](uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(v)); };
-  const uint8_t* bounce = reinterpret_cast<const uint8_t*>((static_cast<uint64_t>(uniform(stage->payload[1])) << 32) |
-                                                           uniform(stage->payload[0]));
-  uint8_t* dst =
-      reinterpret_cast<uint8_t*>((static_cast<uint64_t>(uniform(stage->payload[3])) << 32) | uniform(stage->payload[2]));
+  wave = uniform(wave);
   const uint32_t n = uniform(stage->payload[10]) & 0xFFu;
   const uint32_t per = (n + kCopyWaves - 1) / kCopyWaves;
-  const uint32_t first = wave * per < n ? wave * per : n;
-  const uint32_t end = first + per < n ? first + per : n;
-  wave_copy_descriptors(stage->desc, n, first, 1u, end, bounce, dst, lane, [&] {
+  uint32_t j = wave * per < n ? wave * per : n;
+  const uint32_t end = j + per < n ? j + per : n;
+  // Told once, when the wavefront turns to the last fragment of its share (at once if it has none): the fetcher
+  // uses it to start fetching the next ticket.
+  auto on_last_fragment = [&] {
     if (lane == 0) __hip_atomic_fetch_add(waves_on_last, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-  });
+  };
+  if (j >= end) on_last_fragment();
+  uint32_t nvec_left = 0;
+  CopyRound r;
+  // The next round of the share, or false when there is none.
+  auto produce = [&]() -> bool {
+    if (nvec_left != 0) {  // a fragment longer than one round goes on
+      r.has_edge = false;  // the first round has copied the edge bytes and the shared line
+      r.share_next = false;
+      r.src_vec += static_cast<size_t>(r.nvec) << 4;
+      r.dst_vec += static_cast<size_t>(r.nvec) << 4;
+      r.nvec = nvec_left < kVecPerRound ? nvec_left : kVecPerRound;
+      nvec_left -= r.nvec;
+      return true;
+    }
+    while (j < end) {
+      const u32x4* words = reinterpret_cast<const u32x4*>(&stage->rec[j]);
+      const u32x4 w0 = words[0], w1 = words[1], w2 = words[2];
+      ++j;
+      if (j >= end) on_last_fragment();
+      const uint32_t bits = uniform(w2[2]);
+      const uint32_t kind = bits >> 24;
+      if (kind == kRecSkip) continue;
+      const uint8_t* src = reinterpret_cast<const uint8_t*>((static_cast<uint64_t>(uniform(w0[1])) << 32) | uniform(w0[0]));
+      uint8_t* dst = reinterpret_cast<uint8_t*>((static_cast<uint64_t>(uniform(w0[3])) << 32) | uniform(w0[2]));
+      const uint32_t len = uniform(w2[0]);
+      if (kind == kRecTiny) {
+        copy_tiny_fragment(src, dst, len, lane);
+        continue;
+      }
+      const uint8_t* src_next = reinterpret_cast<const uint8_t*>((static_cast<uint64_t>(uniform(w1[1])) << 32) | uniform(w1[0]));
+      r = first_round_of(src, dst, src_next, len, ((bits >> 16) & 1u) != 0, uniform(w1[2]), uniform(w1[3]), bits & 0xFFu,
+                         (bits >> 8) & 0xFFu, uniform(w2[1]), lane, &nvec_left);
+      return true;
+    }
+    return false;
+  };
+  CopyRegs x;
+  while (produce()) {
+    round_load(r, x, lane);
+    round_store(r, x, lane);
+  }
 }
 
 __device__ void worker_loop(DevState* st, uint32_t* jobs_done, uint32_t flags) {
