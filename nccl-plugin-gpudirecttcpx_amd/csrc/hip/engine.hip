@@ -7,8 +7,9 @@
 //                             or of the fixed `descs_per_ticket`) and writes them into a device-memory ticket
 //                             ring.  It never copies payload.
 //   every other workgroup     "worker": one fetcher wavefront claims the next ticket number with one atomic,
-//                             polls that ticket's slot until its stamps match and stages the ticket's
-//                             descriptors from the mapped slot into LDS; the copy wavefronts copy the fragments,
+//                             polls that ticket's slot until its stamps match, reads the ticket's descriptors
+//                             (one per lane) and leaves in LDS, per fragment, a record of what the copy needs
+//                             to know about it; the copy wavefronts copy the fragments from those records,
 //                             and the last of them to finish counts the ticket done.  Whoever counts the last
 //                             ticket of a submission writes the completion word that the host poller reads.
 //
@@ -334,8 +335,8 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
 
 // ---- worker -------------------------------------------------------------------------------------------------------
 // A worker workgroup is kCopyWaves copy wavefronts and one fetcher wavefront.  Towards the end of ticket i the
-// fetcher claims a number, polls that ticket's slot and pulls the ticket's descriptors over PCIe into the other
-// LDS stage; between two tickets the copy wavefronts only meet the fetcher at one barrier.  The copy wavefront
+// fetcher claims a number, polls that ticket's slot, pulls the ticket's descriptors over PCIe and writes their
+// records into the other LDS stage; between two tickets the copy wavefronts only meet the fetcher at one barrier.  The copy wavefront
 // that finishes a ticket last counts it.
 #ifndef TCPXU_ENGINE_COPY_WAVES
 #define TCPXU_ENGINE_COPY_WAVES 8
