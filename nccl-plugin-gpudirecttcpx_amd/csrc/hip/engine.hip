@@ -577,8 +577,9 @@ __device__ void worker_loop(DevState* st, uint32_t* jobs_done, uint32_t flags) {
         stop_before = stop_up;
         first_look = false;
         if (!stop_before) {
-          // Idle: look again soon at first, then back off so that a thousand idle workgroups do not load the
-          // memory system that busy ones are using.
+          // Idle: look again soon at first, then back off a little, so that a thousand idle workgroups do not
+          // load the memory system that busy ones are using.  (At most two sleeps between looks: with up to
+          // eight a lone 64 KiB request took 0.2 us longer, four in flight 1.2 us, and no workload was faster.)
           for (uint32_t i = 0; i < backoff; ++i) __builtin_amdgcn_s_sleep(4);
           if (backoff < backoff_cap) backoff <<= 1;
         }
@@ -713,7 +714,7 @@ int tcpxuEngineCreate(int device, const tcpxuEngineConfig* config, tcpxuEngine**
     const char* ve = getenv("TCPXU_ENGINE_EAGER");
     const char* vb = getenv("TCPXU_ENGINE_BACKOFF_CAP");
     const uint32_t eager = (ve && *ve) ? static_cast<uint32_t>(atoi(ve)) & 3u : 2u;
-    const uint32_t cap = (vb && *vb) ? static_cast<uint32_t>(atoi(vb)) & 0xFFu : 8u;
+    const uint32_t cap = (vb && *vb) ? static_cast<uint32_t>(atoi(vb)) & 0xFFu : 2u;
     e->flags = eager | (cap << 8);
   }
   int rc = TCPXU_SUCCESS;
