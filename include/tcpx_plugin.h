@@ -126,6 +126,9 @@ typedef struct tcpxDeviceOps {
   int (*visible_alloc)(int device, size_t bytes, void** host_ptr, void** dev_ptr);
   int (*visible_free)(int device, void* host_ptr);
   void (*visible_flush)(void);
+  /* Optional (may be NULL): engine_submit with the request's size as a hint (tcpxuEngineSubmitSized). */
+  int (*engine_submit_sized)(tcpxuEngine* engine, const void* bounce_base, void* dst_base, const void* descs_dev,
+                             uint32_t n_descs, uint64_t payload_bytes, void* done_flag_dev, uint64_t done_value);
 } tcpxDeviceOps;
 
 /* Installs `ops` in place of the HIP layer (NULL restores the default binding).  For host-logic tests only;

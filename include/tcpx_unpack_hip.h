@@ -152,6 +152,12 @@ int tcpxuEngineDestroy(tcpxuEngine* engine);
  * This is the publish of src/net_tcpx.cc:1354-1357 made explicit: count, then a release, then the tail. */
 int tcpxuEngineSubmit(tcpxuEngine* engine, const void* bounce_base, void* dst_base, const void* descs_dev,
                       uint32_t n_descs, void* done_flag_dev, uint64_t done_value);
+/* The same with a hint: `payload_bytes` = the sum of the descriptors' lengths (the size of the request, which the
+ * caller of src/net_tcpx.cc:1354-1357 has at hand in tcpxRequest::offset), 0 = unknown.  The engine hands out a
+ * slot's descriptors in tickets of about 64 KiB, 16 fragments of a page; with the hint, a slot of shorter
+ * fragments gets tickets of more descriptors (up to 64).  Without it fragments are taken to be whole pages. */
+int tcpxuEngineSubmitSized(tcpxuEngine* engine, const void* bounce_base, void* dst_base, const void* descs_dev,
+                           uint32_t n_descs, uint64_t payload_bytes, void* done_flag_dev, uint64_t done_value);
 
 /* Number of submissions the GPU has fully completed since creation (monotone; read from mapped memory). */
 int tcpxuEngineCompleted(tcpxuEngine* engine, uint64_t* completed);
@@ -170,7 +176,7 @@ typedef struct tcpxuStreamItem {
   void* dst_base;
   const tcpxuLoadMeta* descs_host; /* descriptors in ordinary host memory */
   uint32_t n_descs;                /* at most TCPXU_SLOT_PAGES */
-  uint32_t reserved;
+  uint32_t payload_bytes;          /* sum of the descriptors' lengths, 0 = unknown (see tcpxuEngineSubmitSized) */
 } tcpxuStreamItem;
 
 /* Slots the streaming driver can keep in flight: the unpack queues of eight receive comms. */

@@ -79,7 +79,7 @@ class StreamItem(ctypes.Structure):
         ("dst_base", ctypes.c_void_p),
         ("descs_host", ctypes.c_void_p),
         ("n_descs", ctypes.c_uint32),
-        ("reserved", ctypes.c_uint32),
+        ("payload_bytes", ctypes.c_uint32),
     ]
 
 
@@ -164,6 +164,19 @@ _HIP_PROTOTYPES = {
             ctypes.c_void_p,
             ctypes.c_void_p,
             ctypes.c_uint32,
+            ctypes.c_void_p,
+            ctypes.c_uint64,
+        ],
+    ),
+    "tcpxuEngineSubmitSized": (
+        ctypes.c_int,
+        [
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.c_uint32,
+            ctypes.c_uint64,
             ctypes.c_void_p,
             ctypes.c_uint64,
         ],

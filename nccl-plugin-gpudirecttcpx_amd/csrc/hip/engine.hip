@@ -3,7 +3,7 @@
 //
 // Roles inside the one kernel launch
 //   workgroup 0, wavefront 0  "leader": polls the submission ring over PCIe (sixteen entries per round trip),
-//                             cuts each submission into tickets of 8 to 32 consecutive descriptors (by backlog,
+//                             cuts each submission into tickets of 8 to 16 consecutive descriptors (by backlog,
 //                             or of the fixed `descs_per_ticket`) and writes them into a device-memory ticket
 //                             ring.  It never copies payload.
 //   every other workgroup     "worker": one fetcher wavefront claims the next ticket number with one atomic,
@@ -55,23 +55,46 @@ constexpr uint32_t kMaxDescsPerTicket = 64;
 // workgroups, larger ones spend less of each workgroup's time on pick-ups.  `backlog` estimates the descriptors of
 // all submissions not yet completed, counting each in full until it completes (how far the slots in flight have
 // got depends on the ticket size itself and would feed back).  The steps are where throughput measured at 1 to
-// 64 slots of 4 MiB in flight changed hands between sizes; 8 is one fragment per copy wavefront.
-// (Descriptors per worker workgroup below 13, 18, 30, 75; written without the division, which the leader would pay
-// for on every submission.  backlog <= 2^20 and workers < 2^16 keep the products in 32 bits.)
+// 64 slots of 4 MiB in flight changed hands between sizes; 8 is one fragment per copy wavefront, 16 two.  Beyond
+// 16 nothing is gained for fragments of a page: with every source page coming from HBM, 64 slots in flight move
+// 71.0 % of the roofline in tickets of 16, 70.1 % in tickets of 24 and 69.4 % in tickets of 32 (more tickets than
+// workgroups keep every workgroup supplied, and a wavefront that has finished its share waits less for the
+// slowest one).
+// (Descriptors per worker workgroup below 13, 18; written without the division, which the leader would pay for
+// on every submission.  backlog <= 2^20 and workers < 2^16 keep the products in 32 bits.)
 __device__ __forceinline__ uint32_t ticket_size_for(uint32_t backlog, uint32_t workers) {
-  return backlog < 13u * workers ? 8u : backlog < 18u * workers ? 12u : backlog < 30u * workers ? 16u
-                                                          : backlog < 75u * workers ? 24u : 32u;
+  return backlog < 13u * workers ? 8u : backlog < 18u * workers ? 12u : 16u;
 }
 // Ticket size for one submission of n descriptors when `in_flight` submissions (this one included) are not yet
 // completed; each is taken to be as long as this one.  A small submission among many stays whole: with 8 or
 // more in flight the parallelism is in the submissions, and a submission that is one ticket costs the leader
 // one store instead of a pass of its loop.  (64 KiB requests of 16 fragments, p50 publish -> done: 8.7 -> 9.1 us
 // at 8 in flight, 17.5 -> 9.3 us at 32, where the leader's loop had become the queue.)
+//
+// `bytes` is the submission's payload if the caller said (0 = unknown: whole pages).  The largest step, 16, stands
+// for 64 KiB: a submission of shorter fragments gets as many descriptors per ticket as make 64 KiB, in multiples
+// of 8 so that the copy wavefronts' shares come out even, up to 64 (fragments of 2 KiB on average, 64 slots in
+// flight: 52.9 % of the roofline in tickets of 16, 59.1 % in tickets of 32, 61.4 % in tickets of 64).  Written
+// as comparisons: the leader runs this for every submission and a division costs it forty instructions.
 constexpr uint32_t kManyInFlight = 8, kSmallSubmission = 32;
-__device__ __forceinline__ uint32_t ticket_size_for_submission(uint32_t in_flight, uint32_t n, uint32_t workers) {
+constexpr uint32_t kFullTicket = 16;
+__device__ __forceinline__ uint32_t full_ticket_size(uint32_t bytes, uint32_t n) {
+  static_assert(kFullTicket == 16 && kMaxDescsPerTicket == 64, "the steps below: 64 KiB / (bytes / n), in eights");
+  const uint64_t b = bytes;  // n <= 2^20: the products need more than 32 bits
+  return bytes == 0 || b >= 2731ull * n ? 16u
+         : b >= 2048ull * n             ? 24u
+         : b >= 1639ull * n             ? 32u
+         : b >= 1366ull * n             ? 40u
+         : b >= 1171ull * n             ? 48u
+         : b >= 1024ull * n             ? 56u
+                                        : 64u;
+}
+__device__ __forceinline__ uint32_t ticket_size_for_submission(uint32_t in_flight, uint32_t n, uint32_t bytes,
+                                                               uint32_t workers) {
   if (in_flight >= kManyInFlight && n <= kSmallSubmission) return kSmallSubmission;
   const uint64_t all = static_cast<uint64_t>(in_flight) * n;
-  return ticket_size_for(all > (1u << 20) ? (1u << 20) : static_cast<uint32_t>(all), workers);
+  const uint32_t size = ticket_size_for(all > (1u << 20) ? (1u << 20) : static_cast<uint32_t>(all), workers);
+  return size < kFullTicket ? size : full_ticket_size(bytes, n);
 }
 constexpr uint32_t kMaxDescsPerSubmission = 1u << 20;
 constexpr uint32_t kStopReplicas = 64;
@@ -87,7 +110,8 @@ struct alignas(64) Record {
 };
 constexpr int kPayloadWords = 12;
 __host__ __device__ constexpr int payload_slot(int i) { return (i / 3) * 4 + (i % 3); }
-// Submission payload: 0-1 bounce, 2-3 dst, 4-5 descs, 6-7 done_flag, 8-9 done_value, 10 n_descs, 11 unused.
+// Submission payload: 0-1 bounce, 2-3 dst, 4-5 descs, 6-7 done_flag, 8-9 done_value, 10 n_descs, 11 payload bytes
+//                     (0 = not given).
 // Ticket payload:     0-1 bounce, 2-3 dst, 4-5 descs, 6-7 done_flag, 8-9 done_value, 10 n | job << 8 | only << 31,
 //                     11 target.  `only`: the submission's only ticket (the job slot index is below 2^16).
 constexpr uint32_t kOnlyTicket = 1u << 31;
@@ -197,8 +221,9 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
         const uint32_t done_now = bcast(aux, k_of_lane);
         const uint32_t target_prev = bcast(aux, kPollEntries + k_of_lane);
         const uint32_t in_flight = static_cast<uint32_t>(s + k_of_lane) - jobs_completed + 1u;
+        const uint32_t bytes = bcast(sect.z, lane | 3u);  // payload word 11 sits in .z of sector 3
         const uint32_t per_ticket =
-            fixed_per_ticket != 0 ? fixed_per_ticket : ticket_size_for_submission(in_flight, n, gridDim.x - 1);
+            fixed_per_ticket != 0 ? fixed_per_ticket : ticket_size_for_submission(in_flight, n, bytes, gridDim.x - 1);
         const bool one_ticket = small && n <= per_ticket && done_now == target_prev;
         const uint64_t not_fast = ~__ballot(one_ticket);
         uint32_t run = not_fast == 0 ? kPollEntries : static_cast<uint32_t>(__builtin_ctzll(not_fast)) >> 2;
@@ -240,8 +265,9 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
       } else {
         // Submissions not yet completed, this one included, taken to be as long as this one.
         const uint32_t in_flight = static_cast<uint32_t>(s + k) - jobs_completed + 1u;
-        const uint32_t per_ticket =
-            fixed_per_ticket != 0 ? fixed_per_ticket : ticket_size_for_submission(in_flight, n, gridDim.x - 1);
+        const uint32_t per_ticket = fixed_per_ticket != 0
+                                        ? fixed_per_ticket
+                                        : ticket_size_for_submission(in_flight, n, payload_of(fl, 11), gridDim.x - 1);
         const uint32_t nt = (n + per_ticket - 1) / per_ticket;
         const uint32_t slot = static_cast<uint32_t>(s + k) & ring_mask;
         const uint32_t done_now = lane_value(aux, k);
@@ -345,7 +371,7 @@ constexpr uint32_t kCopyWaves = TCPXU_ENGINE_COPY_WAVES;
 constexpr uint32_t kEngineThreads = (kCopyWaves + 1) * kWaveLanes;
 
 // What a copy wavefront needs to know about one fragment, worked out by the fetcher: one descriptor per lane, all
-// 8..32 of a ticket at once, instead of by each copy wavefront from three descriptors per fragment.
+// descriptors of a ticket at once, instead of by each copy wavefront from three descriptors per fragment.
 constexpr uint32_t kRecSkip = 0, kRecTiny = 1, kRecRounds = 2;
 struct alignas(16) RoundRec {
   uint32_t src_lo, src_hi;     // the fragment's first byte
@@ -831,6 +857,11 @@ int tcpxuEngineDestroy(tcpxuEngine* e) {
 
 int tcpxuEngineSubmit(tcpxuEngine* e, const void* bounce_base, void* dst_base, const void* descs_dev,
                       uint32_t n_descs, void* done_flag_dev, uint64_t done_value) {
+  return tcpxuEngineSubmitSized(e, bounce_base, dst_base, descs_dev, n_descs, 0, done_flag_dev, done_value);
+}
+
+int tcpxuEngineSubmitSized(tcpxuEngine* e, const void* bounce_base, void* dst_base, const void* descs_dev,
+                           uint32_t n_descs, uint64_t payload_bytes, void* done_flag_dev, uint64_t done_value) {
   if (!e || !done_flag_dev || done_value == 0 || reinterpret_cast<uintptr_t>(done_flag_dev) % 8 != 0) {
     set_error("submit needs an 8-byte aligned completion word and a nonzero completion value");
     return TCPXU_INVALID_ARGUMENT;
@@ -855,6 +886,7 @@ int tcpxuEngineSubmit(tcpxuEngine* e, const void* bounce_base, void* dst_base, c
     p[2 * i + 1] = static_cast<uint32_t>(v[i] >> 32);
   }
   p[10] = n_descs;
+  p[11] = payload_bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : static_cast<uint32_t>(payload_bytes);
   Record* ent = &e->ctl->ring[e->tail & (e->ring_entries - 1)];
   volatile uint32_t* w = ent->w;
   for (int i = 0; i < kPayloadWords; ++i) w[payload_slot(i)] = p[i];
@@ -989,8 +1021,8 @@ static int stream_items(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n
         tcpxuVisibleFlush();
         descs_dev = static_cast<uint8_t*>(e->stage_dev) + kStageBytes * slot;
       }
-      rc = tcpxuEngineSubmit(e, it.bounce_base, it.dst_base, descs_dev, it.n_descs,
-                             db + flag_stride * slot, next_submit + 1);
+      rc = tcpxuEngineSubmitSized(e, it.bounce_base, it.dst_base, descs_dev, it.n_descs, it.payload_bytes,
+                                  db + flag_stride * slot, next_submit + 1);
       if (rc == kTcpxuInProgress) {
         rc = TCPXU_SUCCESS;
         break;  // engine ring full: reap first

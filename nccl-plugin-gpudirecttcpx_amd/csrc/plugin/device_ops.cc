@@ -53,6 +53,7 @@ const tcpxDeviceOps* default_device_ops() {
   ok &= bind(&g_hip_ops.engine_stop, "tcpxuEngineStop");
   ok &= bind(&g_hip_ops.engine_destroy, "tcpxuEngineDestroy");
   ok &= bind(&g_hip_ops.engine_submit, "tcpxuEngineSubmit");
+  ok &= bind(&g_hip_ops.engine_submit_sized, "tcpxuEngineSubmitSized");
   ok &= bind(&g_hip_ops.last_error, "tcpxuLastError");
   ok &= bind(&g_hip_ops.visible_alloc, "tcpxuVisibleAlloc");
   ok &= bind(&g_hip_ops.visible_free, "tcpxuVisibleFree");

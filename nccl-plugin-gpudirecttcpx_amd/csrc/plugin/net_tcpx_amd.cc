@@ -728,9 +728,15 @@ ncclResult_t tcpxTest(void* request, int* done, int* size) {
           g.ops->visible_flush();
           descs_dev = q->stage_dev + r->slot.idx * kStagedDescs;
         }
-        const int rc = g.ops->engine_submit(comm->device->engine, comm->device->arena, r->data, descs_dev,
-                                            static_cast<uint32_t>(r->slot.cnt_cache),
-                                            &q->meta_dev->done[r->slot.idx].value, r->done_value);
+        // The request's size goes along as a hint (it sizes the engine's tickets for fragments shorter than a page).
+        const uint32_t n_descs = static_cast<uint32_t>(r->slot.cnt_cache);
+        void* done_flag = &q->meta_dev->done[r->slot.idx].value;
+        const int rc = g.ops->engine_submit_sized
+                           ? g.ops->engine_submit_sized(comm->device->engine, comm->device->arena, r->data, descs_dev,
+                                                        n_descs, static_cast<uint64_t>(r->offset), done_flag,
+                                                        r->done_value)
+                           : g.ops->engine_submit(comm->device->engine, comm->device->arena, r->data, descs_dev, n_descs,
+                                                  done_flag, r->done_value);
         if (rc == TCPXU_IN_PROGRESS) {  // submission ring full: try again at the next poll
           --comm->done_seq;
           return ncclSuccess;

@@ -44,7 +44,7 @@ static uint64_t g_submitted = 0, g_mapped_live = 0, g_device_live = 0, g_arenas_
  * descriptors lie in one can be counted. */
 #define EMU_MAX_VISIBLE 256
 static struct { uint8_t* p; size_t bytes; } g_visible[EMU_MAX_VISIBLE];
-static uint64_t g_visible_live = 0, g_staged_submits = 0, g_visible_flushes = 0;
+static uint64_t g_visible_live = 0, g_staged_submits = 0, g_visible_flushes = 0, g_last_payload_bytes = 0;
 static int g_visible_off = 0;
 static int in_visible(const void* p);
 
@@ -78,6 +78,7 @@ uint64_t emu_counter(int which) {
     case 5: return g_visible_live;
     case 6: return g_staged_submits;
     case 7: return g_visible_flushes;
+    case 8: return g_last_payload_bytes;
     default: return 0;
   }
 }
@@ -130,6 +131,11 @@ static int emu_engine_submit(tcpxuEngine* e, const void* bounce, void* dst, cons
   }
   return 0;
 }
+static int emu_engine_submit_sized(tcpxuEngine* e, const void* bounce, void* dst, const void* descs, uint32_t n,
+                                   uint64_t payload_bytes, void* flag, uint64_t value) {
+  g_last_payload_bytes = payload_bytes;
+  return emu_engine_submit(e, bounce, dst, descs, n, flag, value);
+}
 static const char* emu_last_error(void) { return "emulated device"; }
 static int emu_visible_alloc(int dev, size_t bytes, void** host_ptr, void** dev_ptr) {
   (void)dev;
@@ -169,6 +175,6 @@ static const tcpxDeviceOps g_ops = {
     emu_device_count, emu_arena_create,  emu_arena_destroy, emu_mapped_alloc,  emu_mapped_free,
     emu_device_alloc, emu_device_free,   emu_copy_to_device, emu_engine_create, emu_engine_start,
     emu_engine_stop,  emu_engine_destroy, emu_engine_submit, emu_last_error,
-    emu_visible_alloc, emu_visible_free, emu_visible_flush,
+    emu_visible_alloc, emu_visible_free, emu_visible_flush, emu_engine_submit_sized,
 };
 const tcpxDeviceOps* emu_ops(void) { return &g_ops; }

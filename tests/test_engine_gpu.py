@@ -258,7 +258,7 @@ def test_engine_argument_errors(pkg, hip):
 @pytest.mark.parametrize("depth", [1, 5, 16, 64, 128])
 def test_engine_stream_depths(pkg, hip, oracle, depth):
     """The streaming driver (mapped slot ring, warm-up + timed items in one launch) at 1 to 64 slots in flight:
-    the leader then cuts tickets of 8 to 32 descriptors by backlog, and every size must give the oracle's bytes.
+    the leader then cuts tickets of 8 to 16 descriptors by backlog, and every size must give the oracle's bytes.
     Eight distinct 8 MiB chunks, each twice, so every destination is written by two passes of the ring."""
     import torch
 
@@ -299,6 +299,52 @@ def test_engine_stream_depths(pkg, hip, oracle, depth):
     e = Engine(pkg, hip)
     assert hip.tcpxuEngineRunTimed(e.h, items, 4, 0, 129, 1000, ctypes.byref(wall), ctypes.byref(kern), None) == pkg.INVALID_ARGUMENT
     e.destroy()
+
+
+@pytest.mark.parametrize("hint", ["true", "none", "tiny", "huge"])
+def test_engine_ticket_size_follows_the_payload_hint(pkg, hip, oracle, hint):
+    """Ragged and empty fragments (the adversarial workload, 2 KiB a fragment on average) with 64 slots in flight:
+    with the request's byte count given, the leader cuts tickets of up to 64 descriptors, without it tickets of
+    16; a hint is only a hint, so a wrong one (far too small, far too large) must give the same bytes."""
+    import torch
+
+    wl = pkg.Workload(5, seed=0xAD5E12)
+    info = wl.info
+    pool = np.empty(info.pool_bytes, dtype=np.uint8)
+    wl.fill_window(0, pool)
+    size = int(info.dst_bytes) + int(info.dst_misalign)
+    passes = 6
+    stride = (size + 4095) // 4096 * 4096
+    expect = np.full(GUARD + passes * stride + GUARD, SENTINEL, dtype=np.uint8)
+    one = oracle_expected(oracle, pool, wl.descs, int(info.dst_bytes), int(info.dst_misalign))
+    for ps in range(passes):
+        lo = GUARD + ps * stride
+        expect[lo : lo + size] = one[GUARD : GUARD + size]
+    pool_d = torch.from_numpy(pool).to("cuda:0")
+    dst_d = torch.full((expect.nbytes,), SENTINEL, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    descs = np.ascontiguousarray(wl.descs)
+    reqs = [(int(r["first_desc"]), int(r["n_descs"])) for r in wl.requests]
+    items = (pkg.StreamItem * (passes * len(reqs)))()
+    i = 0
+    for ps in range(passes):
+        for first, n in reqs:
+            nbytes = int(descs["len"][first : first + n].sum())
+            items[i].bounce_base = pool_d.data_ptr()
+            items[i].dst_base = dst_d.data_ptr() + GUARD + ps * stride + int(info.dst_misalign)
+            items[i].descs_host = descs.ctypes.data + 16 * first
+            items[i].n_descs = n
+            items[i].payload_bytes = {"true": nbytes, "none": 0, "tiny": 1, "huge": 0xFFFFFFFF}[hint]
+            i += 1
+    e = Engine(pkg, hip)
+    print("engine hint case: %s, %d items" % (hint, len(items)), flush=True)
+    wall, kern = ctypes.c_double(), ctypes.c_double()
+    rc = hip.tcpxuEngineRunTimed(e.h, items, len(items), 0, 64, 20000, ctypes.byref(wall), ctypes.byref(kern), None)
+    pkg.check(rc, "tcpxuEngineRunTimed")
+    assert e.completed() == len(items)
+    e.destroy()
+    got = dst_d.cpu().numpy()
+    assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
 
 
 def test_engine_bursts_around_the_idle_exit(pkg, hip, oracle):

@@ -167,6 +167,19 @@ def test_small_requests_hand_over_a_second_copy_of_their_descriptors(env, comm):
         env.emu.emu_set_visible_off(0)
 
 
+def test_the_request_size_goes_along_with_the_submission(env, comm):
+    """The slot is handed to the engine with the request's byte count as a hint (the sum of its descriptors'
+    lengths); one request at a time, so that the last submission seen is the request just completed."""
+    wl = env.pkg.Workload(5, seed=0x51ED, shrink=5)  # ragged fragments and empty descriptors
+    pool = fill_arena(env, wl)
+    buf, ptr = host_buffer(int(wl.info.dst_bytes))
+    env.driver.run_workload(comm, wl, ptr, n_flows=4, window=1)
+    assert np.array_equal(buf, expected_bytes(pool, wl.frags, wl.requests, int(wl.info.dst_bytes)))
+    last = wl.requests[-1]
+    first, n = int(last["first_desc"]), int(last["n_descs"])
+    assert env.emu.emu_counter(8) == int(wl.descs["len"][first : first + n].sum()) == int(last["bytes"])
+
+
 def test_partial_recvmsg_and_window_one(env, comm):
     """Fragments trickle in three per recvmsg; one request in flight at a time."""
     wl = env.pkg.Workload(2, seed=77, shrink=3)
