@@ -36,7 +36,7 @@ import __graft_entry__ as graft
 # HBM bytes moved per algorithmic byte (2 x fragment bytes) by unpack_engine_kernel on the headline workload:
 # hardware counters FETCH_SIZE (x1.99977, its reading for a copy kernel of known size) and WRITE_SIZE (x1.0),
 # 9387258 KiB + 9385714 KiB against 2 x 9273344 KiB over one launch of 1132 steps.
-TRAFFIC_PER_ALGORITHMIC_BYTE = 1.0074
+TRAFFIC_PER_ALGORITHMIC_BYTE = 1.0061
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 CHUNK_CONFIG = 2
 
