@@ -19,6 +19,16 @@ show 1.6 points more than with 64 or 128 copies, where the figure no longer move
 traffic, not cache hits.  Bounce pool, descriptor lists and destinations are resident before the
 timed region starts; nothing crosses PCIe during it except descriptors and completion words.
 
+How the K steps are timed.  A step is 3 us of GPU work and a request's way through the engine about 10 us, so
+K steps on their own would measure the filling and draining of the queues.  One launch of the persistent kernel
+therefore carries: an untimed fill of at least two queues' worth of steps (never fewer than `--warmup`), then R
+windows of exactly K steps each, back to back, then an untimed tail of one queue's worth that keeps the queues
+full while the last window finishes.  Every completion is stamped by the host poller; a window is timed from the
+completion of the step before it to the completion of its last step; `ms_per_step` x K is the MEDIAN window and
+`value` the payload of K steps over it.  R is at least 50 and large enough that the launch carries 2000 steps or
+more, so that the launch's own duration (HIP events on the engine's stream: `roofline`) is the rate too, with
+launch, ramp and stop below 2 % of it.
+
 Prints ONE JSON line: payload GB/s (`value`), the HBM roofline of the dominant kernel, p50/p99 request
 completion latency, and a memcpy-per-descriptor CPU baseline timed on this machine's host cores.
 """
@@ -33,9 +43,10 @@ import numpy as np
 
 import __graft_entry__ as graft
 
-# HBM bytes moved per algorithmic byte (2 x fragment bytes) by unpack_engine_kernel on the headline workload:
-# hardware counters FETCH_SIZE (x1.99977, its reading for a copy kernel of known size) and WRITE_SIZE (x1.0),
-# 9387258 KiB + 9385714 KiB against 2 x 9273344 KiB over one launch of 1132 steps.
+# HBM bytes moved per algorithmic byte (2 x fragment bytes) by unpack_engine_kernel on the headline workload, from
+# the hardware counters FETCH_SIZE and WRITE_SIZE of one launch of `bench.py --one-launch --steps 20 --warmup 5`
+# (two rocprofv3 --pmc runs), each scaled by what the same counter reads for the plain copy kernel of known size
+# (`--calibrate-copy 256`); the summary with the counter values is profiles/unpack_engine_kernel_8MiB_chunk_pmc_traffic.txt.
 TRAFFIC_PER_ALGORITHMIC_BYTE = 1.0061
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 CHUNK_CONFIG = 2
@@ -45,10 +56,11 @@ def percentile(values, q):
     return float(np.percentile(np.asarray(values, dtype=np.float64), q))
 
 
-def cpu_baseline(oracle, wl, pool, threads, budget_s):
-    """memcpy-per-descriptor over the same descriptor list, pool and destination in host DRAM."""
-    dst = np.empty(wl.info.dst_bytes + 64, dtype=np.uint8)
-    descs = np.ascontiguousarray(wl.descs)
+def cpu_baseline(oracle, descs, dst_bytes, pool, threads, budget_s):
+    """memcpy-per-descriptor over a descriptor list, pool and destination in host memory: payload GB/s, iterations."""
+    dst = np.empty(dst_bytes + 64, dtype=np.uint8)
+    descs = np.ascontiguousarray(descs)
+    payload = float(descs["len"].sum())
     probe = (ctypes.c_double * 3)()
     rc = oracle.tcpx_oracle_unpack_timed(dst.ctypes.data, pool.ctypes.data, descs.ctypes.data, len(descs), threads, 2, 3, probe)
     assert rc == 0
@@ -58,7 +70,7 @@ def cpu_baseline(oracle, wl, pool, threads, budget_s):
     rc = oracle.tcpx_oracle_unpack_timed(dst.ctypes.data, pool.ctypes.data, descs.ctypes.data, len(descs), threads, 5, iters, secs)
     assert rc == 0
     med = float(np.median(np.asarray(secs[:])))
-    return wl.info.payload_bytes / med / 1e9, iters
+    return payload / med / 1e9, iters
 
 
 def plugin_path(pkg, hip, torch, workloads, pool):
@@ -100,7 +112,7 @@ def plugin_path(pkg, hip, torch, workloads, pool):
     }
 
 
-def batch_kernel_line(pkg, hip, torch, dev, chunks=128, pools=15, warmup=3, iters=20):
+def batch_kernel_line(pkg, benchlib, torch, dev, chunks=128, pools=15, warmup=3, iters=20):
     """tcpxuUnpackBatch on `chunks` chunks of the headline workload as ONE descriptor list and one launch: chunk c
     reads copy c % pools of the 256 MiB pool (descriptor offsets are 32-bit: 15 copies stay below 4 GiB) and writes
     its own 8 MiB of the destination, so a launch moves chunks x 8 MiB each way with nothing read or written twice."""
@@ -121,7 +133,7 @@ def batch_kernel_line(pkg, hip, torch, dev, chunks=128, pools=15, warmup=3, iter
     torch.cuda.synchronize()
     us = ctypes.c_double()
     pkg.check(
-        hip.tcpxuUnpackBatchTimed(dev, pool_d.data_ptr(), dst_d.data_ptr() + 256, descs_d.data_ptr(), len(descs), warmup, iters, ctypes.byref(us)),
+        benchlib.tcpxuUnpackBatchTimed(dev, pool_d.data_ptr(), dst_d.data_ptr() + 256, descs_d.data_ptr(), len(descs), warmup, iters, ctypes.byref(us)),
         "tcpxuUnpackBatchTimed",
     )
     payload = float(descs["len"].sum())
@@ -186,8 +198,9 @@ def other_configs(pkg, torch, run):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=4000)
-    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=400, help="K: steps in one timed window")
+    ap.add_argument("--warmup", type=int, default=64, help="W: untimed steps before the first window (at least two queues' worth are run whatever W says)")
+    ap.add_argument("--windows", type=int, default=0, help="R: timed windows of K steps in the launch; 0 = max(50, ceil(2000 / K))")
     ap.add_argument(
         "--chunks",
         type=int,
@@ -199,7 +212,7 @@ def main():
     ap.add_argument("--pools", type=int, default=64, help="copies of the 256 MiB bounce pool the chunks take turns reading from")
     ap.add_argument("--comms", type=int, default=4, help="receive comms kept busy on the one engine (1..4)")
     ap.add_argument("--depth", type=int, default=16, help="slots of one comm's mapped ring in flight (the unpack queue depth)")
-    ap.add_argument("--cpu-seconds", type=float, default=6.0, help="CPU time per baseline leg (16 threads, then 1 thread)")
+    ap.add_argument("--cpu-seconds", type=float, default=5.0, help="CPU time per baseline leg (four legs)")
     ap.add_argument("--skip-extras", action="store_true", help="only the headline measurement")
     ap.add_argument(
         "--one-launch",
@@ -224,6 +237,8 @@ def main():
     args = ap.parse_args()
     if not 1 <= args.comms <= 4 or not 1 <= args.depth <= 16 or not 1 <= args.pools <= 256:
         sys.exit("bench.py: --comms must be 1..4, --depth 1..16, --pools 1..256")
+    if args.steps < 1 or args.warmup < 0 or args.windows < 0:
+        sys.exit("bench.py: --steps must be at least 1, --warmup and --windows not negative")
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU; --gpus %d is not supported (every GPU would run an independent copy)" % args.gpus)
 
@@ -231,6 +246,7 @@ def main():
 
     pkg = graft.load_package()
     hip = pkg.hip_layer()  # raises if the HIP library is missing; there is no fallback
+    benchlib = pkg.bench_layer()  # the streaming driver and the event-timed launches
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     dev = 0
@@ -240,11 +256,11 @@ def main():
         b = torch.empty(n, dtype=torch.uint8, device="cuda:0")
         torch.cuda.synchronize()
         us = ctypes.c_double()
-        pkg.check(hip.tcpxuCopyKernelTimed(dev, b.data_ptr(), a.data_ptr(), n, 0, 10, ctypes.byref(us)), "tcpxuCopyKernelTimed")
+        pkg.check(benchlib.tcpxuCopyKernelTimed(dev, b.data_ptr(), a.data_ptr(), n, 0, 10, ctypes.byref(us)), "tcpxuCopyKernelTimed")
         print(json.dumps({"kernel": "copy_kernel", "launches": 10, "bytes_read_per_launch": n, "bytes_written_per_launch": n, "launch_us": round(us.value, 2)}))
         return
     if args.batch_kernel:
-        print(json.dumps(batch_kernel_line(pkg, hip, torch, dev)))
+        print(json.dumps(batch_kernel_line(pkg, benchlib, torch, dev)))
         return
     name = ctypes.create_string_buffer(256)
     cus = ctypes.c_int()
@@ -275,14 +291,15 @@ def main():
     slots_per_step = len(per_chunk_items[0])
     descs_per_step = float(np.mean([wl.info.n_descs for wl in workloads]))
 
+    item_dtype = np.dtype([("bounce", "<u8"), ("dst", "<u8"), ("descs", "<u8"), ("n", "<u4"), ("bytes", "<u4")])
+    assert item_dtype.itemsize == ctypes.sizeof(pkg.StreamItem)
+    # the request's size (`bytes`) is what a caller of the plugin's test() has at hand
+    ring_items = np.array([it for items in per_chunk_items for it in items], dtype=item_dtype).reshape(args.chunks, slots_per_step)
+
     def item_array(first_step, n_steps):
-        flat = []
-        for s in range(first_step, first_step + n_steps):
-            flat.extend(per_chunk_items[s % args.chunks])
-        arr = (pkg.StreamItem * len(flat))()
-        for i, (b, d, p, n, nbytes) in enumerate(flat):
-            arr[i].bounce_base, arr[i].dst_base, arr[i].descs_host, arr[i].n_descs = b, d, p, n
-            arr[i].payload_bytes = nbytes  # the request's size, which a caller of the plugin's test() has at hand
+        rows = np.ascontiguousarray(ring_items[(first_step + np.arange(n_steps)) % args.chunks].reshape(-1))
+        arr = (pkg.StreamItem * len(rows)).from_buffer(rows)
+        arr._rows = rows  # keeps the memory alive
         return arr
 
     engine = ctypes.c_void_p()
@@ -299,43 +316,55 @@ def main():
         wall, kern = ctypes.c_double(), ctypes.c_double()
         lat = (ctypes.c_double * len(items))() if want_latency else None
         if timed_items is None:
-            rc = hip.tcpxuEngineRunTimed(
+            rc = benchlib.tcpxuEngineRunTimed(
                 engine, items, len(items), warmup_items, depth, 20000, ctypes.byref(wall), ctypes.byref(kern), lat
             )
         else:
-            rc = hip.tcpxuEngineRunWindow(
+            rc = benchlib.tcpxuEngineRunWindow(
                 engine, items, len(items), warmup_items, timed_items, depth, 20000, ctypes.byref(wall), ctypes.byref(kern), lat
             )
         pkg.check(rc, "tcpxuEngineRunTimed")
         return wall.value, kern.value, (np.asarray(lat[:]) if want_latency else None)
 
-    # ---- W warm-up steps, then exactly K timed steps, all inside ONE launch of the persistent kernel -------
-    # `value` is timed by the host over the K steps only; the roofline is the kernel's: the bytes of every step
-    # in the launch over the launch's duration from HIP events, which is also what a kernel trace of this command
-    # shows for the launch.
-    # A tail of untimed steps (one queue's worth) follows the timed ones, so that the last timed steps finish in a
-    # full pipeline like the others; the K timed steps are clocked from the completion of the last warm-up step to
-    # the completion of the last timed step.
-    tail_steps = (args.comms * args.depth + slots_per_step - 1) // slots_per_step
-    all_items = item_array(0, args.warmup + args.steps + tail_steps)
+    def run_windows(items, depth):
+        """One launch over `items` with every completion stamped: the duration of each of the R windows of K steps
+        (completion of the step before the window -> completion of its last step) and of the launch, microseconds."""
+        kern = ctypes.c_double()
+        done = np.zeros(len(items), dtype=np.float64)
+        rc = benchlib.tcpxuEngineRunStamped(
+            engine, items, len(items), depth, 20000, ctypes.byref(kern), done.ctypes.data_as(ctypes.POINTER(ctypes.c_double)), None
+        )
+        pkg.check(rc, "tcpxuEngineRunStamped")
+        step_done = done[slots_per_step - 1 :: slots_per_step]  # completion of each step's last slot
+        edges = step_done[fill_steps - 1 : fill_steps + windows * args.steps : args.steps]
+        assert len(edges) == windows + 1
+        return np.diff(edges), kern.value
+
+    # ---- fill, R windows of exactly K steps, tail: all inside ONE launch of the persistent kernel ---------------
+    queue_steps = (args.comms * args.depth + slots_per_step - 1) // slots_per_step  # steps that fill every queue once
+    fill_steps = max(args.warmup, 2 * queue_steps)
+    windows = args.windows if args.windows > 0 else max(50, (2000 + args.steps - 1) // args.steps)
+    tail_steps = queue_steps
+    steps_per_launch = fill_steps + windows * args.steps + tail_steps
+    all_items = item_array(0, steps_per_launch)
     # An untimed launch first: brings the clocks up from idle and touches every page once.
     if not args.one_launch:
-        run(item_array(0, max(args.warmup, 1)), args.comms * args.depth)
+        run(item_array(0, fill_steps), args.comms * args.depth)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    wall_us, kernel_us, _ = run(
-        all_items, args.comms * args.depth, warmup_items=args.warmup * slots_per_step, timed_items=args.steps * slots_per_step
-    )
+    window_us, kernel_us = run_windows(all_items, args.comms * args.depth)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    payload = float(sum(workloads[(args.warmup + s) % args.chunks].info.payload_bytes for s in range(args.steps)))
-    launch_payload = float(sum(workloads[s % args.chunks].info.payload_bytes for s in range(args.warmup + args.steps + tail_steps)))
+    assert all(int(wl.info.payload_bytes) == int(chunk_bytes) for wl in workloads)  # every step moves the same bytes
+    payload = float(chunk_bytes) * args.steps
+    launch_payload = float(chunk_bytes) * steps_per_launch
+    wall_us = float(np.median(window_us))
     value_gbps = payload / (wall_us * 1e-6) / 1e9
     achieved = 2.0 * launch_payload / (kernel_us * 1e-6) / 1e9
 
     # ---- parity spot check: the last chunk written must equal the oracle's bytes ---------------------------
     oracle = graft.load_oracle()
-    last = (args.warmup + args.steps + tail_steps - 1) % args.chunks
+    last = (steps_per_launch - 1) % args.chunks
     expect = np.full(chunk_bytes, 0xA5, dtype=np.uint8)
     graft.oracle_unpack(oracle, expect, pool, np.ascontiguousarray(workloads[last].descs))
     got = dst_d[256 + last * chunk_bytes : 256 + (last + 1) * chunk_bytes].cpu().numpy()
@@ -361,6 +390,12 @@ def main():
             "pools": args.pools,
             "comms": args.comms,
             "queue_depth_per_comm": args.depth,
+            "fill_steps": fill_steps,
+            "windows": windows,
+            "tail_steps": tail_steps,
+            "timing": "one launch = %d untimed fill steps + %d windows of %d steps + %d untimed tail steps; a window runs from the "
+            "completion of the step before it to the completion of its last step; ms_per_step x steps = the median window"
+            % (fill_steps, windows, args.steps, tail_steps),
             "path": "persistent engine: mapped descriptor ring -> gfx950 unpack kernel -> mapped completion word",
             "descriptors_per_step": round(descs_per_step, 1),
             "slots_per_step": slots_per_step,
@@ -381,21 +416,23 @@ def main():
             "the same counters on the plain copy kernel: x1.99977 and x1.0) came to %.4f x the algorithmic bytes; "
             "that ratio times bytes_per_launch" % TRAFFIC_PER_ALGORITHMIC_BYTE,
             "bytes_per_launch": 2.0 * launch_payload,
-            "steps_per_launch": args.warmup + args.steps + tail_steps,
+            "steps_per_launch": steps_per_launch,
             "launch_us": round(kernel_us, 1),
+        },
+        "window_ms": {
+            "median": round(wall_us / 1000.0, 6),
+            "p10": round(percentile(window_us, 10) / 1000.0, 6),
+            "p90": round(percentile(window_us, 90) / 1000.0, 6),
+            "windows": windows,
+            "rw_frac_of_hbm_peak_at_median": round(2.0 * value_gbps / HBM_PEAK_GBPS, 4),
         },
         "parity_ok": parity_ok,
         "timed_region_s": round(t1 - t0, 4),
     }
-    if args.steps < 500:
-        # A step is 3 us of GPU work and a request's way through the engine about 10 us: a short run measures the
-        # filling and draining of the queues, not the rate.
-        result["note"] = "only %d steps (%.0f MiB): dominated by pipeline fill and drain; the default is 4000 steps" % (
-            args.steps, args.steps * chunk_bytes / 2**20)
-
     if args.comms > 1 and not args.one_launch:
         # The same steps with one comm only: 16 slots (at most 64 MiB) in flight, a launch of its own.
-        w1, k1, _ = run(all_items, args.depth, warmup_items=args.warmup * slots_per_step, timed_items=args.steps * slots_per_step)
+        win1, k1 = run_windows(all_items, args.depth)
+        w1 = float(np.median(win1))
         result["single_comm"] = {
             "value": round(payload / (w1 * 1e-6) / 1e9, 2),
             "unit": "GB/s",
@@ -456,7 +493,7 @@ def main():
         # Launch-per-batch kernel on the same chunk and on the 256 MiB bulk workload, and a plain copy kernel.
         us = ctypes.c_double()
         d0 = torch.from_numpy(np.ascontiguousarray(workloads[0].descs).view(np.uint8)).to("cuda:0")
-        pkg.check(hip.tcpxuUnpackBatchTimed(dev, pool_d.data_ptr(), dst_base, d0.data_ptr(), workloads[0].info.n_descs, 20, 200, ctypes.byref(us)), "batch timed")
+        pkg.check(benchlib.tcpxuUnpackBatchTimed(dev, pool_d.data_ptr(), dst_base, d0.data_ptr(), workloads[0].info.n_descs, 20, 200, ctypes.byref(us)), "batch timed")
         result["launch_per_batch_8MiB"] = {
             "kernel": "unpack_batch_kernel",
             "note": "the same chunk every launch: launch-bound and cache-resident, not an HBM figure",
@@ -470,13 +507,13 @@ def main():
         scratch = torch.empty(2 * n_copy, dtype=torch.uint8, device="cuda:0")
         scratch.zero_()
         torch.cuda.synchronize()
-        pkg.check(hip.tcpxuCopyKernelTimed(dev, scratch.data_ptr() + n_copy, scratch.data_ptr(), n_copy, 3, 20, ctypes.byref(us)), "copy timed")
+        pkg.check(benchlib.tcpxuCopyKernelTimed(dev, scratch.data_ptr() + n_copy, scratch.data_ptr(), n_copy, 3, 20, ctypes.byref(us)), "copy timed")
         result["plain_copy_kernel"] = {"bytes": n_copy, "launch_us": round(us.value, 2), "rw_GBps": round(2 * n_copy / us.value / 1e3, 1)}
         # Each half of that copy on its own (loads only, stores only, same accesses), over 2 GiB: a copy that spends
         # 1/read + 1/write per byte moves 2 / (1/read + 1/write) bytes of read + write per second.
-        pkg.check(hip.tcpxuCopyKernelTimed(dev, None, scratch.data_ptr(), 2 * n_copy, 3, 20, ctypes.byref(us)), "read timed")
+        pkg.check(benchlib.tcpxuCopyKernelTimed(dev, None, scratch.data_ptr(), 2 * n_copy, 3, 20, ctypes.byref(us)), "read timed")
         read_gbps = 2 * n_copy / us.value / 1e3
-        pkg.check(hip.tcpxuCopyKernelTimed(dev, scratch.data_ptr(), None, 2 * n_copy, 3, 20, ctypes.byref(us)), "fill timed")
+        pkg.check(benchlib.tcpxuCopyKernelTimed(dev, scratch.data_ptr(), None, 2 * n_copy, 3, 20, ctypes.byref(us)), "fill timed")
         write_gbps = 2 * n_copy / us.value / 1e3
         result["hbm_yardsticks"] = {
             "read_only_GBps": round(read_gbps, 1),
@@ -488,7 +525,7 @@ def main():
         del scratch
 
         result["other_configs"] = other_configs(pkg, torch, run)
-        result["launch_per_batch_1GiB"] = batch_kernel_line(pkg, hip, torch, dev)
+        result["launch_per_batch_1GiB"] = batch_kernel_line(pkg, benchlib, torch, dev)
 
     pkg.check(hip.tcpxuEngineDestroy(engine), "tcpxuEngineDestroy")
 
@@ -496,17 +533,51 @@ def main():
         result["plugin_path"] = plugin_path(pkg, hip, torch, workloads[: min(8, args.chunks)], pool)
 
     # ---- CPU baseline on this machine's host cores: rank 0, bounded sample ---------------------------------
-    threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16") or 16))
-    gbps_1, it1 = cpu_baseline(oracle, workloads[0], pool, 1, args.cpu_seconds)
-    gbps_t, itt = cpu_baseline(oracle, workloads[0], pool, threads, args.cpu_seconds)
+    # Threads: the cores this process may run on.  A GPU box shows every core of the host to os.cpu_count() while a
+    # one-GPU job is given a share of them (OMP_NUM_THREADS says how many), so that share is the "all cores" leg.
+    logical = os.cpu_count() or 1
+    try:
+        allowed = len(os.sched_getaffinity(0))
+    except (AttributeError, OSError):
+        allowed = logical
+    share = int(os.environ.get("OMP_NUM_THREADS", "0") or 0)
+    threads = max(1, min(allowed, share) if share > 0 else allowed)
+    gbps_1, it1 = cpu_baseline(oracle, workloads[0].descs, int(chunk_bytes), pool, 1, args.cpu_seconds)
+    gbps_t, itt = cpu_baseline(oracle, workloads[0].descs, int(chunk_bytes), pool, threads, args.cpu_seconds)
+    # The same from DRAM: 64 chunks in turn (64 descriptor lists, 512 MiB of destinations, pages from four copies of
+    # the pool, 1 GiB), so that neither side stays in the host's caches -- the care the GPU leg takes with HBM.
+    n_dram = min(64, args.chunks)
+    pool_copies = 4
+    big_pool = np.tile(pool, pool_copies)
+    parts = []
+    for c in range(n_dram):
+        d = np.array(workloads[c].descs, copy=True)
+        d["src_off"] += np.uint32((c % pool_copies) * pool.nbytes)
+        d["dst_off"] += np.uint64(c * int(chunk_bytes))
+        parts.append(d)
+    dram_descs = np.ascontiguousarray(np.concatenate(parts))
+    dram_t, it_dt = cpu_baseline(oracle, dram_descs, n_dram * int(chunk_bytes), big_pool, threads, args.cpu_seconds)
+    dram_1, it_d1 = cpu_baseline(oracle, dram_descs, n_dram * int(chunk_bytes), big_pool, 1, args.cpu_seconds)
+    del big_pool
     result["cpu_baseline"] = {
-        "value": round(gbps_t, 2),
+        "value": round(dram_t, 2),
         "unit": "GB/s",
         "cores": threads,
         "kind": "port",
-        "sample": "the same 8 MiB chunk (descriptor list 0), pool and destination in host DRAM, memcpy per descriptor, "
-        "descriptor list range-partitioned over %d threads, median of %d iterations" % (threads, itt),
-        "single_thread": {"value": round(gbps_1, 2), "cores": 1, "iterations": it1},
+        "sample": "%d chunks of 8 MiB in turn (%d descriptors, %d MiB of destinations, pages from %d copies of the 256 MiB pool), "
+        "all in host DRAM, memcpy per descriptor, descriptor list range-partitioned over %d threads, median of %d passes"
+        % (n_dram, len(dram_descs), n_dram * int(chunk_bytes) >> 20, pool_copies, threads, it_dt),
+        "host_logical_cpus": logical,
+        "cpus_this_process_may_use": allowed,
+        "cpu_share_of_the_job": share if share > 0 else None,
+        "single_thread": {"value": round(dram_1, 2), "cores": 1, "passes": it_d1},
+        "cache_resident": {
+            "what": "the same single 8 MiB chunk over and over (descriptor list 0): sources and destination stay in the host's caches",
+            "value": round(gbps_t, 2),
+            "cores": threads,
+            "iterations": itt,
+            "single_thread": {"value": round(gbps_1, 2), "cores": 1, "iterations": it1},
+        },
     }
     print(json.dumps(result))
     if not parity_ok:

@@ -102,19 +102,6 @@ void tcpxuVisibleFlush(void); /* orders the host's writes to such memory before 
 int tcpxuUnpackBatch(int device, const void* bounce_base, void* dst_base, const tcpxuLoadMeta* descs,
                      uint64_t n_descs, void* stream);
 
-/* Same launch bracketed by HIP events on its stream, repeated `iters` times after `warmup` untimed ones;
- * writes the mean duration of one launch in microseconds.  Measurement helper for benchmarks: the events
- * sit on the stream the kernel is launched on. */
-int tcpxuUnpackBatchTimed(int device, const void* bounce_base, void* dst_base, const tcpxuLoadMeta* descs,
-                          uint64_t n_descs, int warmup, int iters, double* mean_us);
-
-/* Plain device-to-device copy kernel of `bytes` (multiple of 16), timed the same way: the achievable-copy
- * yardstick printed beside the unpack figure, and the known-size kernel used to calibrate HBM counters.
- * With dst == NULL only the loads are issued (a read of `bytes`), with src == NULL only the stores (a fill):
- * what the memory system gives to each half of a copy on its own. */
-int tcpxuCopyKernelTimed(int device, void* dst, const void* src, size_t bytes, int warmup, int iters,
-                         double* mean_us);
-
 /* ---- (4) persistent unpack engine -------------------------------------------------------------------- */
 
 /* One engine per GPU: a persistent kernel that polls a submission ring in mapped host memory, unpacks every
@@ -128,8 +115,9 @@ typedef struct tcpxuEngineConfig {
   uint32_t workgroups;      /* persistent grid size, 0 = fill the GPU */
   uint32_t descs_per_ticket;/* descriptors one workgroup takes at a time (1..64); 0 = chosen per submission from
                                the backlog of descriptors not yet unpacked: 8 when the engine is idle (lowest
-                               latency) up to 32 when every workgroup has work queued (highest throughput); a
-                               submission of at most 32 descriptors stays whole once 8 or more are in flight */
+                               latency), 12, then 16 when every workgroup has work queued (highest throughput), and
+                               with a payload hint that tells of short fragments as many as make 64 KiB, up to 64;
+                               a submission of at most 32 descriptors stays whole once 8 or more are in flight */
   uint32_t spin_limit;      /* the kernel leaves by itself after this many consecutive empty polls of the ring
                                (about 1.2 us each) and is launched again by the next submission, so that a
                                device-wide synchronize never waits on an idle engine; 0 = default (400, about
@@ -159,63 +147,30 @@ int tcpxuEngineSubmit(tcpxuEngine* engine, const void* bounce_base, void* dst_ba
 int tcpxuEngineSubmitSized(tcpxuEngine* engine, const void* bounce_base, void* dst_base, const void* descs_dev,
                            uint32_t n_descs, uint64_t payload_bytes, void* done_flag_dev, uint64_t done_value);
 
+/* Limits: n_descs may not exceed 65536 tickets' worth -- 65536 x descs_per_ticket, or 524288 (65536 x 8) with
+ * descs_per_ticket = 0, and never 1048576: TCPXU_INVALID_ARGUMENT otherwise, decided on the host, nothing queued.
+ * TCPXU_INTERNAL_ERROR from a submit means the kernel stopped answering while the entry was already queued: the
+ * engine then refuses every later submit, so a caller cannot queue the same work twice by retrying. */
+
+/* The ticket arithmetic of the engine, on the host (no GPU needed): for an engine of `workgroups` workgroups and
+ * the given descs_per_ticket (0 = by backlog), a submission of n_descs descriptors and payload_bytes (0 = unknown)
+ * with `in_flight` submissions not yet completed (itself included) is handed out in *n_tickets tickets of
+ * *per_ticket descriptors; *max_descs is the most descriptors a submission may carry.  Outputs may be NULL.
+ * TCPXU_INVALID_ARGUMENT for an n_descs beyond that limit. */
+int tcpxuEngineTicketPlan(uint32_t workgroups, uint32_t descs_per_ticket, uint32_t in_flight, uint32_t n_descs,
+                          uint64_t payload_bytes, uint32_t* per_ticket, uint32_t* n_tickets, uint32_t* max_descs);
+
 /* Number of submissions the GPU has fully completed since creation (monotone; read from mapped memory). */
 int tcpxuEngineCompleted(tcpxuEngine* engine, uint64_t* completed);
 
 /* The configuration in effect (defaults resolved: actual grid size, ring size; ticket size 0 = by backlog). */
 int tcpxuEngineGetConfig(tcpxuEngine* engine, tcpxuEngineConfig* config);
 
+/* The GPU the engine was created on. */
+int tcpxuEngineDevice(tcpxuEngine* engine, int* device);
+
 /* 1 if the persistent kernel is running, 0 if stopped or away after being idle. */
 int tcpxuEngineRunning(tcpxuEngine* engine, int* running);
-
-/* ---- streaming driver (measurement helper) ------------------------------------------------------------ */
-
-/* One slot's worth of work for tcpxuEngineStream. */
-typedef struct tcpxuStreamItem {
-  const void* bounce_base;
-  void* dst_base;
-  const tcpxuLoadMeta* descs_host; /* descriptors in ordinary host memory */
-  uint32_t n_descs;                /* at most TCPXU_SLOT_PAGES */
-  uint32_t payload_bytes;          /* sum of the descriptors' lengths, 0 = unknown (see tcpxuEngineSubmitSized) */
-} tcpxuStreamItem;
-
-/* Slots the streaming driver can keep in flight: the unpack queues of eight receive comms. */
-#define TCPXU_STREAM_MAX_DEPTH (8 * TCPXU_QUEUE_DEPTH)
-
-/* Drives a started engine the way the plugin's proxy loop does, from one host thread, with no Python in the
- * loop: a mapped ring of `depth` slots (1..TCPXU_STREAM_MAX_DEPTH; TCPXU_QUEUE_DEPTH is one comm's unpack queue,
- * a multiple of it is that many comms taking turns) of TCPXU_SLOT_PAGES descriptors each; for every
- * item, in order: wait until the slot's previous occupant has completed, copy the item's descriptors into the
- * slot (the memcpy of src/net_tcpx.cc:1128-1130), publish it (src/net_tcpx.cc:1354-1357), and poll completion
- * words in FIFO order (the tcpxTest / tcpxIrecvConsumed cadence).  Writes the wall time from the first publish
- * to the last completion to *wall_us and, if latency_us is not NULL, each item's publish-to-completion-seen
- * time in microseconds to latency_us[0..n_items).  Returns TCPXU_INTERNAL_ERROR if nothing completes for
- * `stall_timeout_ms` milliseconds. */
-int tcpxuEngineStream(tcpxuEngine* engine, const tcpxuStreamItem* items, uint64_t n_items, uint32_t depth,
-                      uint32_t stall_timeout_ms, double* wall_us, double* latency_us);
-
-/* Same, with the first `warmup_items` items left out of *wall_us: the clock starts at the publish of item
- * `warmup_items` and stops at the last completion. */
-int tcpxuEngineStreamWarm(tcpxuEngine* engine, const tcpxuStreamItem* items, uint64_t n_items,
-                          uint64_t warmup_items, uint32_t depth, uint32_t stall_timeout_ms, double* wall_us,
-                          double* latency_us);
-
-/* tcpxuEngineStart + tcpxuEngineStream + tcpxuEngineStop in one call on a stopped engine, so that the
- * persistent kernel's launch covers exactly these items (warm-up included); *kernel_us is that launch's duration
- * from HIP events on the engine's stream (the figure a kernel trace shows for it), *wall_us as in
- * tcpxuEngineStreamWarm. */
-int tcpxuEngineRunTimed(tcpxuEngine* engine, const tcpxuStreamItem* items, uint64_t n_items,
-                        uint64_t warmup_items, uint32_t depth, uint32_t stall_timeout_ms, double* wall_us,
-                        double* kernel_us, double* latency_us);
-
-/* Like tcpxuEngineRunTimed, but *wall_us covers items [first_timed, first_timed + n_timed) from completion to
- * completion: the clock starts when item first_timed - 1 is seen completed (at the first publish if first_timed
- * is 0) and stops when item first_timed + n_timed - 1 is; items after that keep the queues full while the timed
- * ones finish.  This is the time the engine takes for n_timed items in steady state, however few they are;
- * *kernel_us is the whole launch as before. */
-int tcpxuEngineRunWindow(tcpxuEngine* engine, const tcpxuStreamItem* items, uint64_t n_items, uint64_t first_timed,
-                         uint64_t n_timed, uint32_t depth, uint32_t stall_timeout_ms, double* wall_us,
-                         double* kernel_us, double* latency_us);
 
 #ifdef __cplusplus
 }

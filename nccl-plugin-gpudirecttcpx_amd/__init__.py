@@ -1,8 +1,8 @@
 """MI355X-native receive-side unpack path of a GPUDirect-TCPX style net plugin: ctypes view of the C-ABI.
 
 This package holds no compute of its own.  It loads the in-tree shared libraries built from ``csrc/`` and
-exposes their C entry points (``include/tcpx_unpack_hip.h``, ``include/tcpx_synth.h``,
-``include/tcpx_plugin.h``) with argument types attached, so tests and the benchmark call exactly what a C or
+exposes their C entry points (``include/tcpx_unpack_hip.h``, ``include/tcpx_unpack_bench.h``,
+``include/tcpx_synth.h``, ``include/tcpx_plugin.h``) with argument types attached, so tests and the benchmark call exactly what a C or
 C++ host would call.  There is no CPU fallback: if a library is missing, loading raises.
 
 The directory name carries a hyphen, so it is imported through ``__graft_entry__.load_package()`` under the
@@ -124,31 +124,6 @@ _HIP_PROTOTYPES = {
         ctypes.c_int,
         [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p],
     ),
-    "tcpxuUnpackBatchTimed": (
-        ctypes.c_int,
-        [
-            ctypes.c_int,
-            ctypes.c_void_p,
-            ctypes.c_void_p,
-            ctypes.c_void_p,
-            ctypes.c_uint64,
-            ctypes.c_int,
-            ctypes.c_int,
-            ctypes.POINTER(ctypes.c_double),
-        ],
-    ),
-    "tcpxuCopyKernelTimed": (
-        ctypes.c_int,
-        [
-            ctypes.c_int,
-            ctypes.c_void_p,
-            ctypes.c_void_p,
-            ctypes.c_size_t,
-            ctypes.c_int,
-            ctypes.c_int,
-            ctypes.POINTER(ctypes.c_double),
-        ],
-    ),
     "tcpxuEngineCreate": (
         ctypes.c_int,
         [ctypes.c_int, ctypes.POINTER(EngineConfig), ctypes.POINTER(ctypes.c_void_p)],
@@ -184,6 +159,63 @@ _HIP_PROTOTYPES = {
     "tcpxuEngineCompleted": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint64)]),
     "tcpxuEngineRunning": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]),
     "tcpxuEngineGetConfig": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(EngineConfig)]),
+    "tcpxuEngineDevice": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]),
+    "tcpxuEngineTicketPlan": (
+        ctypes.c_int,
+        [
+            ctypes.c_uint32,
+            ctypes.c_uint32,
+            ctypes.c_uint32,
+            ctypes.c_uint32,
+            ctypes.c_uint64,
+            ctypes.POINTER(ctypes.c_uint32),
+            ctypes.POINTER(ctypes.c_uint32),
+            ctypes.POINTER(ctypes.c_uint32),
+        ],
+    ),
+}
+
+_BENCH_PROTOTYPES = {
+    "tcpxuBenchLastError": (ctypes.c_char_p, []),
+    "tcpxuCopyKernelLaunch": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "tcpxuEngineRunStamped": (
+        ctypes.c_int,
+        [
+            ctypes.c_void_p,
+            ctypes.POINTER(StreamItem),
+            ctypes.c_uint64,
+            ctypes.c_uint32,
+            ctypes.c_uint32,
+            ctypes.POINTER(ctypes.c_double),
+            ctypes.POINTER(ctypes.c_double),
+            ctypes.POINTER(ctypes.c_double),
+        ],
+    ),
+    "tcpxuUnpackBatchTimed": (
+        ctypes.c_int,
+        [
+            ctypes.c_int,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.c_uint64,
+            ctypes.c_int,
+            ctypes.c_int,
+            ctypes.POINTER(ctypes.c_double),
+        ],
+    ),
+    "tcpxuCopyKernelTimed": (
+        ctypes.c_int,
+        [
+            ctypes.c_int,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.c_size_t,
+            ctypes.c_int,
+            ctypes.c_int,
+            ctypes.POINTER(ctypes.c_double),
+        ],
+    ),
     "tcpxuEngineStream": (
         ctypes.c_int,
         [
@@ -407,6 +439,14 @@ def hip_layer():
     return _cache["hip"]
 
 
+def bench_layer():
+    """``libtcpxu_bench.so``: measurement helpers on top of the HIP layer (include/tcpx_unpack_bench.h)."""
+    if "bench" not in _cache:
+        hip_layer()  # its dependency, loaded first so that the symbols resolve whatever the search path
+        _cache["bench"] = _bind(_load("libtcpxu_bench.so"), _BENCH_PROTOTYPES)
+    return _cache["bench"]
+
+
 def synth_lib():
     if "synth" not in _cache:
         _cache["synth"] = _bind(_load("libtcpx_synth.so"), _SYNTH_PROTOTYPES)
@@ -430,7 +470,10 @@ class HipError(RuntimeError):
 
 def check(rc, fn="call"):
     if rc != SUCCESS:
-        raise HipError(fn, rc, hip_layer().tcpxuLastError().decode(errors="replace"))
+        msg = hip_layer().tcpxuLastError().decode(errors="replace")
+        if "bench" in _cache:
+            msg = (_cache["bench"].tcpxuBenchLastError().decode(errors="replace") + " | " + msg).strip(" |")
+        raise HipError(fn, rc, msg)
 
 
 class Workload:

@@ -62,7 +62,7 @@ constexpr uint32_t kMaxDescsPerTicket = 64;
 // slowest one).
 // (Descriptors per worker workgroup below 13, 18; written without the division, which the leader would pay for
 // on every submission.  backlog <= 2^20 and workers < 2^16 keep the products in 32 bits.)
-__device__ __forceinline__ uint32_t ticket_size_for(uint32_t backlog, uint32_t workers) {
+__host__ __device__ __forceinline__ uint32_t ticket_size_for(uint32_t backlog, uint32_t workers) {
   return backlog < 13u * workers ? 8u : backlog < 18u * workers ? 12u : 16u;
 }
 // Ticket size for one submission of n descriptors when `in_flight` submissions (this one included) are not yet
@@ -78,7 +78,7 @@ __device__ __forceinline__ uint32_t ticket_size_for(uint32_t backlog, uint32_t w
 // as comparisons: the leader runs this for every submission and a division costs it forty instructions.
 constexpr uint32_t kManyInFlight = 8, kSmallSubmission = 32;
 constexpr uint32_t kFullTicket = 16;
-__device__ __forceinline__ uint32_t full_ticket_size(uint32_t bytes, uint32_t n) {
+__host__ __device__ __forceinline__ uint32_t full_ticket_size(uint32_t bytes, uint32_t n) {
   static_assert(kFullTicket == 16 && kMaxDescsPerTicket == 64, "the steps below: 64 KiB / (bytes / n), in eights");
   const uint64_t b = bytes;  // n <= 2^20: the products need more than 32 bits
   return bytes == 0 || b >= 2731ull * n ? 16u
@@ -89,14 +89,22 @@ __device__ __forceinline__ uint32_t full_ticket_size(uint32_t bytes, uint32_t n)
          : b >= 1024ull * n             ? 56u
                                         : 64u;
 }
-__device__ __forceinline__ uint32_t ticket_size_for_submission(uint32_t in_flight, uint32_t n, uint32_t bytes,
-                                                               uint32_t workers) {
+__host__ __device__ __forceinline__ uint32_t ticket_size_for_submission(uint32_t in_flight, uint32_t n,
+                                                                        uint32_t bytes, uint32_t workers) {
   if (in_flight >= kManyInFlight && n <= kSmallSubmission) return kSmallSubmission;
   const uint64_t all = static_cast<uint64_t>(in_flight) * n;
   const uint32_t size = ticket_size_for(all > (1u << 20) ? (1u << 20) : static_cast<uint32_t>(all), workers);
   return size < kFullTicket ? size : full_ticket_size(bytes, n);
 }
 constexpr uint32_t kMaxDescsPerSubmission = 1u << 20;
+constexpr uint32_t kSmallestAdaptiveTicket = 8;  // the least ticket_size_for_submission returns
+// The most descriptors one submission may carry: all its tickets must fit the ticket ring at once, or the leader
+// could never hand it out (it defers a submission until the ring has room for all of its tickets).
+__host__ __device__ constexpr uint32_t max_descs_for(uint32_t fixed_per_ticket) {
+  const uint64_t smallest = fixed_per_ticket != 0 ? fixed_per_ticket : kSmallestAdaptiveTicket;
+  const uint64_t fit = smallest * kTicketRing;
+  return fit < kMaxDescsPerSubmission ? static_cast<uint32_t>(fit) : kMaxDescsPerSubmission;
+}
 constexpr uint32_t kStopReplicas = 64;
 constexpr uint32_t kPollEntries = 16;  // submission entries fetched per leader poll (16 B per lane)
 constexpr uint32_t kAuxTicketsDone = 32, kAuxHostStop = 33, kAuxJobsCompleted = 34;  // lanes of the auxiliary load
@@ -676,17 +684,33 @@ struct tcpxuEngine {
   uint32_t* job_target = nullptr;  // [ring_entries], device memory, leader-private
   uint64_t tail = 0;  // host copy
   bool launched = false;  // between a launch and the Stop that reaps it (the kernel may have left by itself)
+  bool failed = false;    // the kernel stopped answering (see tcpxuEngineSubmitSized); nothing more is accepted
   uint64_t launches = 0;
-  // Mapped slot ring of the streaming driver.  Allocated on first use and kept until the engine is destroyed:
-  // hipHostFree waits for every stream of the device, so nothing may be freed while the kernel runs.
-  void* stream_host = nullptr;
-  void* stream_dev = nullptr;
-  // Device memory the host can write: a copy of the descriptors of small stream items (kStageDescs each), or null.
-  void* stage_host = nullptr;
-  void* stage_dev = nullptr;
-  bool stage_tried = false;
   std::mutex mu;
 };
+
+// Engine calls arrive on threads that belong to somebody else (NCCL's proxy thread calls tcpxTest, which may have
+// to relaunch the kernel): the calling thread's current device is put back when the call returns.
+namespace {
+class DeviceScope {
+ public:
+  explicit DeviceScope(int device) {
+    if (hipGetDevice(&saved_) != hipSuccess) saved_ = -1;
+    rc_ = use_device(device);
+    if (saved_ == device) saved_ = -1;  // nothing to put back
+  }
+  ~DeviceScope() {
+    if (saved_ >= 0) (void)hipSetDevice(saved_);
+  }
+  int rc() const { return rc_; }
+  DeviceScope(const DeviceScope&) = delete;
+  DeviceScope& operator=(const DeviceScope&) = delete;
+
+ private:
+  int saved_ = -1;
+  int rc_ = TCPXU_SUCCESS;
+};
+}  // namespace
 
 static size_t ctl_bytes(uint32_t ring_entries) { return offsetof(HostCtl, ring) + sizeof(Record) * ring_entries; }
 
@@ -710,7 +734,8 @@ int tcpxuEngineCreate(int device, const tcpxuEngineConfig* config, tcpxuEngine**
     set_error("descs_per_ticket %u must be in [0,%u]", cfg.descs_per_ticket, kMaxDescsPerTicket);
     return TCPXU_INVALID_ARGUMENT;
   }
-  TCPXU_TRY(use_device(device));
+  DeviceScope scope(device);
+  TCPXU_TRY(scope.rc());
   const uint32_t cus = static_cast<uint32_t>(std::max(1, device_compute_units(device)));
   if (cfg.workgroups == 0) {
     // Fill the compute units, but leave a few wavefront slots free on each so that other kernels (copies, the
@@ -772,7 +797,8 @@ int tcpxuEngineCreate(int device, const tcpxuEngineConfig* config, tcpxuEngine**
 
 // Launches the kernel.  Caller holds e->mu; any previous launch has ended (its exit word is set).
 static int launch_locked(tcpxuEngine* e) {
-  TCPXU_TRY(use_device(e->device));
+  DeviceScope scope(e->device);
+  TCPXU_TRY(scope.rc());
   // Per-launch state: exit bookkeeping and stop words start from zero; positions and counters are kept.
   TCPXU_HIP(hipMemsetAsync(reinterpret_cast<uint8_t*>(e->st) + offsetof(DevState, exited_wgs), 0,
                            offsetof(DevState, tickets) - offsetof(DevState, exited_wgs), e->stream));
@@ -812,7 +838,8 @@ int tcpxuEngineStop(tcpxuEngine* e, double* elapsed_us) {
     set_error("engine is not started");
     return TCPXU_INVALID_USAGE;
   }
-  TCPXU_TRY(use_device(e->device));
+  DeviceScope scope(e->device);
+  TCPXU_TRY(scope.rc());
   std::atomic_thread_fence(std::memory_order_seq_cst);
   reinterpret_cast<std::atomic<uint64_t>*>(&e->ctl->stop)->store(1, std::memory_order_seq_cst);
   // Wait for the kernel's own exit word first, with a deadline: a stuck kernel then surfaces as an error
@@ -843,14 +870,12 @@ int tcpxuEngineDestroy(tcpxuEngine* e) {
     int rc = tcpxuEngineStop(e, nullptr);
     if (rc != TCPXU_SUCCESS) return rc;  // never free memory under a running kernel
   }
-  (void)hipSetDevice(e->device);
+  DeviceScope scope(e->device);
   if (e->ev_start) (void)hipEventDestroy(e->ev_start);
   if (e->ev_stop) (void)hipEventDestroy(e->ev_stop);
   if (e->stream) (void)hipStreamDestroy(e->stream);
   if (e->st) (void)hipFree(e->st);
   if (e->ctl) (void)hipHostFree(e->ctl);
-  if (e->stream_host) (void)hipHostFree(e->stream_host);
-  if (e->stage_host) (void)tcpxuVisibleFree(e->device, e->stage_host);
   delete e;
   return TCPXU_SUCCESS;
 }
@@ -870,11 +895,18 @@ int tcpxuEngineSubmitSized(tcpxuEngine* e, const void* bounce_base, void* dst_ba
     set_error("submit needs bounce, destination and a 16-byte aligned descriptor address");
     return TCPXU_INVALID_ARGUMENT;
   }
-  if (n_descs > kMaxDescsPerSubmission) {
-    set_error("%u descriptors in one submission exceed the limit of %u", n_descs, kMaxDescsPerSubmission);
+  // Refused here, on the host: a submission whose tickets can never all fit the ticket ring would sit at the head of
+  // the submission ring for ever, and the leader neither stops nor idles out with an entry waiting.
+  if (n_descs > max_descs_for(e->per_ticket)) {
+    set_error("%u descriptors in one submission exceed the limit of %u (tickets of %u at least, %u tickets in flight at most)",
+              n_descs, max_descs_for(e->per_ticket), e->per_ticket ? e->per_ticket : kSmallestAdaptiveTicket, kTicketRing);
     return TCPXU_INVALID_ARGUMENT;
   }
   std::lock_guard<std::mutex> lock(e->mu);
+  if (e->failed) {
+    set_error("the engine stopped answering earlier and accepts nothing more");
+    return TCPXU_INTERNAL_ERROR;
+  }
   const uint64_t head = reinterpret_cast<std::atomic<uint64_t>*>(&e->ctl->head)->load(std::memory_order_acquire);
   if (e->tail - head >= e->ring_entries) return kTcpxuInProgress;
   uint32_t p[kPayloadWords] = {};
@@ -903,7 +935,11 @@ int tcpxuEngineSubmitSized(tcpxuEngine* e, const void* bounce_base, void* dst_ba
       const auto t0 = std::chrono::steady_clock::now();
       while (host_load(&e->ctl->exiting) != 0 && host_load(&e->ctl->exited) == 0) {
         if (std::chrono::steady_clock::now() - t0 > std::chrono::seconds(5)) {
-          set_error("engine kernel announced that it is leaving and never did");
+          // The entry is in the ring and stays there: this is not "not submitted, try again".  The engine is
+          // marked failed so that the caller cannot queue the same work twice by retrying.
+          e->failed = true;
+          set_error("engine kernel announced that it is leaving and never did; the submission stays queued and the "
+                    "engine accepts nothing more");
           return TCPXU_INTERNAL_ERROR;
         }
       }
@@ -928,159 +964,38 @@ int tcpxuEngineGetConfig(tcpxuEngine* e, tcpxuEngineConfig* config) {
   return TCPXU_SUCCESS;
 }
 
+int tcpxuEngineDevice(tcpxuEngine* e, int* device) {
+  if (!e || !device) return TCPXU_INVALID_ARGUMENT;
+  *device = e->device;
+  return TCPXU_SUCCESS;
+}
+
+int tcpxuEngineTicketPlan(uint32_t workgroups, uint32_t descs_per_ticket, uint32_t in_flight, uint32_t n_descs,
+                          uint64_t payload_bytes, uint32_t* per_ticket, uint32_t* n_tickets, uint32_t* max_descs) {
+  if (workgroups < 2 || workgroups > (1u << 16) || descs_per_ticket > kMaxDescsPerTicket || in_flight == 0) {
+    set_error("ticket plan: 2..65536 workgroups, tickets of 0..%u, at least one submission in flight", kMaxDescsPerTicket);
+    return TCPXU_INVALID_ARGUMENT;
+  }
+  const uint32_t limit = max_descs_for(descs_per_ticket);
+  if (max_descs) *max_descs = limit;
+  if (n_descs > limit) {
+    set_error("%u descriptors in one submission exceed the limit of %u", n_descs, limit);
+    return TCPXU_INVALID_ARGUMENT;
+  }
+  const uint32_t bytes = payload_bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : static_cast<uint32_t>(payload_bytes);
+  const uint32_t per = descs_per_ticket != 0 ? descs_per_ticket
+                                             : ticket_size_for_submission(in_flight, n_descs, bytes, workgroups - 1);
+  if (per_ticket) *per_ticket = per;
+  if (n_tickets) *n_tickets = (n_descs + per - 1) / per;
+  return TCPXU_SUCCESS;
+}
+
 int tcpxuEngineRunning(tcpxuEngine* e, int* running) {
   if (!e || !running) return TCPXU_INVALID_ARGUMENT;
   std::lock_guard<std::mutex> lock(e->mu);
   *running = e->launched &&
              reinterpret_cast<std::atomic<uint64_t>*>(&e->ctl->exited)->load(std::memory_order_acquire) == 0;
   return TCPXU_SUCCESS;
-}
-
-// Descriptors of a stream item that are also copied into host-visible device memory, and the room per slot.
-constexpr uint32_t kStageDescs = 16;
-constexpr size_t kStageBytes = kStageDescs * sizeof(tcpxuLoadMeta);
-constexpr uint64_t kStageInFlight = 16;
-
-int tcpxuEngineStream(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_items, uint32_t depth,
-                      uint32_t stall_timeout_ms, double* wall_us, double* latency_us) {
-  return tcpxuEngineStreamWarm(e, items, n_items, 0, depth, stall_timeout_ms, wall_us, latency_us);
-}
-
-// The streaming loop.  The clock runs over items [first_timed, first_timed + n_timed): it stops when the last of
-// them is seen completed, and starts either at the publish of the first of them (`from_completion` false) or when
-// the item before them is seen completed (true: completion to completion, the time the engine takes for n_timed
-// items in a queue that was full before and, if more items follow, stays full after).
-static int stream_items(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_items, uint64_t first_timed,
-                        uint64_t n_timed, bool from_completion, uint32_t depth, uint32_t stall_timeout_ms,
-                        double* wall_us, double* latency_us) {
-  if (!e || !items || !wall_us || depth == 0 || depth > TCPXU_STREAM_MAX_DEPTH) return TCPXU_INVALID_ARGUMENT;
-  if (first_timed > n_items || n_timed > n_items - first_timed) return TCPXU_INVALID_ARGUMENT;
-  const uint64_t warmup_items = first_timed;
-  const uint64_t last_timed = first_timed + n_timed;  // one past
-  for (uint64_t i = 0; i < n_items; ++i) {
-    if (items[i].n_descs > TCPXU_SLOT_PAGES) {
-      set_error("stream item %llu has %u descriptors, a slot holds %d", static_cast<unsigned long long>(i),
-                items[i].n_descs, TCPXU_SLOT_PAGES);
-      return TCPXU_INVALID_ARGUMENT;
-    }
-  }
-  if (stall_timeout_ms == 0) stall_timeout_ms = 10000;
-  // Mapped block: `depth` completion words (one cache line each), then `depth` descriptor slots.
-  const size_t flag_stride = 64;
-  const size_t slot_bytes = sizeof(tcpxuLoadMeta) * TCPXU_SLOT_PAGES;
-  const size_t flags_bytes = flag_stride * TCPXU_STREAM_MAX_DEPTH;
-  if (!e->stream_host)
-    TCPXU_TRY(tcpxuMappedAlloc(e->device, flags_bytes + slot_bytes * TCPXU_STREAM_MAX_DEPTH, &e->stream_host,
-                               &e->stream_dev));
-  if (!e->stage_tried) {
-    // Optional: without it every item's descriptors are read from the mapped slot.
-    e->stage_tried = true;
-    if (tcpxuVisibleAlloc(e->device, kStageBytes * TCPXU_STREAM_MAX_DEPTH, &e->stage_host, &e->stage_dev) != TCPXU_SUCCESS)
-      e->stage_host = e->stage_dev = nullptr;
-  }
-  uint8_t* hb = static_cast<uint8_t*>(e->stream_host);
-  uint8_t* db = static_cast<uint8_t*>(e->stream_dev);
-  memset(hb, 0, flags_bytes);
-  using clock = std::chrono::steady_clock;
-  std::vector<clock::time_point> published(depth);
-  int rc = TCPXU_SUCCESS;
-  uint64_t next_submit = 0, next_done = 0;
-  auto t_begin = clock::now();
-  auto last_progress = t_begin;
-  auto t_end = t_begin;
-  while (next_done < n_items) {
-    bool progress = false;
-    // Reap completions in FIFO order.
-    while (next_done < next_submit) {
-      const uint32_t slot = static_cast<uint32_t>(next_done % depth);
-      auto* flag = reinterpret_cast<std::atomic<uint64_t>*>(hb + flag_stride * slot);
-      if (flag->load(std::memory_order_acquire) != next_done + 1) break;
-      const auto now = clock::now();
-      if (latency_us)
-        latency_us[next_done] = std::chrono::duration<double, std::micro>(now - published[slot]).count();
-      ++next_done;
-      if (from_completion && next_done == warmup_items) t_begin = now;
-      if (next_done <= last_timed) t_end = now;
-      progress = true;
-    }
-    // Publish while a slot is free.
-    while (next_submit < n_items && next_submit - next_done < depth) {
-      const uint32_t slot = static_cast<uint32_t>(next_submit % depth);
-      const tcpxuStreamItem& it = items[next_submit];
-      uint8_t* slot_host = hb + flags_bytes + slot_bytes * slot;
-      if (it.n_descs)
-        memcpy(slot_host, it.descs_host, sizeof(tcpxuLoadMeta) * it.n_descs);
-      published[slot] = clock::now();
-      if (next_submit == warmup_items && (!from_completion || warmup_items == 0)) t_begin = published[slot];
-      const void* descs_dev = db + flags_bytes + slot_bytes * slot;
-      if (e->stage_host && it.n_descs != 0 && it.n_descs <= kStageDescs && next_submit - next_done < kStageInFlight) {
-        // A small request with few ahead of it: its descriptors also go into the GPU's own memory, ahead of the
-        // submission.  (With many in flight the request waits in queues anyway, and the write through the BAR with
-        // its flush, about 0.2 us of host time, would cap the rate at which one thread can publish.)
-        memcpy(static_cast<uint8_t*>(e->stage_host) + kStageBytes * slot, it.descs_host, sizeof(tcpxuLoadMeta) * it.n_descs);
-        tcpxuVisibleFlush();
-        descs_dev = static_cast<uint8_t*>(e->stage_dev) + kStageBytes * slot;
-      }
-      rc = tcpxuEngineSubmitSized(e, it.bounce_base, it.dst_base, descs_dev, it.n_descs, it.payload_bytes,
-                                  db + flag_stride * slot, next_submit + 1);
-      if (rc == kTcpxuInProgress) {
-        rc = TCPXU_SUCCESS;
-        break;  // engine ring full: reap first
-      }
-      if (rc != TCPXU_SUCCESS) break;
-      ++next_submit;
-      progress = true;
-    }
-    if (rc != TCPXU_SUCCESS) break;
-    const auto now = clock::now();
-    if (progress) {
-      last_progress = now;
-    } else if (now - last_progress > std::chrono::milliseconds(stall_timeout_ms)) {
-      set_error("stream stalled: %llu of %llu items completed, %llu published",
-                static_cast<unsigned long long>(next_done), static_cast<unsigned long long>(n_items),
-                static_cast<unsigned long long>(next_submit));
-      rc = TCPXU_INTERNAL_ERROR;
-      break;
-    }
-  }
-  *wall_us = std::chrono::duration<double, std::micro>(t_end - t_begin).count();
-  return rc;
-}
-
-int tcpxuEngineStreamWarm(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_items, uint64_t warmup_items,
-                          uint32_t depth, uint32_t stall_timeout_ms, double* wall_us, double* latency_us) {
-  if (warmup_items > n_items) return TCPXU_INVALID_ARGUMENT;
-  return stream_items(e, items, n_items, warmup_items, n_items - warmup_items, false, depth, stall_timeout_ms, wall_us,
-                      latency_us);
-}
-
-int tcpxuEngineRunTimed(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_items, uint64_t warmup_items,
-                        uint32_t depth, uint32_t stall_timeout_ms, double* wall_us, double* kernel_us,
-                        double* latency_us) {
-  if (!e || !kernel_us) return TCPXU_INVALID_ARGUMENT;
-  // Touch the stream block before the launch so that no allocation happens while the kernel is timed.
-  if (!e->stream_host) {
-    const size_t bytes = (64 + sizeof(tcpxuLoadMeta) * TCPXU_SLOT_PAGES) * TCPXU_STREAM_MAX_DEPTH;
-    TCPXU_TRY(tcpxuMappedAlloc(e->device, bytes, &e->stream_host, &e->stream_dev));
-  }
-  TCPXU_TRY(tcpxuEngineStart(e));
-  const int rc = tcpxuEngineStreamWarm(e, items, n_items, warmup_items, depth, stall_timeout_ms, wall_us, latency_us);
-  const int rc_stop = tcpxuEngineStop(e, kernel_us);
-  return rc != TCPXU_SUCCESS ? rc : rc_stop;
-}
-
-int tcpxuEngineRunWindow(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_items, uint64_t first_timed,
-                         uint64_t n_timed, uint32_t depth, uint32_t stall_timeout_ms, double* wall_us,
-                         double* kernel_us, double* latency_us) {
-  if (!e || !kernel_us || n_timed == 0) return TCPXU_INVALID_ARGUMENT;
-  if (!e->stream_host) {
-    const size_t bytes = (64 + sizeof(tcpxuLoadMeta) * TCPXU_SLOT_PAGES) * TCPXU_STREAM_MAX_DEPTH;
-    TCPXU_TRY(tcpxuMappedAlloc(e->device, bytes, &e->stream_host, &e->stream_dev));
-  }
-  TCPXU_TRY(tcpxuEngineStart(e));
-  const int rc = stream_items(e, items, n_items, first_timed, n_timed, true, depth, stall_timeout_ms, wall_us, latency_us);
-  const int rc_stop = tcpxuEngineStop(e, kernel_us);
-  return rc != TCPXU_SUCCESS ? rc : rc_stop;
 }
 
 }  // extern "C"

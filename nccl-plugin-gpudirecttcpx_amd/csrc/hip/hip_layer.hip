@@ -71,58 +71,6 @@ __global__ __launch_bounds__(kWgThreads) void unpack_batch_kernel(const uint8_t*
   }
 }
 
-// Plain copy, 64 bytes per thread per step, with the payload accesses of the unpack kernels: the yardstick for
-// what a copy kernel reaches here.
-__global__ __launch_bounds__(kWgThreads) void copy_kernel(uint8_t* __restrict__ dst, const uint8_t* __restrict__ src,
-                                                          uint64_t n_vec) {
-  const uint64_t stride = static_cast<uint64_t>(gridDim.x) * kWgThreads;
-  for (uint64_t base = static_cast<uint64_t>(blockIdx.x) * kWgThreads * kVecPerLane; base < n_vec;
-       base += stride * kVecPerLane) {
-    u32x4 r[kVecPerLane];
-#pragma unroll
-    for (int k = 0; k < kVecPerLane; ++k) {
-      const uint64_t v = base + static_cast<uint64_t>(k) * kWgThreads + threadIdx.x;
-      if (v < n_vec) r[k] = load_vec_sys(src + (v << 4));
-    }
-#pragma unroll
-    for (int k = 0; k < kVecPerLane; ++k) {
-      const uint64_t v = base + static_cast<uint64_t>(k) * kWgThreads + threadIdx.x;
-      if (v < n_vec) store_vec_stream(dst + (v << 4), r[k]);
-    }
-  }
-}
-
-// The two halves of the copy on their own, with the same accesses: what the memory system gives to loads only and
-// to stores only.  The loads are folded into one word per lane that is stored only if it has a value it
-// practically never has, which keeps them from being optimised away without adding traffic.
-__global__ __launch_bounds__(kWgThreads) void read_kernel(const uint8_t* __restrict__ src, uint64_t n_vec,
-                                                          uint32_t* __restrict__ sink) {
-  const uint64_t stride = static_cast<uint64_t>(gridDim.x) * kWgThreads;
-  u32x4 acc = {0u, 0u, 0u, 0u};
-  for (uint64_t base = static_cast<uint64_t>(blockIdx.x) * kWgThreads * kVecPerLane; base < n_vec;
-       base += stride * kVecPerLane) {
-#pragma unroll
-    for (int k = 0; k < kVecPerLane; ++k) {
-      const uint64_t v = base + static_cast<uint64_t>(k) * kWgThreads + threadIdx.x;
-      if (v < n_vec) acc ^= load_vec_sys(src + (v << 4));
-    }
-  }
-  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9E3779B9u && (acc[0] + acc[1]) == 0x7F4A7C15u) *sink = acc[2];
-}
-
-__global__ __launch_bounds__(kWgThreads) void fill_kernel(uint8_t* __restrict__ dst, uint64_t n_vec) {
-  const uint64_t stride = static_cast<uint64_t>(gridDim.x) * kWgThreads;
-  const u32x4 x = {threadIdx.x, blockIdx.x, 0xA5A5A5A5u, 0x5A5A5A5Au};
-  for (uint64_t base = static_cast<uint64_t>(blockIdx.x) * kWgThreads * kVecPerLane; base < n_vec;
-       base += stride * kVecPerLane) {
-#pragma unroll
-    for (int k = 0; k < kVecPerLane; ++k) {
-      const uint64_t v = base + static_cast<uint64_t>(k) * kWgThreads + threadIdx.x;
-      if (v < n_vec) store_vec_stream(dst + (v << 4), x);
-    }
-  }
-}
-
 struct DeviceProps {
   bool valid = false;
   int compute_units = 0;
@@ -368,124 +316,6 @@ int tcpxuUnpackBatch(int device, const void* bounce_base, void* dst_base, const 
                      uint64_t n_descs, void* stream) {
   TCPXU_TRY(use_device(device));
   return launch_batch(device, bounce_base, dst_base, descs, n_descs, static_cast<hipStream_t>(stream));
-}
-
-// Mean of per-launch durations: every launch sits between its own pair of events on the launch stream, so
-// gaps between launches are not counted.
-static int time_launches(hipStream_t stream, int warmup, int iters, double* mean_us, int (*launch)(void*, hipStream_t),
-                         void* ctx) {
-  std::vector<hipEvent_t> ev(static_cast<size_t>(iters) * 2, nullptr);
-  int rc = TCPXU_SUCCESS;
-  for (int i = 0; i < warmup && rc == TCPXU_SUCCESS; ++i) rc = launch(ctx, stream);
-  for (auto& e : ev) {
-    if (rc == TCPXU_SUCCESS && hipEventCreate(&e) != hipSuccess) {
-      set_error("hipEventCreate failed");
-      rc = TCPXU_DEVICE_ERROR;
-    }
-  }
-  if (rc == TCPXU_SUCCESS && hipStreamSynchronize(stream) != hipSuccess) rc = TCPXU_DEVICE_ERROR;
-  for (int i = 0; i < iters && rc == TCPXU_SUCCESS; ++i) {
-    if (hipEventRecord(ev[2 * i], stream) != hipSuccess) rc = TCPXU_DEVICE_ERROR;
-    if (rc == TCPXU_SUCCESS) rc = launch(ctx, stream);
-    if (rc == TCPXU_SUCCESS && hipEventRecord(ev[2 * i + 1], stream) != hipSuccess) rc = TCPXU_DEVICE_ERROR;
-  }
-  if (rc == TCPXU_SUCCESS) {
-    hipError_t e = hipStreamSynchronize(stream);
-    if (e != hipSuccess) {
-      set_error("stream synchronize failed: %s", hipGetErrorString(e));
-      rc = TCPXU_DEVICE_ERROR;
-    }
-  }
-  if (rc == TCPXU_SUCCESS) {
-    double total_ms = 0.0;
-    for (int i = 0; i < iters; ++i) {
-      float ms = 0.f;
-      if (hipEventElapsedTime(&ms, ev[2 * i], ev[2 * i + 1]) != hipSuccess) rc = TCPXU_DEVICE_ERROR;
-      total_ms += ms;
-    }
-    *mean_us = total_ms * 1000.0 / iters;
-  }
-  for (auto e : ev)
-    if (e) (void)hipEventDestroy(e);
-  return rc;
-}
-
-struct BatchLaunch {
-  int device;
-  const void* bounce;
-  void* dst;
-  const tcpxuLoadMeta* descs;
-  uint64_t n;
-};
-
-int tcpxuUnpackBatchTimed(int device, const void* bounce_base, void* dst_base, const tcpxuLoadMeta* descs,
-                          uint64_t n_descs, int warmup, int iters, double* mean_us) {
-  if (!mean_us || iters <= 0 || warmup < 0 || n_descs == 0) return TCPXU_INVALID_ARGUMENT;
-  TCPXU_TRY(use_device(device));
-  hipStream_t stream;
-  TCPXU_HIP(hipStreamCreate(&stream));
-  BatchLaunch b{device, bounce_base, dst_base, descs, n_descs};
-  int rc = time_launches(
-      stream, warmup, iters, mean_us,
-      [](void* c, hipStream_t s) {
-        auto* b = static_cast<BatchLaunch*>(c);
-        return launch_batch(b->device, b->bounce, b->dst, b->descs, b->n, s);
-      },
-      &b);
-  (void)hipStreamDestroy(stream);
-  return rc;
-}
-
-struct CopyLaunch {
-  uint8_t* dst;
-  const uint8_t* src;
-  uint64_t n_vec;
-  uint32_t grid;
-  uint32_t* sink;
-};
-
-int tcpxuCopyKernelTimed(int device, void* dst, const void* src, size_t bytes, int warmup, int iters,
-                         double* mean_us) {
-  if (!mean_us || iters <= 0 || warmup < 0 || (!dst && !src) || bytes == 0 || bytes % 16 != 0 ||
-      reinterpret_cast<uintptr_t>(dst) % 16 != 0 || reinterpret_cast<uintptr_t>(src) % 16 != 0) {
-    set_error("copy kernel needs 16-byte aligned buffers (at least one of them) and a size that is a multiple of 16");
-    return TCPXU_INVALID_ARGUMENT;
-  }
-  TCPXU_TRY(use_device(device));
-  const uint64_t n_vec = bytes / 16;
-  const uint64_t per_wg = static_cast<uint64_t>(kWgThreads) * kVecPerLane;
-  const uint64_t cus = static_cast<uint64_t>(std::max(1, device_compute_units(device)));
-  const uint32_t grid = static_cast<uint32_t>(std::min<uint64_t>((n_vec + per_wg - 1) / per_wg, cus * 16));
-  uint32_t* sink = nullptr;
-  if (!dst) TCPXU_HIP(hipMalloc(reinterpret_cast<void**>(&sink), 64));
-  hipStream_t stream;
-  if (hipStreamCreate(&stream) != hipSuccess) {
-    (void)hipFree(sink);
-    set_error("hipStreamCreate failed");
-    return TCPXU_DEVICE_ERROR;
-  }
-  CopyLaunch c{static_cast<uint8_t*>(dst), static_cast<const uint8_t*>(src), n_vec, grid, sink};
-  int rc = time_launches(
-      stream, warmup, iters, mean_us,
-      [](void* p, hipStream_t s) {
-        auto* c = static_cast<CopyLaunch*>(p);
-        if (!c->dst) {
-          hipLaunchKernelGGL(read_kernel, dim3(c->grid), dim3(kWgThreads), 0, s, c->src, c->n_vec, c->sink);
-        } else if (!c->src) {
-          hipLaunchKernelGGL(fill_kernel, dim3(c->grid), dim3(kWgThreads), 0, s, c->dst, c->n_vec);
-        } else {
-          hipLaunchKernelGGL(copy_kernel, dim3(c->grid), dim3(kWgThreads), 0, s, c->dst, c->src, c->n_vec);
-        }
-        if (hipGetLastError() != hipSuccess) {
-          set_error("copy kernel launch failed");
-          return TCPXU_DEVICE_ERROR;
-        }
-        return TCPXU_SUCCESS;
-      },
-      &c);
-  (void)hipStreamDestroy(stream);
-  (void)hipFree(sink);
-  return rc;
 }
 
 }  // extern "C"

@@ -19,7 +19,7 @@ def pytest_configure(config):
 def _ensure_built():
     """Tests load what is built; they compile only if nothing is there."""
     pkg = graft.load_package()
-    needed = [os.path.join(pkg.LIB_DIR, n) for n in ("libtcpxu_hip.so", "libtcpx_synth.so", "libnccl-net.so")]
+    needed = [os.path.join(pkg.LIB_DIR, n) for n in ("libtcpxu_hip.so", "libtcpxu_bench.so", "libtcpx_synth.so", "libnccl-net.so")]
     needed.append(os.path.join(ROOT, "oracle", "liboracle.so"))
     if not all(os.path.exists(p) for p in needed):
         graft.build()
@@ -39,6 +39,11 @@ def oracle(pkg):
 @pytest.fixture(scope="session")
 def hip(pkg):
     return pkg.hip_layer()
+
+
+@pytest.fixture(scope="session")
+def benchlib(pkg):
+    return pkg.bench_layer()
 
 
 SENTINEL = 0xA5

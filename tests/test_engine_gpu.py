@@ -256,7 +256,7 @@ def test_engine_argument_errors(pkg, hip):
 
 
 @pytest.mark.parametrize("depth", [1, 5, 16, 64, 128])
-def test_engine_stream_depths(pkg, hip, oracle, depth):
+def test_engine_stream_depths(pkg, hip, oracle, depth, benchlib):
     """The streaming driver (mapped slot ring, warm-up + timed items in one launch) at 1 to 64 slots in flight:
     the leader then cuts tickets of 8 to 16 descriptors by backlog, and every size must give the oracle's bytes.
     Eight distinct 8 MiB chunks, each twice, so every destination is written by two passes of the ring."""
@@ -289,7 +289,7 @@ def test_engine_stream_depths(pkg, hip, oracle, depth):
     print("engine stream case: depth=%d items=%d" % (depth, len(flat)), flush=True)
     wall, kern = ctypes.c_double(), ctypes.c_double()
     lat = (ctypes.c_double * len(flat))()
-    rc = hip.tcpxuEngineRunTimed(e.h, items, len(flat), 4, depth, 20000, ctypes.byref(wall), ctypes.byref(kern), lat)
+    rc = benchlib.tcpxuEngineRunTimed(e.h, items, len(flat), 4, depth, 20000, ctypes.byref(wall), ctypes.byref(kern), lat)
     pkg.check(rc, "tcpxuEngineRunTimed")
     assert e.completed() == len(flat) and 0 < wall.value <= kern.value * 1.5 and min(lat) > 0
     e.destroy()
@@ -297,12 +297,12 @@ def test_engine_stream_depths(pkg, hip, oracle, depth):
     assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
     # more than TCPXU_STREAM_MAX_DEPTH slots is refused before anything is launched
     e = Engine(pkg, hip)
-    assert hip.tcpxuEngineRunTimed(e.h, items, 4, 0, 129, 1000, ctypes.byref(wall), ctypes.byref(kern), None) == pkg.INVALID_ARGUMENT
+    assert benchlib.tcpxuEngineRunTimed(e.h, items, 4, 0, 129, 1000, ctypes.byref(wall), ctypes.byref(kern), None) == pkg.INVALID_ARGUMENT
     e.destroy()
 
 
 @pytest.mark.parametrize("hint", ["true", "none", "tiny", "huge"])
-def test_engine_ticket_size_follows_the_payload_hint(pkg, hip, oracle, hint):
+def test_engine_ticket_size_follows_the_payload_hint(pkg, hip, oracle, hint, benchlib):
     """Ragged and empty fragments (the adversarial workload, 2 KiB a fragment on average) with 64 slots in flight:
     with the request's byte count given, the leader cuts tickets of up to 64 descriptors, without it tickets of
     16; a hint is only a hint, so a wrong one (far too small, far too large) must give the same bytes."""
@@ -339,7 +339,7 @@ def test_engine_ticket_size_follows_the_payload_hint(pkg, hip, oracle, hint):
     e = Engine(pkg, hip)
     print("engine hint case: %s, %d items" % (hint, len(items)), flush=True)
     wall, kern = ctypes.c_double(), ctypes.c_double()
-    rc = hip.tcpxuEngineRunTimed(e.h, items, len(items), 0, 64, 20000, ctypes.byref(wall), ctypes.byref(kern), None)
+    rc = benchlib.tcpxuEngineRunTimed(e.h, items, len(items), 0, 64, 20000, ctypes.byref(wall), ctypes.byref(kern), None)
     pkg.check(rc, "tcpxuEngineRunTimed")
     assert e.completed() == len(items)
     e.destroy()
@@ -406,7 +406,7 @@ def test_engine_bursts_around_the_idle_exit(pkg, hip, oracle):
 
 
 @pytest.mark.parametrize("depth", [3, 16, 128])
-def test_engine_storm_of_mixed_small_submissions(pkg, hip, oracle, depth):
+def test_engine_storm_of_mixed_small_submissions(pkg, hip, oracle, depth, benchlib):
     """Thousands of submissions of 0 to 300 ragged fragments in random order, `depth` of them in flight: runs of
     submissions that the leader turns into tickets sixteen at a time are broken at every position by empty ones,
     by ones just over the one-ticket limit and by ones that need many tickets; each submission owns a stretch of
@@ -449,14 +449,14 @@ def test_engine_storm_of_mixed_small_submissions(pkg, hip, oracle, depth):
     print("engine storm case: depth=%d submissions=%d descriptors=%d" % (depth, len(subs), len(descs)), flush=True)
     wall, kern = ctypes.c_double(), ctypes.c_double()
     lat = (ctypes.c_double * len(subs))()
-    pkg.check(hip.tcpxuEngineRunTimed(e.h, items, len(subs), 0, depth, 20000, ctypes.byref(wall), ctypes.byref(kern), lat), "tcpxuEngineRunTimed")
+    pkg.check(benchlib.tcpxuEngineRunTimed(e.h, items, len(subs), 0, depth, 20000, ctypes.byref(wall), ctypes.byref(kern), lat), "tcpxuEngineRunTimed")
     assert e.completed() == len(subs) and min(lat) > 0
     e.destroy()
     got = dst_d.cpu().numpy()
     assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
 
 
-def test_engine_run_window_times_the_middle_of_a_stream(pkg, hip, oracle):
+def test_engine_run_window_times_the_middle_of_a_stream(pkg, hip, oracle, benchlib):
     """tcpxuEngineRunWindow: warm-up items, timed items and a tail in one launch; the clock covers the timed ones
     from completion to completion, so it is shorter than the launch, and every item's bytes are the oracle's."""
     import torch
@@ -487,13 +487,13 @@ def test_engine_run_window_times_the_middle_of_a_stream(pkg, hip, oracle):
     print("engine window case: items=%d" % n, flush=True)
     wall, kern = ctypes.c_double(), ctypes.c_double()
     lat = (ctypes.c_double * n)()
-    pkg.check(hip.tcpxuEngineRunWindow(e.h, items, n, n // 4, n // 2, 8, 20000, ctypes.byref(wall), ctypes.byref(kern), lat), "tcpxuEngineRunWindow")
+    pkg.check(benchlib.tcpxuEngineRunWindow(e.h, items, n, n // 4, n // 2, 8, 20000, ctypes.byref(wall), ctypes.byref(kern), lat), "tcpxuEngineRunWindow")
     assert e.completed() == n and 0 < wall.value < kern.value and min(lat) > 0
     first = ctypes.c_double()
-    pkg.check(hip.tcpxuEngineRunWindow(e.h, items, n, 0, n, 8, 20000, ctypes.byref(first), ctypes.byref(kern), None), "tcpxuEngineRunWindow")
+    pkg.check(benchlib.tcpxuEngineRunWindow(e.h, items, n, 0, n, 8, 20000, ctypes.byref(first), ctypes.byref(kern), None), "tcpxuEngineRunWindow")
     assert wall.value < first.value <= kern.value  # the whole stream takes longer than its middle half
-    assert hip.tcpxuEngineRunWindow(e.h, items, n, n // 2, n, 8, 1000, ctypes.byref(wall), ctypes.byref(kern), None) == pkg.INVALID_ARGUMENT
-    assert hip.tcpxuEngineRunWindow(e.h, items, n, 0, 0, 8, 1000, ctypes.byref(wall), ctypes.byref(kern), None) == pkg.INVALID_ARGUMENT
+    assert benchlib.tcpxuEngineRunWindow(e.h, items, n, n // 2, n, 8, 1000, ctypes.byref(wall), ctypes.byref(kern), None) == pkg.INVALID_ARGUMENT
+    assert benchlib.tcpxuEngineRunWindow(e.h, items, n, 0, 0, 8, 1000, ctypes.byref(wall), ctypes.byref(kern), None) == pkg.INVALID_ARGUMENT
     e.destroy()
     got = dst_d.cpu().numpy()
     assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)

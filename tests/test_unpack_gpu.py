@@ -169,7 +169,7 @@ def test_argument_errors(pkg, hip):
     pkg.check(hip.tcpxuArenaDestroy(0, p), "arena destroy")
 
 
-def test_yardstick_kernels_copy_read_fill(pkg, hip):
+def test_yardstick_kernels_copy_read_fill(pkg, hip, benchlib):
     """The measurement helpers behind the benchmark's copy, read-only and write-only figures: the copy is exact
     (odd size in vectors, so the last workgroup is partial), the read leaves its source alone, the fill writes
     every vector of the range and nothing beyond it."""
@@ -180,17 +180,17 @@ def test_yardstick_kernels_copy_read_fill(pkg, hip):
     dst = torch.full((n + 64,), SENTINEL, dtype=torch.uint8, device="cuda:0")
     keep = src.clone()
     us = ctypes.c_double()
-    pkg.check(hip.tcpxuCopyKernelTimed(0, dst.data_ptr(), src.data_ptr(), n, 1, 3, ctypes.byref(us)), "copy")
+    pkg.check(benchlib.tcpxuCopyKernelTimed(0, dst.data_ptr(), src.data_ptr(), n, 1, 3, ctypes.byref(us)), "copy")
     assert us.value > 0 and torch.equal(dst[:n], src) and bool((dst[n:] == SENTINEL).all())
-    pkg.check(hip.tcpxuCopyKernelTimed(0, None, src.data_ptr(), n, 1, 3, ctypes.byref(us)), "read")
+    pkg.check(benchlib.tcpxuCopyKernelTimed(0, None, src.data_ptr(), n, 1, 3, ctypes.byref(us)), "read")
     assert us.value > 0 and torch.equal(src, keep)
     dst.fill_(SENTINEL)
-    pkg.check(hip.tcpxuCopyKernelTimed(0, dst.data_ptr(), None, n, 1, 3, ctypes.byref(us)), "fill")
+    pkg.check(benchlib.tcpxuCopyKernelTimed(0, dst.data_ptr(), None, n, 1, 3, ctypes.byref(us)), "fill")
     words = dst[:n].view(torch.int32).view(-1, 4)
     assert us.value > 0 and bool((words[:, 2] == -0x5A5A5A5B).all()) and bool((words[:, 3] == 0x5A5A5A5A).all())
     assert bool((dst[n:] == SENTINEL).all())
-    assert hip.tcpxuCopyKernelTimed(0, None, None, n, 1, 3, ctypes.byref(us)) == pkg.INVALID_ARGUMENT
-    assert hip.tcpxuCopyKernelTimed(0, dst.data_ptr(), src.data_ptr(), n + 8, 1, 3, ctypes.byref(us)) == pkg.INVALID_ARGUMENT
+    assert benchlib.tcpxuCopyKernelTimed(0, None, None, n, 1, 3, ctypes.byref(us)) == pkg.INVALID_ARGUMENT
+    assert benchlib.tcpxuCopyKernelTimed(0, dst.data_ptr(), src.data_ptr(), n + 8, 1, 3, ctypes.byref(us)) == pkg.INVALID_ARGUMENT
 
 
 def test_batch_launches_replayed_from_a_hip_graph(pkg, hip, oracle):
