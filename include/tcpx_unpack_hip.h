@@ -172,6 +172,23 @@ int tcpxuEngineDevice(tcpxuEngine* engine, int* device);
 /* 1 if the persistent kernel is running, 0 if stopped or away after being idle. */
 int tcpxuEngineRunning(tcpxuEngine* engine, int* running);
 
+/* ---- (5) one slot without any allocation ---------------------------------------------------------------- */
+
+/* tcpxuEngineSubmit for callers that cannot allocate and cannot keep a persistent kernel: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.
+ * Unpacks one slot -- `n_descs` descriptors (at most TCPXU_SLOT_PAGES = 2048; more is TCPXU_INVALID_ARGUMENT and
+ * nothing is launched) at `descs_dev`, from `bounce_base` into `dst_base` -- with ordinary launches on `stream`
+ * (a hipStream_t, NULL = the default stream): the engine's worker workgroups over tickets that a small kernel
+ * writes first, and the workgroup that finishes the slot's last ticket stores `done_value` to `*done_flag_dev`
+ * (device-visible 8-byte word, e.g. the alias of mapped host memory; may be NULL when stream order is all the
+ * caller needs).  Asynchronous.  It calls no hipMalloc, hipFree or other allocating routine: ticket records,
+ * ticket cursor and done counters live in a fixed array of device memory inside the library (17 KiB, held by
+ * every GPU the library runs on until the process ends), which every call on a GPU shares and which each call
+ * clears with its own first kernel.  Calls that overlap on one GPU (two streams, two threads) race on that
+ * array: issue them on one stream, or order them otherwise. */
+int tcpxuUnpackSlotNoAlloc(int device, const void* bounce_base, void* dst_base, const void* descs_dev,
+                           uint32_t n_descs, void* done_flag_dev, uint64_t done_value, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -156,6 +156,19 @@ _HIP_PROTOTYPES = {
             ctypes.c_uint64,
         ],
     ),
+    "tcpxuUnpackSlotNoAlloc": (
+        ctypes.c_int,
+        [
+            ctypes.c_int,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.c_uint32,
+            ctypes.c_void_p,
+            ctypes.c_uint64,
+            ctypes.c_void_p,
+        ],
+    ),
     "tcpxuEngineCompleted": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint64)]),
     "tcpxuEngineRunning": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]),
     "tcpxuEngineGetConfig": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(EngineConfig)]),

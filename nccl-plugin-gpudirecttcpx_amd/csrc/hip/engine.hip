@@ -139,6 +139,8 @@ struct alignas(256) StopWord {
 };
 
 struct DevState {  // device memory
+  static constexpr uint32_t kTickets = kTicketRing;
+  static constexpr uint32_t kStops = kStopReplicas;
   alignas(64) uint64_t ticket_head;     // next ticket number to claim
   alignas(64) uint64_t tickets_done;    // tickets whose payload is written
   alignas(64) uint64_t jobs_completed;  // submissions completed since creation
@@ -150,6 +152,23 @@ struct DevState {  // device memory
   alignas(64) Record tickets[kTicketRing];
   // uint32_t jobs_done[ring_entries], then uint32_t job_target[ring_entries] follow
 };
+
+// The same roles for one slot handed out by one ordinary launch (tcpxuUnpackSlotNoAlloc): tickets 0 .. n-1 are
+// written by a small kernel before the workers start, there is no leader and no stop word is ever raised.
+constexpr uint32_t kOneShotTicketSize = 8;  // one fragment per copy wavefront: the most workgroups per slot
+constexpr uint32_t kOneShotTickets = TCPXU_SLOT_PAGES / kOneShotTicketSize;
+struct OneShotState {
+  static constexpr uint32_t kTickets = kOneShotTickets;
+  static constexpr uint32_t kStops = 1;
+  alignas(64) uint64_t ticket_head;
+  alignas(64) uint64_t tickets_done;
+  alignas(64) uint64_t jobs_completed;
+  alignas(64) uint32_t jobs_done[16];  // [0]: tickets of the slot counted so far
+  alignas(64) uint64_t unused_flag;    // completion word of a caller that passed none
+  alignas(256) StopWord stop[kStops];
+  alignas(64) Record tickets[kOneShotTickets];
+};
+static_assert((kOneShotTickets & (kOneShotTickets - 1)) == 0, "ticket numbers are masked");
 
 // ---- scoped memory operations -------------------------------------------------------------------------------------
 #define SYS __HIP_MEMORY_SCOPE_SYSTEM
@@ -406,9 +425,10 @@ __device__ __forceinline__ uint32_t lane_shift(uint32_t v, uint32_t from_lane) {
 
 // Fetcher: look once at the slot of ticket number `ticket` (one 64-byte read, with this workgroup's stop word in
 // the same round trip).  Returns 1 and stages the ticket if it is there.  Wave-uniform.
-__device__ uint32_t try_fetch_ticket(DevState* st, const uint32_t* stop_word, uint64_t ticket, Stage* stage,
+template <typename State>
+__device__ uint32_t try_fetch_ticket(State* st, const uint32_t* stop_word, uint64_t ticket, Stage* stage,
                                      uint32_t lane, bool* stop_up) {
-  const Record* rec = &st->tickets[ticket & (kTicketRing - 1)];
+  const Record* rec = &st->tickets[ticket & (State::kTickets - 1)];
   const uint32_t expect = static_cast<uint32_t>(ticket + 1);
   uint32_t word = 0;
   if (lane < 16) word = sys_load(&rec->w[lane]);
@@ -468,7 +488,8 @@ __device__ uint32_t try_fetch_ticket(DevState* st, const uint32_t* stop_word, ui
 
 // Counts a finished ticket (all of its payload is in memory); the last ticket of a submission publishes the
 // completion word.
-__device__ void retire_ticket(DevState* st, uint32_t* jobs_done, const Stage* stage, uint32_t lane) {
+template <typename State>
+__device__ void retire_ticket(State* st, uint32_t* jobs_done, const Stage* stage, uint32_t lane) {
   if (lane == 0) {
     const uint32_t job = (stage->payload[10] & ~kOnlyTicket) >> 8;
     const uint32_t target = stage->payload[11];
@@ -552,7 +573,12 @@ __device__ void copy_ticket(const Stage* stage, uint32_t wave, uint32_t lane, ui
   }
 }
 
-__device__ void worker_loop(DevState* st, uint32_t* jobs_done, uint32_t flags) {
+// `ticket_limit`: ticket numbers from this one on do not exist and end the workgroup that claims one (the engine
+// passes none: its workgroups leave by the stop words); `look_limit`: looks at a ticket that is not there after
+// which the workgroup gives up (0 = never, the engine's workers wait for the leader as long as it lives).
+template <typename State>
+__device__ void worker_loop(State* st, uint32_t* jobs_done, uint32_t flags, uint64_t ticket_limit,
+                            uint32_t look_limit) {
   __shared__ Stage stages[2];
   __shared__ uint32_t s_waves_done;  // copy wavefronts that have finished (and drained) a ticket, running total
   __shared__ uint32_t s_waves_on_last;  // copy wavefronts that have turned to their last fragment of a ticket, ditto
@@ -577,7 +603,7 @@ __device__ void worker_loop(DevState* st, uint32_t* jobs_done, uint32_t flags) {
     // left of the copy then takes about as long as the pick-up, so neither waits for the other.  (flags bit 1
     // clear: claim only when the copy has finished; bit 0 set: claim right away while tickets are queueing up,
     // i.e. the previous ticket was already there at the first look.)
-    const uint32_t* stop_word = &st->stop[blockIdx.x % kStopReplicas].value;
+    const uint32_t* stop_word = &st->stop[blockIdx.x % State::kStops].value;
     uint32_t staged = 0;
     bool eager = false;
     const bool allow_eager = (flags & 1u) != 0;
@@ -594,11 +620,16 @@ __device__ void worker_loop(DevState* st, uint32_t* jobs_done, uint32_t flags) {
       if (lane == 0) t = __hip_atomic_fetch_add(&st->ticket_head, 1ull, __ATOMIC_RELAXED, SYS);
       const uint64_t ticket = bcast64(t, 0);
       bool give_up = false, stop_before = false, first_look = true;
-      uint32_t backoff = 1;
+      uint32_t backoff = 1, looks = 0;
       for (;;) {
         bool stop_up = false;
-        if (try_fetch_ticket(st, stop_word, ticket, next, lane, &stop_up)) {
+        if (ticket < ticket_limit && try_fetch_ticket(st, stop_word, ticket, next, lane, &stop_up)) {
           eager = first_look && allow_eager;
+          break;
+        }
+        if (ticket >= ticket_limit || (look_limit != 0 && ++looks >= look_limit)) {
+          give_up = true;
+          if (lane == 0) next->go = 0;
           break;
         }
         if (stop_before) {
@@ -646,7 +677,7 @@ __global__ __launch_bounds__(kEngineThreads) void unpack_engine_kernel(HostCtl* 
   if (blockIdx.x == 0) {
     if (threadIdx.x < kWaveLanes) leader_loop(ctl, st, jobs_done, job_target, ring_mask, per_ticket, spin_limit);
   } else {
-    worker_loop(st, jobs_done, flags);
+    worker_loop(st, jobs_done, flags, ~0ull, 0u);
   }
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -661,6 +692,52 @@ __global__ __launch_bounds__(kEngineThreads) void unpack_engine_kernel(HostCtl* 
       sys_store(&ctl->exited, static_cast<uint64_t>(sys_load(&st->exit_reason)));
     }
   }
+}
+
+// ---- one slot, one ordinary launch, nothing allocated ---------------------------------------------------------------
+// Scratch memory of tcpxuUnpackSlotNoAlloc: what the engine keeps in the DevState it allocates (ticket records, the
+// ticket cursor, the done counters), for one slot, held by every GPU the library runs on until the process ends.
+// In host code this name is only a handle for hipGetSymbolAddress; kernels get the address it returns.
+static __device__ __align__(256) unsigned char scratch[sizeof(OneShotState)];
+
+// Writes the slot's tickets (what the leader does for a submission) and clears the counters; with no descriptors
+// it completes the slot itself.  One workgroup of kOneShotTickets threads, thread t writes ticket t.
+__global__ __launch_bounds__(kOneShotTickets) void oneshot_prepare_kernel(OneShotState* st, uint64_t bounce,
+                                                                         uint64_t dst, uint64_t descs,
+                                                                         uint32_t n_descs, uint64_t done_flag,
+                                                                         uint64_t done_value) {
+  const uint32_t t = threadIdx.x;
+  if (done_flag == 0) done_flag = reinterpret_cast<uint64_t>(&st->unused_flag);
+  if (t == 0) {
+    sys_store(&st->ticket_head, static_cast<uint64_t>(0));
+    sys_store(&st->tickets_done, static_cast<uint64_t>(0));
+    sys_store(&st->jobs_completed, static_cast<uint64_t>(0));
+    sys_store(&st->jobs_done[0], 0u);
+    sys_store(&st->stop[0].value, 0u);
+    if (n_descs == 0) sys_store(reinterpret_cast<uint64_t*>(done_flag), done_value);
+  }
+  const uint32_t nt = (n_descs + kOneShotTicketSize - 1) / kOneShotTicketSize;
+  if (t >= nt) return;
+  const uint64_t d = descs + static_cast<uint64_t>(t) * kOneShotTicketSize * sizeof(tcpxuLoadMeta);
+  const uint32_t count = std::min(kOneShotTicketSize, n_descs - t * kOneShotTicketSize);
+  const uint32_t payload[kPayloadWords] = {
+      static_cast<uint32_t>(bounce),    static_cast<uint32_t>(bounce >> 32),    static_cast<uint32_t>(dst),
+      static_cast<uint32_t>(dst >> 32), static_cast<uint32_t>(d),               static_cast<uint32_t>(d >> 32),
+      static_cast<uint32_t>(done_flag), static_cast<uint32_t>(done_flag >> 32), static_cast<uint32_t>(done_value),
+      static_cast<uint32_t>(done_value >> 32), count | (nt == 1 ? kOnlyTicket : 0u) /* job slot 0 */, nt};
+  const uint32_t stamp = t + 1u;
+  uint8_t* rec = reinterpret_cast<uint8_t*>(&st->tickets[t]);
+#pragma unroll
+  for (int sector = 0; sector < 4; ++sector)
+    store_vec_sys(rec + 16 * sector, u32x4{payload[3 * sector], payload[3 * sector + 1], payload[3 * sector + 2], stamp});
+}
+
+// The engine's worker workgroups over tickets 0 .. n_tickets-1 and nothing else: a workgroup that claims a number
+// beyond them leaves.  The tickets were written by the launch before this one on the same stream, so the first
+// look finds each; the look limit only keeps a misuse (two calls overlapping on one GPU) from spinning for ever.
+__global__ __launch_bounds__(kEngineThreads) void unpack_oneshot_kernel(OneShotState* st, uint32_t flags,
+                                                                    uint32_t n_tickets) {
+  worker_loop(st, st->jobs_done, flags, n_tickets, 1u << 16);
 }
 
 }  // namespace
@@ -987,6 +1064,59 @@ int tcpxuEngineTicketPlan(uint32_t workgroups, uint32_t descs_per_ticket, uint32
                                              : ticket_size_for_submission(in_flight, n_descs, bytes, workgroups - 1);
   if (per_ticket) *per_ticket = per;
   if (n_tickets) *n_tickets = (n_descs + per - 1) / per;
+  return TCPXU_SUCCESS;
+}
+
+// The address of `scratch` on each device, asked for once per device with that device current.
+static OneShotState* g_scratch_ptr[kMaxDevices];
+static std::mutex g_scratch_mu;
+
+static int scratch_for(int device, OneShotState** out) {
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[device]) {
+    void* p = nullptr;
+    TCPXU_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p || reinterpret_cast<uintptr_t>(p) % 256 != 0) {
+      set_error("scratch symbol resolved to %p on device %d", p, device);
+      return TCPXU_INTERNAL_ERROR;
+    }
+    g_scratch_ptr[device] = static_cast<OneShotState*>(p);
+  }
+  *out = g_scratch_ptr[device];
+  return TCPXU_SUCCESS;
+}
+
+int tcpxuUnpackSlotNoAlloc(int device, const void* bounce_base, void* dst_base, const void* descs_dev,
+                           uint32_t n_descs, void* done_flag_dev, uint64_t done_value, void* stream) {
+  if (n_descs > TCPXU_SLOT_PAGES) {
+    set_error("%u descriptors exceed the %d of one slot, the most this entry point's fixed scratch memory serves",
+              n_descs, TCPXU_SLOT_PAGES);
+    return TCPXU_INVALID_ARGUMENT;
+  }
+  if (reinterpret_cast<uintptr_t>(done_flag_dev) % 8 != 0 || (done_flag_dev && done_value == 0)) {
+    set_error("the completion word must be 8-byte aligned and its value nonzero");
+    return TCPXU_INVALID_ARGUMENT;
+  }
+  if (n_descs > 0 && (!bounce_base || !dst_base || !descs_dev || reinterpret_cast<uintptr_t>(descs_dev) % 16 != 0)) {
+    set_error("unpack needs bounce, destination and a 16-byte aligned descriptor address");
+    return TCPXU_INVALID_ARGUMENT;
+  }
+  DeviceScope scope(device);
+  TCPXU_TRY(scope.rc());
+  OneShotState* st = nullptr;
+  TCPXU_TRY(scratch_for(device, &st));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(oneshot_prepare_kernel, dim3(1), dim3(kOneShotTickets), 0, s, st,
+                     reinterpret_cast<uint64_t>(bounce_base), reinterpret_cast<uint64_t>(dst_base),
+                     reinterpret_cast<uint64_t>(descs_dev), n_descs, reinterpret_cast<uint64_t>(done_flag_dev), done_value);
+  TCPXU_HIP(hipGetLastError());
+  if (n_descs == 0) return TCPXU_SUCCESS;
+  const uint32_t n_tickets = (n_descs + kOneShotTicketSize - 1) / kOneShotTicketSize;
+  const uint32_t cus = static_cast<uint32_t>(std::max(1, device_compute_units(device)));
+  const uint32_t grid = std::min(n_tickets, 2u * cus);
+  // flags: fetchers claim their next ticket when every copy wavefront is on its last fragment; idle backoff cap 2
+  hipLaunchKernelGGL(unpack_oneshot_kernel, dim3(grid), dim3(kEngineThreads), 0, s, st, 2u | (2u << 8), n_tickets);
+  TCPXU_HIP(hipGetLastError());
   return TCPXU_SUCCESS;
 }
 
