@@ -134,6 +134,14 @@ ssize_t process_recv_cmsg(struct msghdr* msg, DataPipe* p, int offset, uint64_t 
         continue;
       }
     }
+    // The token list is the slot's, one per flow, and a request may put several chunks on one flow: it is full
+    // when it holds as many runs as a slot holds descriptors.  (The reference zeroes the count per task and so
+    // never gets here; it also forgets the earlier chunks' pages.)
+    if (*p->pgtok_cnt >= static_cast<size_t>(kSlotPages)) {
+      WARN("flow holds %zu page-token runs for one request, the most a slot records; failstop", *p->pgtok_cnt);
+      *result = fail_stop("too many page-token runs on one flow of a request");
+      return -1;
+    }
     p->pgtoks[*p->pgtok_cnt] = PageToken{v.frag_token, 1};
     (*p->pgtok_cnt)++;
   }

@@ -2,13 +2,16 @@
 //
 // Call pattern (NCCL's receive proxy, or a test driver in its place):
 //   irecv -> test* -> [consume the data] -> iflush? -> irecvConsumed
-// What differs from the reference by design: a request reports done=1 only after the GPU engine has written its
-// completion word, i.e. after the payload is in the receive buffer -- in the reference done=1 means "descriptor
-// count published" and NCCL's own kernel does the copy later.  Everything else (states, order checks, result
-// codes) follows src/net_tcpx.cc.
+// Who copies is a switch (NCCL_GPUDIRECTTCPX_AMD_DEVICE_TYPE).  "host" (default): the plugin advertises an
+// ordinary host-driven network, its GPU engine unpacks every request and a request reports done=1 only after the
+// engine has written its completion word, i.e. after the payload is in the receive buffer.  "unpack": the
+// reference's division of labour -- done=1 means "descriptor count published" (src/net_tcpx.cc:1354-1357), the
+// device handle is advertised and the caller's own kernel does the copy; the engine is never started.
+// Everything else (states, order checks, result codes) follows src/net_tcpx.cc.
 #include <errno.h>
 #include <limits.h>
 #include <sched.h>
+#include <strings.h>
 
 #include <algorithm>
 #include <atomic>
@@ -110,6 +113,19 @@ void parse_sched_alg() {
   } else {
     INFO(NCCL_INIT, "invalid NCCL_GPUDIRECTTCPX_SCHED_ALG %s. Using RR by default", v);
   }
+}
+
+// NCCL_GPUDIRECTTCPX_AMD_DEVICE_TYPE: "host" when unset, and also (with a warning) when not a known name.
+void parse_device_type() {
+  g.device_type = kDeviceHost;
+  const char* v = getenv("NCCL_GPUDIRECTTCPX_AMD_DEVICE_TYPE");
+  if (!v || !*v) return;
+  if (strcasecmp(v, "unpack") == 0) {
+    g.device_type = kDeviceUnpack;
+  } else if (strcasecmp(v, "host") != 0) {
+    WARN("NCCL_GPUDIRECTTCPX_AMD_DEVICE_TYPE=%s ignored: not \"host\" or \"unpack\"; using host", v);
+  }
+  INFO(NCCL_INIT, "device type %s", g.device_type == kDeviceUnpack ? "unpack (the caller's kernel copies)" : "host (the plugin's engine copies)");
 }
 
 // Timestamp of a tracepoint: the wall clock like the reference's exporter lines, or the injected clock.
@@ -426,6 +442,7 @@ ncclResult_t tcpxInit(ncclDebugLogger_t logFunction) {
   int_flag(&g.sampling_factor, "TELEMETRY_SAMPLING_FACTOR", 1, INT_MAX - 1);
   parse_slowness_flags();
   parse_sched_alg();
+  parse_device_type();
   if (!g.ops_injected) {
     g.ops = default_device_ops();
     if (!g.ops) {
@@ -504,8 +521,13 @@ ncclResult_t tcpxGetProperties(int dev, ncclNetProperties_v7_t* props) {
   props->maxComms = 65536;
   props->latency = 0;
   props->maxRecvs = 1;
-  props->netDeviceType = NCCL_NET_DEVICE_UNPACK;
-  props->netDeviceVersion = NCCL_NET_DEVICE_UNPACK_VERSION;
+  if (g.device_type == kDeviceUnpack) {  // src/net_tcpx.cc:739-740
+    props->netDeviceType = NCCL_NET_DEVICE_UNPACK;
+    props->netDeviceVersion = NCCL_NET_DEVICE_UNPACK_VERSION;
+  } else {  // the engine owns the copy: nothing for a consumer kernel to do
+    props->netDeviceType = NCCL_NET_DEVICE_HOST;
+    props->netDeviceVersion = NCCL_NET_DEVICE_INVALID_VERSION;
+  }
   return ncclSuccess;
 }
 
@@ -530,12 +552,18 @@ ncclResult_t tcpxSynthArenaCreate(int dev, size_t bytes, void** base) {
 ncclResult_t tcpxListen(int dev, void* handle, void** listenComm) {
   if (!g.initialized || dev < 0 || dev >= g.n_devices || !handle || !listenComm) return ncclInternalError;
   static std::atomic<uint64_t> next_id{1};
-  ListenComm* l = static_cast<ListenComm*>(calloc(1, sizeof *l));
+  ListenComm* l = new (std::nothrow) ListenComm;
   if (!l) return ncclSystemError;
   l->dev = dev;
   l->id = next_id.fetch_add(1);
+  l->backlog.store(0);
+  ConnectHandle h{kConnectMagic, l->id, dev};
   memset(handle, 0, NCCL_NET_HANDLE_MAXSIZE);
-  memcpy(handle, l, sizeof *l);  // the connect handle: which listener, on which device
+  memcpy(handle, &h, sizeof h);  // the connect handle: which listener, on which device
+  {
+    std::lock_guard<std::mutex> lock(g.listen_mu);
+    g.listeners.push_back(l);
+  }
   *listenComm = l;
   return ncclSuccess;
 }
@@ -559,11 +587,31 @@ static ncclResult_t new_comm(int dev, bool passive, Comm** out) {
 ncclResult_t tcpxConnect_v5(int dev, void* handle, void** sendComm, ncclNetDeviceHandle_v7_t** sendDevHandle) {
   if (!g.initialized || dev < 0 || dev >= g.n_devices || !handle || !sendComm) return ncclInternalError;
   // The sending side is outside this build (no NIC, no sockets): the comm exists so that the call sequence of a
-  // real job can be replayed, but tcpxIsend_v5 on it reports an error.
+  // real job can be replayed, but tcpxIsend_v5 on it reports an error.  What connect does do is what a TCP
+  // connect does to a listening socket: it finds the listener the handle names and joins its backlog, where
+  // accept will find it; a handle that names no open listener is "connection refused".
+  ConnectHandle h;
+  memcpy(&h, handle, sizeof h);
+  if (h.magic != kConnectMagic) {
+    WARN("connect: the handle was not written by tcpxListen");
+    return ncclInternalError;
+  }
   Comm* c = nullptr;
   TCPXCHECK(new_comm(dev, false, &c));
+  {
+    std::lock_guard<std::mutex> lock(g.listen_mu);
+    ListenComm* l = nullptr;
+    for (ListenComm* x : g.listeners)
+      if (x->id == h.id) l = x;
+    if (!l) {
+      WARN("connect: listener %lu is not open (connection refused)", static_cast<unsigned long>(h.id));
+      delete c;
+      return ncclSystemError;
+    }
+    l->backlog.fetch_add(1, std::memory_order_release);
+  }
   *sendComm = c;
-  (void)sendDevHandle;
+  (void)sendDevHandle;  // the sending side has no device handle (src/net_tcpx.cc:754-759)
   return ncclSuccess;
 }
 
@@ -571,16 +619,25 @@ ncclResult_t tcpxAccept_v5(void* listenComm, void** recvComm, ncclNetDeviceHandl
   if (!g.initialized || !listenComm || !recvComm) return ncclInternalError;
   ListenComm* l = static_cast<ListenComm*>(listenComm);
   DeviceState* ds = &g.devices[l->dev];
+  *recvComm = nullptr;
+  // Nobody has connected yet: success with no comm, and the caller asks again (the reference's accept is
+  // non-blocking in the same way, which is why src/net_tcpx.cc:764 looks at *recvComm before using it).
+  uint32_t waiting = l->backlog.load(std::memory_order_acquire);
+  do {
+    if (waiting == 0) return ncclSuccess;
+  } while (!l->backlog.compare_exchange_weak(waiting, waiting - 1, std::memory_order_acq_rel));
   if (!ds->arena) {
     WARN("device %d has no bounce arena: call tcpxSynthArenaCreate first", l->dev);
+    l->backlog.fetch_add(1, std::memory_order_release);  // the connection stays in the backlog
     return ncclInternalError;
   }
   Comm* c = nullptr;
   TCPXCHECK(new_comm(l->dev, true, &c));
-  ncclResult_t rc = ensure_engine(ds);
+  ncclResult_t rc = g.device_type == kDeviceHost ? ensure_engine(ds) : ncclSuccess;
   if (rc == ncclSuccess) rc = unpack_queue_new(l->dev, true, &c->queue);  // tcpxGetDeviceHandle, src/net_tcpx.cc:1452-1471
   if (rc != ncclSuccess) {
     delete c;
+    l->backlog.fetch_add(1, std::memory_order_release);
     return rc;
   }
   {
@@ -590,11 +647,19 @@ ncclResult_t tcpxAccept_v5(void* listenComm, void** recvComm, ncclNetDeviceHandl
   if (c->use_helper) c->helper = std::thread(helper_main, c);
   if (recvDevHandle && *recvDevHandle) {
     ncclNetDeviceHandle_v7_t* h = *recvDevHandle;
-    h->netDeviceType = NCCL_NET_DEVICE_UNPACK;
-    h->netDeviceVersion = NCCL_NET_DEVICE_UNPACK_VERSION;
-    h->handle = c->queue->dev_handle;
-    h->size = sizeof(struct unpackNetDeviceHandle);
-    h->needsProxyProgress = 1;
+    if (g.device_type == kDeviceUnpack) {  // src/net_tcpx.cc:1463-1467
+      h->netDeviceType = NCCL_NET_DEVICE_UNPACK;
+      h->netDeviceVersion = NCCL_NET_DEVICE_UNPACK_VERSION;
+      h->handle = c->queue->dev_handle;
+      h->size = sizeof(struct unpackNetDeviceHandle);
+      h->needsProxyProgress = 1;
+    } else {  // nothing for a device-side consumer: the queue is this plugin's own business
+      h->netDeviceType = NCCL_NET_DEVICE_HOST;
+      h->netDeviceVersion = NCCL_NET_DEVICE_INVALID_VERSION;
+      h->handle = nullptr;
+      h->size = 0;
+      h->needsProxyProgress = 0;
+    }
   }
   *recvComm = c;
   return ncclSuccess;
@@ -716,6 +781,16 @@ ncclResult_t tcpxTest(void* request, int* done, int* size) {
         // (src/net_tcpx.cc:1354-1357 is the count + fences; the doorbell is this build's).
         *r->slot.cnt = r->slot.cnt_cache;
         std::atomic_thread_fence(std::memory_order_release);
+        if (g.device_type == kDeviceUnpack) {
+          // The reference's publish and nothing else: the count is visible to the device (the store fence pushes
+          // it out of the write-combining buffers, src/net_tcpx.cc:1356), and whoever holds the device handle
+          // copies.  done=1 means "published".
+          __builtin_ia32_sfence();
+          comm->unpack_cnt++;
+          request_advance(comm, kReqTransmitting);
+          *done = 1;
+          return ncclSuccess;
+        }
         q->meta->done[r->slot.idx].value = 0;
         r->done_value = ++comm->done_seq;
         // The descriptors the engine reads: the mapped slot, or -- for a small request, of which a comm has at
@@ -841,7 +916,13 @@ ncclResult_t tcpxClose(void* oComm) {
 }
 
 ncclResult_t tcpxCloseListen(void* oComm) {
-  free(oComm);
+  ListenComm* l = static_cast<ListenComm*>(oComm);
+  if (!l) return ncclSuccess;
+  {
+    std::lock_guard<std::mutex> lock(g.listen_mu);
+    g.listeners.erase(std::remove(g.listeners.begin(), g.listeners.end(), l), g.listeners.end());
+  }
+  delete l;
   return ncclSuccess;
 }
 

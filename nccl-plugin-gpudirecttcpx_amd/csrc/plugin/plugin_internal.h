@@ -273,9 +273,22 @@ struct Comm {  // struct tcpxComm, src/common.h:159-216
   bool use_helper = false;
 };
 
+// What tcpxListen writes into the caller's 128-byte handle and tcpxConnect_v5 reads back (the reference puts the
+// listening socket's address there, src/connect.cc; with no sockets, the listener's identity does the same job).
+struct ConnectHandle {
+  uint64_t magic;  // kConnectMagic
+  uint64_t id;     // the listener
+  int32_t dev;
+};
+constexpr uint64_t kConnectMagic = 0x7463707861636365ull;  // "tcpxacce"
+static_assert(sizeof(ConnectHandle) <= NCCL_NET_HANDLE_MAXSIZE, "the connect handle must fit NCCL's handle");
+
 struct ListenComm {  // struct tcpxListenComm, src/common.h:112-124
   int dev;
   uint64_t id;
+  // Connections made to this listener and not yet accepted (the listening socket's backlog).  connect() runs on
+  // whichever thread the peer uses, accept() on the owner's.
+  std::atomic<uint32_t> backlog;
 };
 
 // ---- per-GPU and global state -------------------------------------------------------------------------------------
@@ -304,9 +317,19 @@ struct DeviceState {
   std::vector<QueueBlock> free_blocks;
 };
 
+// Who copies.  kDeviceHost: this plugin's engine unpacks every request and test() reports done after the copy; the
+// plugin advertises an ordinary host-driven network (NCCL_NET_DEVICE_HOST), so no consumer kernel touches the
+// queue.  kDeviceUnpack: the reference's division of labour -- the plugin only publishes descriptor counts
+// (src/net_tcpx.cc:1354-1357), advertises NCCL_NET_DEVICE_UNPACK with the device handle, and the caller's kernel
+// copies; the engine is never started.
+constexpr int kDeviceHost = 0, kDeviceUnpack = 1;
+
 struct Global {
   std::mutex mu;
   bool initialized = false;
+  int device_type = kDeviceHost;  // NCCL_GPUDIRECTTCPX_AMD_DEVICE_TYPE=host|unpack
+  std::mutex listen_mu;
+  std::vector<ListenComm*> listeners;  // open listeners, for connect() to find by id
   ncclDebugLogger_t logger = nullptr;
   const tcpxDeviceOps* ops = nullptr;
   bool ops_injected = false;

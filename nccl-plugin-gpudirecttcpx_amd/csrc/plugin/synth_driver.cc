@@ -2,8 +2,8 @@
 //
 // The same sequence the reference's callers produce for the receive path -- irecv (src/net_tcpx.cc:921-944), one
 // control message per chunk from the peer (struct tcpxCtrl, src/common.h:127-133), the chunk's fragments from
-// the kernel (src/sock/tcpx.h:136-228), test() polled until done (src/net_tcpx.cc:1311-1374), irecvConsumed
-// (src/net_tcpx.cc:1477-1543) -- with up to `window` requests posted at a time, as NCCL keeps several steps in
+// the kernel (src/sock/tcpx.h:136-228), test() polled until done (src/net_tcpx.cc:1311-1374), iflush
+// (src/net_tcpx.cc:946-954), irecvConsumed (src/net_tcpx.cc:1477-1543) -- with up to `window` requests posted at a time, as NCCL keeps several steps in
 // flight.  Used by tests and by the benchmark to drive the plugin without an interpreter in the loop.
 #include <time.h>
 
@@ -106,6 +106,18 @@ extern "C" ncclResult_t tcpxSynthRunRequests(void* recvComm, const tcpxSynthFrag
     if ((rc = tcpxTest(posted.front().request, &done, &size)) != ncclSuccess) break;
     if (done) {
       if (latency_s) latency_s[posted.front().index] = now_s() - posted.front().fed;
+      // NCCL's proxy flushes a finished receive before it hands the buffer on (iflush takes the request in the
+      // request slot and answers with its size, src/net_tcpx.cc:946-954), then reports the slot consumed.
+      const tcpxSynthRequest& fr = requests[posted.front().index];
+      void* fdata = static_cast<char*>(dst_base) + fr.dst_off;
+      int fsize = -1;
+      void* freq = posted.front().request;
+      if ((rc = tcpxIflush_v5(comm, 1, &fdata, &fsize, &mhandle, &freq)) != ncclSuccess) break;
+      if (fsize != static_cast<int>(fr.bytes)) {
+        WARN("iflush answered size %d for a request of %u bytes", fsize, fr.bytes);
+        rc = ncclInternalError;
+        break;
+      }
       if ((rc = tcpxIrecvConsumed(comm, 1, posted.front().request)) != ncclSuccess) break;
       posted.pop_front();
       deadline = now_s() + 1e-3 * timeout_ms;

@@ -31,7 +31,14 @@ class RecvComm:
         self.comm = ctypes.c_void_p()
         self.dev_handle = NetDeviceHandle()
         ph = ctypes.pointer(self.dev_handle)
+        # nobody has connected yet: accept succeeds and hands out no comm
         ok(self.lib.tcpxAccept_v5(self.listen, ctypes.byref(self.comm), ctypes.byref(ph)), "tcpxAccept_v5")
+        assert not self.comm.value, "accept handed out a comm before anybody connected"
+        # the peer (in a real job another process, holding the 128-byte handle) connects; then accept pairs with it
+        self.send_comm = ctypes.c_void_p()
+        ok(self.lib.tcpxConnect_v5(dev, handle, ctypes.byref(self.send_comm), None), "tcpxConnect_v5")
+        ok(self.lib.tcpxAccept_v5(self.listen, ctypes.byref(self.comm), ctypes.byref(ph)), "tcpxAccept_v5")
+        assert self.comm.value, "accept found no connection after connect"
         self.mhandles = {}
 
     def reg(self, ptr, size, mem_type=NCCL_PTR_CUDA):
@@ -56,6 +63,15 @@ class RecvComm:
         size = ctypes.c_int(-12345)
         rc = self.lib.tcpxTest(req, ctypes.byref(done), ctypes.byref(size))
         return rc, done.value, size.value
+
+    def iflush(self, ptr, req, mh):
+        """(result, size answered): the request goes in through the request slot, as NCCL's proxy passes it."""
+        data = (ctypes.c_void_p * 1)(ptr)
+        sizes = (ctypes.c_int * 1)(-1)
+        mhs = (ctypes.c_void_p * 1)(mh)
+        reqs = (ctypes.c_void_p * 1)(req.value if hasattr(req, "value") else req)
+        rc = self.lib.tcpxIflush_v5(self.comm, 1, data, sizes, mhs, reqs)
+        return rc, sizes[0]
 
     def consumed(self, req):
         return self.lib.tcpxIrecvConsumed(self.comm, 1, req)
@@ -92,6 +108,7 @@ class RecvComm:
 
     def close(self):
         ok(self.lib.tcpxClose(self.comm), "tcpxClose")
+        ok(self.lib.tcpxClose(self.send_comm), "tcpxClose")
         ok(self.lib.tcpxCloseListen(self.listen), "tcpxCloseListen")
 
 
@@ -163,6 +180,10 @@ def run_workload(comm, workload, dst_ptr, n_flows, window=8, timeout_s=60.0, aft
             latencies.append(time.perf_counter() - t_fed)
             if after_request:
                 after_request(idx)
+            r = reqs[idx]
+            rc, flushed = comm.iflush(dst_ptr + int(r["dst_off"]), req, mh)  # irecv -> test* -> iflush -> irecvConsumed
+            ok(rc, "tcpxIflush_v5")
+            assert flushed == int(r["bytes"]), (flushed, int(r["bytes"]))
             ok(comm.consumed(req), "tcpxIrecvConsumed")
             posted.pop(0)
             deadline = time.time() + timeout_s

@@ -21,6 +21,7 @@ def _ensure_built():
     pkg = graft.load_package()
     needed = [os.path.join(pkg.LIB_DIR, n) for n in ("libtcpxu_hip.so", "libtcpxu_bench.so", "libtcpx_synth.so", "libnccl-net.so")]
     needed.append(os.path.join(ROOT, "oracle", "liboracle.so"))
+    needed.append(os.path.join(ROOT, "tests", "native", "bin", "plugin_dlopen_host"))
     if not all(os.path.exists(p) for p in needed):
         graft.build()
     return pkg

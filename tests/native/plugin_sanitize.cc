@@ -36,11 +36,13 @@ static int run_case(int config, uint32_t shrink, uint8_t* arena, size_t arena_by
   const tcpxSynthRequest* reqs = tcpxSynthRequests(wl);
 
   char handle[NCCL_NET_HANDLE_MAXSIZE];
-  void *listen = nullptr, *comm = nullptr;
+  void *listen = nullptr, *comm = nullptr, *send_comm = nullptr;
   CHECK(tcpxListen(0, handle, &listen) == ncclSuccess);
   ncclNetDeviceHandle_v7_t dev_handle;
   ncclNetDeviceHandle_v7_t* dh = &dev_handle;
-  CHECK(tcpxAccept_v5(listen, &comm, &dh) == ncclSuccess);
+  CHECK(tcpxAccept_v5(listen, &comm, &dh) == ncclSuccess && comm == nullptr);  // nobody has connected yet
+  CHECK(tcpxConnect_v5(0, handle, &send_comm, nullptr) == ncclSuccess && send_comm != nullptr);
+  CHECK(tcpxAccept_v5(listen, &comm, &dh) == ncclSuccess && comm != nullptr);
 
   std::atomic<bool> stop{false};
   std::atomic<uint64_t> drained{0};
@@ -84,6 +86,7 @@ static int run_case(int config, uint32_t shrink, uint8_t* arena, size_t arena_by
     CHECK(drained + n + cs.trace_dropped >= 5ull * info.n_requests);
   }
   CHECK(tcpxClose(comm) == ncclSuccess);
+  CHECK(tcpxClose(send_comm) == ncclSuccess);
   CHECK(tcpxCloseListen(listen) == ncclSuccess);
   tcpxSynthDestroy(wl);
   printf("case config %d shrink %u: %u requests, %llu fragments, %.3f s ok\n", config, shrink, info.n_requests,

@@ -158,3 +158,57 @@ def test_native_driver_full_size(env, oracle):
         assert comm.outstanding_pages() == 0 and len(lat) == info.n_requests
         comm.close()
         assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
+
+
+class WithEmptyRequests:
+    """A workload with zero-size requests put between its own: (requests, frags, info) as run_workload reads them."""
+
+    def __init__(self, wl, at):
+        reqs = list(wl.requests)
+        for k in sorted(at, reverse=True):
+            empty = np.zeros(1, dtype=wl.requests.dtype)[0]
+            empty["first_desc"] = reqs[k]["first_desc"] if k < len(reqs) else 0
+            empty["dst_off"] = reqs[k]["dst_off"] if k < len(reqs) else 0
+            reqs.insert(k, empty)
+        self.requests = np.array(reqs, dtype=wl.requests.dtype)
+        self.frags, self.info = wl.frags, wl.info
+
+
+def test_zero_size_messages_and_iflush_between_real_requests(env, oracle):
+    """irecv -> test* -> iflush -> irecvConsumed on the real engine, with the empty message (a TCPX_CTRL_INLINE
+    control message: it takes a slot, publishes a count of 0 and is consumed through the fast path,
+    src/net_tcpx.cc:1248-1276,1361,1500-1504) at the start, in the middle and at the end of a run of 64 KiB
+    requests.  iflush answers each request's size and does no work (src/net_tcpx.cc:946-954); run_workload checks
+    the answer for every request, this test checks bytes, slots and pages."""
+    torch = env.torch
+    wl = env.pkg.Workload(3, seed=0xF1A5, shrink=5)  # 64 requests of 16 x 4 KiB
+    info = wl.info
+    pool = np.empty(info.pool_bytes, dtype=np.uint8)
+    wl.fill_window(0, pool)
+    upload(env, pool)
+    expect = np.full(GUARD + info.dst_bytes + GUARD, SENTINEL, dtype=np.uint8)
+    graft.oracle_unpack(oracle, expect[GUARD : GUARD + info.dst_bytes], pool, np.ascontiguousarray(wl.descs))
+    dst = torch.full((GUARD + info.dst_bytes + GUARD,), SENTINEL, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    mixed = WithEmptyRequests(wl, at=[0, 7, 7, 20, 33, info.n_requests])
+    n_all = len(mixed.requests)
+    assert n_all == info.n_requests + 6 and sum(int(r["bytes"]) == 0 for r in mixed.requests) == 6
+    comm = env.driver.RecvComm(0)
+    print("plugin case: %d requests, 6 of them empty" % n_all, flush=True)
+    for window in (1, 8):
+        env.driver.run_workload(comm, mixed, dst.data_ptr() + GUARD, n_flows=4, window=window, timeout_s=30)
+    got = dst.cpu().numpy()
+    assert comm.outstanding_pages() == 0
+    head, tail, idx = comm.queue_state()
+    assert head == tail == 2 * n_all and len(set(idx)) == 1  # an empty message takes a slot like any other
+    stats = env.pkg.CommStats()
+    assert env.lib.tcpxGetCommStats(comm.comm, ctypes.byref(stats)) == 0
+    assert stats.unpack_cnt == 2 * info.n_requests  # only requests with payload go to the GPU
+    # n != 1 is an error, and a flush never creates a request of its own (src/net_tcpx.cc:949-953)
+    one = (ctypes.c_void_p * 1)(dst.data_ptr())
+    sizes = (ctypes.c_int * 1)(-5)
+    none = (ctypes.c_void_p * 1)(None)
+    assert env.lib.tcpxIflush_v5(comm.comm, 2, one, sizes, none, none) == 3
+    assert env.lib.tcpxIflush_v5(comm.comm, 1, one, sizes, none, none) == 0 and sizes[0] == -5 and not none[0]
+    comm.close()
+    assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)

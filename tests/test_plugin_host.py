@@ -87,19 +87,18 @@ def test_v7_table_matches_reference_layout(env):
 
 
 def test_properties_and_device_handle(env, comm):
-    """src/net_tcpx.cc:725-744 and 1463-1467."""
+    """src/net_tcpx.cc:725-744 and 1463-1467, in the default device type "host": the plugin's engine owns the
+    copy, so it advertises an ordinary host-driven network and hands out no device handle (a consumer kernel that
+    saw UNPACK would copy every request a second time).  The "unpack" type is covered in test_device_type.py."""
     n = ctypes.c_int()
     assert env.lib.tcpxDevices(ctypes.byref(n)) == 0 and n.value == 1
     p = env.pkg.NetProperties()
     assert env.lib.tcpxGetProperties(0, ctypes.byref(p)) == 0
     assert (p.guid, p.ptrSupport, p.port, p.maxComms, p.latency, p.maxRecvs) == (0, 3, 0, 65536, 0.0, 1)
-    assert (p.netDeviceType, p.netDeviceVersion, p.speed) == (1, 7, 10000)
+    assert (p.netDeviceType, p.netDeviceVersion, p.speed) == (0, 0, 10000)
     assert env.lib.tcpxGetProperties(5, ctypes.byref(p)) == INTERNAL_ERROR
     h = comm.dev_handle
-    assert (h.netDeviceType, h.netDeviceVersion, h.size, h.needsProxyProgress) == (1, 7, 24, 1)
-    # the 24-byte device handle: {meta, bounce_buf, head = -1} (src/devcomm/nccl/unpack1.cu:54-63)
-    raw = (ctypes.c_uint64 * 3).from_address(h.handle)
-    assert raw[1] == env.arena and raw[2] == 2**64 - 1 and raw[0] != 0
+    assert (h.netDeviceType, h.netDeviceVersion, h.handle, h.size, h.needsProxyProgress) == (0, 0, None, 0, 0)
 
 
 def fill_arena(env, wl):
@@ -421,6 +420,38 @@ def test_too_many_fragments_is_fatal(env, comm):
         if rc != 0:
             break
     assert rc == INTERNAL_ERROR
+    comm.dereg(mh)
+
+
+def test_page_token_runs_of_one_flow_are_bounded(env, comm, capfd):
+    """A request may put several chunks on one flow, and their page tokens accumulate in the slot's one list for
+    that flow (2048 runs).  Two chunks of 1100 fragments with tokens that never coalesce would write run 2049 past
+    the end of the list; the builder stops there, like the reference stops on descriptor overflow
+    (src/sock/tcpx.h:183-199), instead of after the fact when the chunk is reaped."""
+    per_chunk, size = 1100, 8
+    n = 2 * per_chunk
+    frags = np.zeros(n, dtype=env.pkg.Workload(1, shrink=6).frag_dtype)
+    frags["frag_offset"] = np.arange(n) * 2 * 4096  # every other page: no two tokens are neighbours
+    frags["frag_size"] = size
+    frags["frag_token"] = np.arange(n) * 2
+    total = n * size
+    buf, ptr = host_buffer(total)
+    mh = comm.reg(ptr, total)
+    rc, req = comm.irecv(ptr, total, mh)
+    assert rc == 0
+    comm.ctrl(0, per_chunk * size, 0, total)
+    comm.ctrl(0, per_chunk * size, per_chunk * size, total)
+    comm.deliver(0, frags)
+    rc = 0
+    for _ in range(50):
+        rc, done, _ = comm.test(req)
+        assert not done
+        if rc != 0:
+            break
+    assert rc == INTERNAL_ERROR
+    # stopped by the builder at the 2049th run, not later by the count check when the chunk is reaped
+    err = capfd.readouterr().err
+    assert "page-token runs" in err and "request too many pages" not in err
     comm.dereg(mh)
 
 
