@@ -112,7 +112,7 @@ typedef struct tcpxuEngine tcpxuEngine;
 
 typedef struct tcpxuEngineConfig {
   uint32_t ring_entries;    /* submission ring size, power of two >= 16, 0 = default (1024) */
-  uint32_t workgroups;      /* persistent grid size, 0 = fill the GPU */
+  uint32_t workgroups;      /* persistent grid size, 0 = two worker workgroups per compute unit + the leader */
   uint32_t descs_per_ticket;/* descriptors one workgroup takes at a time (1..64); 0 = chosen per submission from
                                the backlog of descriptors not yet unpacked: 8 when the engine is idle (lowest
                                latency), 12, then 16 when every workgroup has work queued (highest throughput), and

@@ -815,15 +815,17 @@ int tcpxuEngineCreate(int device, const tcpxuEngineConfig* config, tcpxuEngine**
   TCPXU_TRY(scope.rc());
   const uint32_t cus = static_cast<uint32_t>(std::max(1, device_compute_units(device)));
   if (cfg.workgroups == 0) {
-    // Fill the compute units, but leave a few wavefront slots free on each so that other kernels (copies, the
-    // caller's own work) can still be scheduled while the engine runs: a CU has 32 slots.
-    int max_active = 0;
-    TCPXU_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&max_active, unpack_engine_kernel, kEngineThreads, 0));
-    const uint32_t waves_per_wg = kEngineThreads / kWaveLanes;
-    uint32_t per_cu = static_cast<uint32_t>(std::max(max_active, 1));
-    while (per_cu > 1 && per_cu * waves_per_wg > 28) --per_cu;
-    const char* v = getenv("TCPXU_ENGINE_WGS_PER_CU");
-    if (v && *v) per_cu = std::min(std::max(static_cast<uint32_t>(atoi(v)), 1u), static_cast<uint32_t>(std::max(max_active, 1)));
+    // Two worker workgroups per compute unit: 18 of a compute unit's 32 wavefront slots, so that other kernels
+    // (copies, the caller's own work) are scheduled beside the engine while it runs.  More buys nothing: the
+    // memory system is full with two (8 MiB chunks, 64 slots in flight: 70.8 % of the HBM roofline with two, 70.7 %
+    // with three; one is not enough, 59 %), and requests/s of small requests is the same or better with two.
+    // (Fixed rather than asked of the occupancy query: the kernel needs 56 vector registers and 6.2 KiB of LDS,
+    // three of its workgroups fit a compute unit, and the query has answered "one" in a process that had launched
+    // other kernels before.  A grid larger than what is resident would still be correct -- no workgroup waits for
+    // another worker -- only pointless.)
+    uint32_t per_cu = 2;
+    const char* v = getenv("TCPXU_ENGINE_WGS_PER_CU");  // tuning aid: 1..3
+    if (v && *v) per_cu = std::min(std::max(static_cast<uint32_t>(atoi(v)), 1u), 3u);
     cfg.workgroups = cus * per_cu + 1;
   }
   if (cfg.workgroups < 2 || cfg.workgroups > (1u << 16)) {

@@ -395,8 +395,10 @@ def test_engine_bursts_around_the_idle_exit(pkg, hip, oracle):
     for t in threads:
         t.join(timeout=5)
     assert not any(t.is_alive() for t in threads) and not errors, errors
+    # How often the poll above saw the kernel gone depends on how the host schedules four threads: reported, not
+    # asserted.  That an idle kernel leaves and a submission brings it back is asserted, without any timing, by
+    # test_engine_leaves_when_idle_and_returns_on_submit.
     print("engine burst case: kernel found away %d times" % away, flush=True)
-    assert away >= 3, "the pauses were meant to let the kernel leave now and then"
     got = g.result()
     e.stop()
     assert e.completed() == n
@@ -495,5 +497,80 @@ def test_engine_run_window_times_the_middle_of_a_stream(pkg, hip, oracle, benchl
     assert benchlib.tcpxuEngineRunWindow(e.h, items, n, n // 2, n, 8, 1000, ctypes.byref(wall), ctypes.byref(kern), None) == pkg.INVALID_ARGUMENT
     assert benchlib.tcpxuEngineRunWindow(e.h, items, n, 0, 0, 8, 1000, ctypes.byref(wall), ctypes.byref(kern), None) == pkg.INVALID_ARGUMENT
     e.destroy()
+    got = dst_d.cpu().numpy()
+    assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
+
+
+def test_other_kernels_run_beside_the_engine(pkg, hip, oracle, benchlib):
+    """The engine takes two workgroups of nine wavefronts per compute unit and leaves the rest of each to others:
+    while it streams 64 slots of 4 MiB on its own stream, copy kernels launched on another stream must start and
+    finish (each within a deadline), their bytes must be right, and the unpack must still be byte-exact."""
+    import threading
+
+    import torch
+
+    chunks = [pkg.Workload(2, seed=0xC0E5 + c) for c in range(4)]
+    info0 = chunks[0].info
+    cb = int(info0.dst_bytes)
+    pool = np.empty(info0.pool_bytes, dtype=np.uint8)
+    chunks[0].fill_window(0, pool)
+    expect = np.full(GUARD + len(chunks) * cb + GUARD, SENTINEL, dtype=np.uint8)
+    for c, wl in enumerate(chunks):
+        expect[GUARD + c * cb : GUARD + (c + 1) * cb] = oracle_expected(oracle, pool, wl.descs, cb, 0)[GUARD : GUARD + cb]
+    pool_d = torch.from_numpy(pool).to("cuda:0")
+    dst_d = torch.full((expect.nbytes,), SENTINEL, dtype=torch.uint8, device="cuda:0")
+    per_chunk = [
+        [np.ascontiguousarray(wl.descs[int(r["first_desc"]) : int(r["first_desc"]) + int(r["n_descs"])]) for r in wl.requests]
+        for wl in chunks
+    ]
+    flat = []
+    for rep in range(400):  # 3200 slots of 4 MiB: about 10 ms of streaming
+        for c, lists in enumerate(per_chunk):
+            for d in lists:
+                flat.append((pool_d.data_ptr(), dst_d.data_ptr() + GUARD + c * cb, d.ctypes.data, len(d)))
+    items = (pkg.StreamItem * len(flat))()
+    for i, (b, d, p, n) in enumerate(flat):
+        items[i].bounce_base, items[i].dst_base, items[i].descs_host, items[i].n_descs = b, d, p, n
+    n_copy = 64 << 20
+    src = torch.randint(0, 256, (n_copy,), dtype=torch.uint8, device="cuda:0")
+    out = torch.zeros(n_copy, dtype=torch.uint8, device="cuda:0")
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    e = Engine(pkg, hip)
+    cfg = pkg.EngineConfig()
+    pkg.check(hip.tcpxuEngineGetConfig(e.h, ctypes.byref(cfg)), "tcpxuEngineGetConfig")
+    cus = ctypes.c_int()
+    pkg.check(hip.tcpxuDeviceInfo(0, None, 0, ctypes.byref(cus)), "tcpxuDeviceInfo")
+    assert cfg.workgroups == 2 * cus.value + 1
+    result = {}
+
+    def stream_all():
+        wall, kern = ctypes.c_double(), ctypes.c_double()
+        result["rc"] = benchlib.tcpxuEngineRunTimed(e.h, items, len(flat), 0, 64, 20000, ctypes.byref(wall), ctypes.byref(kern), None)
+        result["kernel_us"] = kern.value
+
+    print("co-residency case: %d slots on the engine, copies of %d MiB beside it" % (len(flat), n_copy >> 20), flush=True)
+    t = threading.Thread(target=stream_all)
+    t.start()
+    while not e.running() and t.is_alive():  # the launch is the thread's first act
+        time.sleep(20e-6)
+    copies_while_running = 0
+    while t.is_alive():
+        pkg.check(benchlib.tcpxuCopyKernelLaunch(0, out.data_ptr(), src.data_ptr(), n_copy, side.cuda_stream), "tcpxuCopyKernelLaunch")
+        done = torch.cuda.Event()
+        done.record(side)
+        deadline = time.time() + 10
+        while not done.query():
+            assert time.time() < deadline, "a copy kernel did not finish while the engine was running"
+        if t.is_alive() and e.running():
+            copies_while_running += 1
+    t.join(timeout=30)
+    assert not t.is_alive() and result["rc"] == 0
+    side.synchronize()
+    print("co-residency case: %d copies finished while the engine streamed (%.0f us launch)" % (copies_while_running, result["kernel_us"]), flush=True)
+    assert copies_while_running >= 1, "no copy kernel finished while the engine kernel was running"
+    assert e.completed() == len(flat)
+    e.destroy()
+    assert torch.equal(out, src)
     got = dst_d.cpu().numpy()
     assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
