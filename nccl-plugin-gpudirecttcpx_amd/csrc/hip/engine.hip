@@ -854,10 +854,19 @@ int tcpxuEngineCreate(int device, const tcpxuEngineConfig* config, tcpxuEngine**
     e->ctl = static_cast<HostCtl*>(h);
     e->ctl_dev = static_cast<HostCtl*>(d);
     const size_t st_bytes = sizeof(DevState) + 2 * sizeof(uint32_t) * cfg.ring_entries;
-    if (hipMalloc(reinterpret_cast<void**>(&e->st), st_bytes) != hipSuccess ||
-        hipMemset(e->st, 0, st_bytes) != hipSuccess ||
+    // The state is cleared on the engine's own stream, and an event pair goes through it, so that whatever the
+    // runtime sets up at a stream's first use (its hardware queue: half a millisecond) is paid here and not by the
+    // first request.
+    // Asking for the kernel's attributes makes the runtime load its code now (lazy otherwise: the first launch
+    // would spend half a millisecond on it, after the launch's start event has been recorded).
+    hipFuncAttributes attr;
+    if (hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(unpack_engine_kernel)) != hipSuccess ||
+        hipMalloc(reinterpret_cast<void**>(&e->st), st_bytes) != hipSuccess ||
         hipStreamCreateWithFlags(&e->stream, hipStreamNonBlocking) != hipSuccess ||
         hipEventCreate(&e->ev_start) != hipSuccess || hipEventCreate(&e->ev_stop) != hipSuccess ||
+        hipEventRecord(e->ev_start, e->stream) != hipSuccess ||
+        hipMemsetAsync(e->st, 0, st_bytes, e->stream) != hipSuccess ||
+        hipEventRecord(e->ev_stop, e->stream) != hipSuccess || hipStreamSynchronize(e->stream) != hipSuccess ||
         hipDeviceSynchronize() != hipSuccess) {
       set_error("engine allocation failed: %s", hipGetErrorString(hipGetLastError()));
       rc = TCPXU_DEVICE_ERROR;
