@@ -73,16 +73,25 @@ def cpu_baseline(oracle, descs, dst_bytes, pool, threads, budget_s):
     return payload / med / 1e9, iters
 
 
-def plugin_path(pkg, hip, torch, workloads, pool):
+def plugin_path(pkg, hip, torch, workloads, pool, helper_thread=False):
     """The same chunks through the whole plugin (libnccl-net.so): irecv -> control messages -> synthetic recvmsg
-    with its control messages -> descriptor builder -> slot -> engine -> test() -> irecvConsumed, driven by the
-    request loop inside the library.  The host builds one descriptor per fragment here, so this is a host-bound
-    figure: what the receive path costs per fragment on one proxy thread."""
+    with its control messages -> descriptor builder -> slot -> engine -> test() -> iflush -> irecvConsumed, driven by
+    the request loop inside the library.  The host builds one descriptor per fragment here, so this is a host-bound
+    figure: what the receive path costs per fragment on one proxy thread (or, with `helper_thread`, on the proxy
+    thread plus the plugin's socket thread, NCCL_GPUDIRECTTCPX_AMD_HELPER_THREAD=1)."""
     from nccl_plugin_gpudirecttcpx_amd import synth_driver
 
     lib = pkg.plugin_lib()
-    if lib.tcpxInit(None) != 0:
-        return {"error": "tcpxInit failed"}
+    saved = os.environ.get("NCCL_GPUDIRECTTCPX_AMD_HELPER_THREAD")
+    os.environ["NCCL_GPUDIRECTTCPX_AMD_HELPER_THREAD"] = "1" if helper_thread else "0"
+    try:
+        if lib.tcpxInit(None) != 0:
+            return {"error": "tcpxInit failed"}
+    finally:
+        if saved is None:
+            os.environ.pop("NCCL_GPUDIRECTTCPX_AMD_HELPER_THREAD", None)
+        else:
+            os.environ["NCCL_GPUDIRECTTCPX_AMD_HELPER_THREAD"] = saved
     base = ctypes.c_void_p()
     assert lib.tcpxSynthArenaCreate(0, pool.nbytes, ctypes.byref(base)) == 0
     pkg.check(hip.tcpxuCopyToDevice(0, base, pool.ctypes.data, pool.nbytes), "tcpxuCopyToDevice")
@@ -104,7 +113,8 @@ def plugin_path(pkg, hip, torch, workloads, pool):
     assert lib.tcpxFinalize() == 0
     payload = 2 * len(workloads) * chunk_bytes
     return {
-        "what": "8 MiB chunks through ncclNet_v7 (irecv/test/irecvConsumed) with the synthetic devmem socket, one proxy thread",
+        "what": "8 MiB chunks through ncclNet_v7 (irecv/test/iflush/irecvConsumed) with the synthetic devmem socket, "
+        + ("the proxy thread plus the plugin's socket thread" if helper_thread else "one proxy thread"),
         "payload_GBps": round(payload / seconds / 1e9, 2),
         "host_ns_per_fragment": round(seconds / frags * 1e9, 1),
         "request_fed_to_done_us_p50": round(percentile(lat, 50) * 1e6, 1),
@@ -540,6 +550,7 @@ def main():
 
     if not args.skip_extras and not args.one_launch:
         result["plugin_path"] = plugin_path(pkg, hip, torch, workloads[: min(8, args.chunks)], pool)
+        result["plugin_path"]["with_socket_thread"] = plugin_path(pkg, hip, torch, workloads[: min(8, args.chunks)], pool, helper_thread=True)
 
     # ---- CPU baseline on this machine's host cores: rank 0, bounded sample ---------------------------------
     # Threads: the cores this process may run on.  A GPU box shows every core of the host to os.cpu_count() while a

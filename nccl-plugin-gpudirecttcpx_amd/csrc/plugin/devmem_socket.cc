@@ -14,80 +14,102 @@ DataPipe::DataPipe()
     // 2048 control messages of CMSG_SPACE(sizeof(struct iovec)) bytes (src/devcomm/unpack_defs1.h:32-36).
     : ctrl_data(static_cast<size_t>(kSlotPages) * CMSG_SPACE(sizeof(struct iovec))), scatter_list(kSlotPages) {}
 
-ssize_t DevmemSocket::recvmsg(struct msghdr* msg, size_t max_bytes) {
+void DevmemSocket::push(const tcpxSynthFrag* frags, size_t n) {
   std::lock_guard<std::mutex> lock(mu);
+  arrived.insert(arrived.end(), frags, frags + n);
+}
+
+ssize_t DevmemSocket::recvmsg(struct msghdr* msg, size_t max_bytes) {
   msg->msg_flags = 0;
+  if (head == rx.size()) {  // everything taken over earlier has been received: look for new arrivals
+    rx.clear();
+    head = 0;
+    {
+      std::lock_guard<std::mutex> lock(mu);
+      rx.swap(arrived);
+    }
+    for (const tcpxSynthFrag& f : rx) payload_frags += f.frag_size != 0;
+  }
   // A recvmsg that returns no bytes means "peer closed" to the caller, so empty fragments (which the adversarial
   // workload contains) only ever travel together with a non-empty one.
-  bool any_payload = false;
-  for (const tcpxSynthFrag& f : rx) {
-    if (f.frag_size != 0) {
-      any_payload = true;
-      break;
-    }
+  if (payload_frags == 0 && head < rx.size()) {
+    // Only empty fragments are left on this side: the payload they travel with may have arrived meanwhile.
+    std::lock_guard<std::mutex> lock(mu);
+    for (const tcpxSynthFrag& f : arrived) payload_frags += f.frag_size != 0;
+    rx.insert(rx.end(), arrived.begin(), arrived.end());
+    arrived.clear();
   }
-  if (!any_payload || max_bytes == 0) {
+  if (payload_frags == 0 || max_bytes == 0) {
     msg->msg_controllen = 0;
     errno = EAGAIN;
     return -1;
   }
+  const uint32_t frag_limit = max_frags_per_recvmsg.load(std::memory_order_relaxed);
   const size_t room = msg->msg_controllen;
   const size_t per_cmsg = CMSG_SPACE(sizeof(DevmemVec));
+  static_assert(CMSG_SPACE(sizeof(DevmemVec)) == CMSG_LEN(sizeof(DevmemVec)) + 4, "one control message: header, 12 bytes, 4 of padding");
   char* out = static_cast<char*>(msg->msg_control);
   size_t used = 0;
   size_t bytes = 0;
   uint32_t n_payload = 0;
-  while (!rx.empty()) {
-    tcpxSynthFrag& f = rx.front();
+  uint64_t refs = 0;
+  while (head < rx.size()) {
+    tcpxSynthFrag& f = rx[head];
     if (f.frag_size != 0) {
       if (bytes >= max_bytes) break;
-      if (max_frags_per_recvmsg != 0 && n_payload >= max_frags_per_recvmsg) break;
-    } else if (bytes == 0 && n_payload == 0) {
-      // leading empty fragments ride with the payload that follows them
+      if (frag_limit != 0 && n_payload >= frag_limit) break;
     }
     if (used + per_cmsg > room) {
       msg->msg_flags |= MSG_CTRUNC;
       break;
     }
     const uint32_t take = static_cast<uint32_t>(std::min<size_t>(f.frag_size, max_bytes - bytes));
+    // One control message: the header's three fields, the vector, and the padding that the kernel zeroes too.
     struct cmsghdr* cm = reinterpret_cast<struct cmsghdr*>(out + used);
-    memset(cm, 0, per_cmsg);
+    cm->cmsg_len = CMSG_LEN(sizeof(DevmemVec));
     cm->cmsg_level = SOL_SOCKET;
     cm->cmsg_type = kScmDevmemOffset;
-    cm->cmsg_len = CMSG_LEN(sizeof(DevmemVec));
     const DevmemVec v{f.frag_offset, take, f.frag_token};
     memcpy(CMSG_DATA(cm), &v, sizeof v);
+    memset(CMSG_DATA(cm) + sizeof v, 0, 4);
     used += per_cmsg;
     bytes += take;
     if (f.frag_size != 0) ++n_payload;
     // Every control message hands one page reference to the receiver.
     if (device && f.frag_token < device->n_pages) {
       device->page_refs[f.frag_token].fetch_add(1, std::memory_order_relaxed);
-      device->pages_outstanding.fetch_add(1, std::memory_order_relaxed);
+      ++refs;
     }
     if (take == f.frag_size) {
-      rx.pop_front();
+      payload_frags -= f.frag_size != 0;
+      ++head;
     } else {  // byte budget ended inside the fragment: the rest stays queued
       f.frag_offset += take;
       f.frag_size -= take;
       break;
     }
   }
+  if (refs) device->pages_outstanding.fetch_add(refs, std::memory_order_relaxed);
   msg->msg_controllen = used;
   return static_cast<ssize_t>(bytes);
 }
 
 int DevmemSocket::dontneed(const PageToken* tokens, size_t n) {
   if (!device) return 0;
-  for (size_t i = 0; i < n; ++i) {
+  uint64_t given_back = 0;
+  int rc = 0;
+  for (size_t i = 0; i < n && rc == 0; ++i) {
     for (uint32_t k = 0; k < tokens[i].token_count; ++k) {
       const uint32_t page = tokens[i].token_start + k;
-      if (page >= device->n_pages) return -1;
-      if (device->page_refs[page].fetch_sub(1, std::memory_order_relaxed) <= 0) return -1;  // freed twice
-      device->pages_outstanding.fetch_sub(1, std::memory_order_relaxed);
+      if (page >= device->n_pages || device->page_refs[page].fetch_sub(1, std::memory_order_relaxed) <= 0) {
+        rc = -1;  // no such page, or freed twice
+        break;
+      }
+      ++given_back;
     }
   }
-  return 0;
+  device->pages_outstanding.fetch_sub(given_back, std::memory_order_relaxed);
+  return rc;
 }
 
 ssize_t process_recv_cmsg(struct msghdr* msg, DataPipe* p, int offset, uint64_t dst_base_offset,

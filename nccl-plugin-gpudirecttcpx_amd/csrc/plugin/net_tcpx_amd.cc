@@ -162,35 +162,38 @@ inline bool request_done(const Request* r) {
 ncclResult_t flow_progress(Comm* comm, int flow) {
   FlowData* fd = &comm->flows[flow];
   TaskRing* tasks = &fd->tasks;
-  if (tasks->has(kTaskActive)) {
-    Task* t = tasks->first(kTaskActive);
-    ncclResult_t res = ncclSuccess;
-    const ssize_t bytes = devmem_recv(&fd->sock, t->size, t->offset, t->pipe, static_cast<uint64_t>(t->request_offset), &res);
-    if (res != ncclSuccess) {
-      t->result = res;
-      return res;
-    }
-    // TCPX_TASK_TP_RECVMSG (src/net_tcpx.cc:167, src/stats/tracepoint.cc:72-82): a recvmsg that finds nothing
-    // yet is a possible slowness; the call itself is counted while task-level stats are on.
-    if (bytes < 0 && g.slow_switch[kSlowSendRecv] && (errno == EAGAIN || errno == EWOULDBLOCK || errno == EINTR || errno == ENOBUFS)) {
-      uint64_t nanos = 0;
-      if (t->watch.should_warn(g.clock, &nanos)) {
-        fd->rx_slow_cnt.fetch_add(1, std::memory_order_relaxed);
-        if (g.slow_report[kSlowSendRecv]) {
-          WARN("%p:%p, nic %d, %s, flow %d recv timeout error %d, %s: [%d/%d]/%d cnt %u, nanos %lu", static_cast<void*>(t),
-               static_cast<void*>(comm), comm->dev, g.dev_names[comm->dev], flow, errno, strerror(errno), t->offset, t->size,
-               t->r->size, t->watch.same_count, static_cast<unsigned long>(nanos));
+  // The flow's tasks in order: a task whose bytes have all arrived makes room for the next one in the same call (the
+  // socket delivers in order, so a task that has to wait ends the pass).
+  for (int served = 0; served < kMaxTasks; ++served) {
+    if (tasks->has(kTaskActive)) {
+      Task* t = tasks->first(kTaskActive);
+      ncclResult_t res = ncclSuccess;
+      const ssize_t bytes = devmem_recv(&fd->sock, t->size, t->offset, t->pipe, static_cast<uint64_t>(t->request_offset), &res);
+      if (res != ncclSuccess) {
+        t->result = res;
+        return res;
+      }
+      // TCPX_TASK_TP_RECVMSG (src/net_tcpx.cc:167, src/stats/tracepoint.cc:72-82): a recvmsg that finds nothing
+      // yet is a possible slowness; the call itself is counted while task-level stats are on.
+      if (bytes < 0 && g.slow_switch[kSlowSendRecv] && (errno == EAGAIN || errno == EWOULDBLOCK || errno == EINTR || errno == ENOBUFS)) {
+        uint64_t nanos = 0;
+        if (t->watch.should_warn(g.clock, &nanos)) {
+          FlowData::bump(fd->rx_slow_cnt);
+          if (g.slow_report[kSlowSendRecv]) {
+            WARN("%p:%p, nic %d, %s, flow %d recv timeout error %d, %s: [%d/%d]/%d cnt %u, nanos %lu", static_cast<void*>(t),
+                 static_cast<void*>(comm), comm->dev, g.dev_names[comm->dev], flow, errno, strerror(errno), t->offset, t->size,
+                 t->r->size, t->watch.same_count, static_cast<unsigned long>(nanos));
+          }
         }
       }
+      if (g.task_stats) FlowData::bump(fd->rx_cnt);
+      if (bytes > 0) {
+        t->offset += static_cast<int>(bytes);
+        fd->bytes += static_cast<uint64_t>(bytes);
+      }
+      if (t->offset == t->size) task_advance(comm, tasks, kTaskActive);  // ACTIVE -> COMPLETING
     }
-    if (g.task_stats) fd->rx_cnt.fetch_add(1, std::memory_order_relaxed);
-    if (bytes > 0) {
-      t->offset += static_cast<int>(bytes);
-      fd->bytes += static_cast<uint64_t>(bytes);
-    }
-    if (t->offset == t->size) task_advance(comm, tasks, kTaskActive);  // ACTIVE -> COMPLETING
-  }
-  if (tasks->has(kTaskCompleting)) {
+    if (!tasks->has(kTaskCompleting)) break;  // the active task, if any, is still waiting for bytes
     // The reference asks gpu_inline_test here, which always answers "done" (src/devcomm/nccl/inline.cu:55-60).
     task_advance(comm, tasks, kTaskCompleting);  // COMPLETING -> INACTIVE
   }
@@ -243,15 +246,9 @@ void enqueue_task(Comm* comm, Request* r) {
   if (r->size == r->offset) request_advance(comm, kReqActive);  // REQUEST_INACTIVE -> finish_active
 }
 
-// tcpxCommProgress, src/net_tcpx.cc:1099-1308 (receive branch)
-ncclResult_t comm_progress(Comm* comm) {
-  if (comm->rq.empty()) return ncclSuccess;
-
-  if (!comm->use_helper) {
-    for (int f = 0; f < comm->num_flows; ++f) TCPXCHECK(flow_progress(comm, f));
-  }
-
-  // Reap finished tasks: their descriptors move into the request's slot (src/net_tcpx.cc:1119-1151).
+// Reaps finished tasks: their descriptors move into the request's slot (src/net_tcpx.cc:1119-1151), and the flows
+// whose task ring has room are offered to the scheduler.
+ncclResult_t reap_tasks(Comm* comm) {
   comm->sched->reset();  // src/net_tcpx.cc:1114
   for (int i = 0; i < comm->num_flows; ++i) {
     int idx = comm->end_flow_idx - i;
@@ -276,7 +273,32 @@ ncclResult_t comm_progress(Comm* comm) {
     // Priority = task slots in use: the emptiest flow is served first (src/net_tcpx.cc:1152-1155).
     if (tasks->has_free()) comm->sched->schedule(idx, kMaxTasks - static_cast<int>(tasks->num_free()));
   }
+  return ncclSuccess;
+}
 
+ncclResult_t take_control_messages(Comm* comm, bool* enqueued);
+
+// tcpxCommProgress, src/net_tcpx.cc:1099-1308 (receive branch)
+ncclResult_t comm_progress(Comm* comm) {
+  if (comm->rq.empty()) return ncclSuccess;
+  // One call makes up to kProgressPasses passes of: sockets, reap, control messages.  The reference makes one and
+  // is called again by the next test(); a pass that has just started tasks is followed by another at once here,
+  // because the bytes of a chunk whose control message has been read have usually arrived already and the tasks
+  // they finish make room for the next control messages.
+  constexpr int kProgressPasses = 4;
+  for (int pass = 0; pass < kProgressPasses; ++pass) {
+    if (!comm->use_helper) {
+      for (int f = 0; f < comm->num_flows; ++f) TCPXCHECK(flow_progress(comm, f));
+    }
+    TCPXCHECK(reap_tasks(comm));
+    bool enqueued = false;
+    TCPXCHECK(take_control_messages(comm, &enqueued));
+    if (!enqueued || comm->use_helper) break;
+  }
+  return ncclSuccess;
+}
+
+ncclResult_t take_control_messages(Comm* comm, bool* enqueued) {
   if (comm->rq.has(kReqPosted)) request_advance(comm, kReqPosted);  // POSTED -> ACTIVE (src/net_tcpx.cc:1158-1180)
 
   if (!comm->rq.has(kReqActive) || !comm->sched->has_flow()) return ncclSuccess;
@@ -287,17 +309,20 @@ ncclResult_t comm_progress(Comm* comm) {
     if (!ctrl_done(ar)) {
       CtrlMessage ctrl;
       bool got_ctrl = false;
-      {
+      if (comm->ctrl_local.empty()) {  // take over everything that has arrived: one lock per burst, not per message
         std::lock_guard<std::mutex> lock(comm->ctrl_mu);
-        if (!comm->ctrl_rx.empty()) {
-          ctrl = comm->ctrl_rx.front();
-          comm->ctrl_rx.pop_front();
-          got_ctrl = true;
-        }
+        comm->ctrl_local.swap(comm->ctrl_rx);
+      }
+      if (!comm->ctrl_local.empty()) {
+        ctrl = comm->ctrl_local.front();
+        comm->ctrl_local.pop_front();
+        got_ctrl = true;
       }
       // Every look at the control socket counts towards its slowness watch; a message resets it
       // (src/net_tcpx.cc:1234-1246).
-      if (g.slow_switch[kSlowRxCtrl]) {
+      // (A look that finds a message as the first look since the last reset would note the time and be reset again
+      // just below: it is skipped, clock read and all.)
+      if (g.slow_switch[kSlowRxCtrl] && !(got_ctrl && comm->ctrl_watch.same_count == 0)) {
         uint64_t nanos = 0;
         if (comm->ctrl_watch.should_warn(g.clock, &nanos)) {
           comm->rx_ctrl_slow_cnt++;
@@ -313,7 +338,7 @@ ncclResult_t comm_progress(Comm* comm) {
         WARN("control message names flow %u, comm has %d", ctrl.index, comm->num_flows);
         return ncclInternalError;
       }
-      if (ctrl.type != TCPX_CTRL_INLINE) comm->flows[ctrl.index].rx_ctrl_done_cnt.fetch_add(1, std::memory_order_relaxed);
+      if (ctrl.type != TCPX_CTRL_INLINE) FlowData::bump(comm->flows[ctrl.index].rx_ctrl_done_cnt);
       ar->next_flow = ctrl.index;  // tcpxCtrlRecv, src/net_tcpx.cc:995-1014
       ar->next_size = static_cast<int>(ctrl.size);
       if (ar->size_pending < 0) ar->size_pending = ar->size = static_cast<int>(ctrl.total);
@@ -324,8 +349,7 @@ ncclResult_t comm_progress(Comm* comm) {
           WARN("no more unpack queue slot, head %lu tail %lu", static_cast<unsigned long>(comm->queue->head),
                static_cast<unsigned long>(comm->queue->tail));
           // The control message is consumed and cannot be re-read: put it back so that a later poll retries.
-          std::lock_guard<std::mutex> lock(comm->ctrl_mu);
-          comm->ctrl_rx.push_front(ctrl);
+          comm->ctrl_local.push_front(ctrl);
           ar->next_flow = -1;
           break;
         }
@@ -356,6 +380,7 @@ ncclResult_t comm_progress(Comm* comm) {
     if (!tasks->has_free()) break;  // "No free space for recv task": retried at the next poll
     comm->end_flow_idx = ar->next_flow;
     enqueue_task(comm, ar);
+    *enqueued = true;
   } while (ar->offset < ar->size);
   return ncclSuccess;
 }
@@ -397,6 +422,26 @@ int sched_alg_from_name(const char* name, bool* valid) {
   const bool rr = name && strcmp(name, "RR") == 0, katy = name && strcmp(name, "KATY") == 0;
   if (valid) *valid = rr || katy;
   return katy ? kSchedKaty : kSchedRoundRobin;
+}
+
+void ctrl_send_batch(Comm* comm, const CtrlMessage* messages, size_t n) {
+  std::lock_guard<std::mutex> lock(comm->ctrl_mu);
+  comm->ctrl_rx.insert(comm->ctrl_rx.end(), messages, messages + n);
+}
+
+ncclResult_t deliver_fragments(Comm* comm, uint32_t flow, const tcpxSynthFrag* frags, uint32_t n_frags) {
+  const size_t arena = comm->device->arena_bytes;
+  for (uint32_t i = 0; i < n_frags; ++i) {
+    const tcpxSynthFrag& f = frags[i];
+    // The devmem contract: a fragment lies inside the arena and inside one 4 KiB page.
+    if (static_cast<size_t>(f.frag_offset) + f.frag_size > arena ||
+        (f.frag_offset % SLICE_PAGE_SIZE) + f.frag_size > SLICE_PAGE_SIZE) {
+      WARN("fragment %u (offset %u, size %u) breaks the devmem contract", i, f.frag_offset, f.frag_size);
+      return ncclInvalidArgument;
+    }
+  }
+  comm->flows[flow].sock.push(frags, n_frags);
+  return ncclSuccess;
 }
 
 FlowScheduler* new_flow_scheduler(int alg) {
@@ -940,29 +985,13 @@ ncclResult_t tcpxSynthCtrlSend(void* recvComm, uint16_t type, uint16_t flow, uin
 ncclResult_t tcpxSynthDeliver(void* recvComm, uint32_t flow, const tcpxSynthFrag* frags, uint32_t n_frags) {
   Comm* comm = static_cast<Comm*>(recvComm);
   if (!comm || !comm->passive || flow >= static_cast<uint32_t>(comm->num_flows) || (!frags && n_frags)) return ncclInvalidArgument;
-  const size_t arena = comm->device->arena_bytes;
-  for (uint32_t i = 0; i < n_frags; ++i) {
-    const tcpxSynthFrag& f = frags[i];
-    // The devmem contract: a fragment lies inside the arena and inside one 4 KiB page.
-    if (static_cast<size_t>(f.frag_offset) + f.frag_size > arena ||
-        (f.frag_offset % SLICE_PAGE_SIZE) + f.frag_size > SLICE_PAGE_SIZE) {
-      WARN("fragment %u (offset %u, size %u) breaks the devmem contract", i, f.frag_offset, f.frag_size);
-      return ncclInvalidArgument;
-    }
-  }
-  DevmemSocket* s = &comm->flows[flow].sock;
-  std::lock_guard<std::mutex> lock(s->mu);
-  s->rx.insert(s->rx.end(), frags, frags + n_frags);
-  return ncclSuccess;
+  return deliver_fragments(comm, flow, frags, n_frags);
 }
 
 ncclResult_t tcpxSynthSetRecvmsgLimit(void* recvComm, uint32_t max_frags_per_recvmsg) {
   Comm* comm = static_cast<Comm*>(recvComm);
   if (!comm) return ncclInvalidArgument;
-  for (int f = 0; f < kMaxFlows; ++f) {
-    std::lock_guard<std::mutex> lock(comm->flows[f].sock.mu);
-    comm->flows[f].sock.max_frags_per_recvmsg = max_frags_per_recvmsg;
-  }
+  for (int f = 0; f < kMaxFlows; ++f) comm->flows[f].sock.max_frags_per_recvmsg.store(max_frags_per_recvmsg, std::memory_order_relaxed);
   return ncclSuccess;
 }
 

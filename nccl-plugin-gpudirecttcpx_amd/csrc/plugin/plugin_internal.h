@@ -70,6 +70,14 @@ void log_line(ncclDebugLogLevel level, unsigned long flags, const char* file, in
 //   entered >= left[0] >= left[1] >= ... >= left[Stages-1]   and   entered - left[Stages-1] <= Capacity.
 // With Counter = std::atomic<uint32_t> one thread may own `entered` and some stages while another owns the rest
 // (single producer, single consumer per counter).
+// A counter is written by exactly one thread: its new value is published with a release store and read with an
+// acquire load (plain moves on x86; the default sequentially consistent store would be a locked exchange on every
+// state transition of every task).
+inline uint32_t counter_load(const uint32_t& c) { return c; }
+inline void counter_store(uint32_t& c, uint32_t v) { c = v; }
+inline uint32_t counter_load(const std::atomic<uint32_t>& c) { return c.load(std::memory_order_acquire); }
+inline void counter_store(std::atomic<uint32_t>& c, uint32_t v) { c.store(v, std::memory_order_release); }
+
 template <typename Item, int Capacity, int Stages, typename Counter>
 struct StageRing {
   alignas(64) Counter entered;
@@ -77,21 +85,21 @@ struct StageRing {
   alignas(64) Item items[Capacity];
 
   StageRing() {
-    entered = 0;
-    for (int k = 0; k < Stages; ++k) left[k] = 0;
+    counter_store(entered, 0);
+    for (int k = 0; k < Stages; ++k) counter_store(left[k], 0);
   }
-  uint32_t in_flight() const { return static_cast<uint32_t>(entered) - static_cast<uint32_t>(left[Stages - 1]); }
+  uint32_t in_flight() const { return counter_load(entered) - counter_load(left[Stages - 1]); }
   bool empty() const { return in_flight() == 0; }
   uint32_t num_free() const { return Capacity - in_flight(); }
   bool has_free() const { return num_free() > 0; }
-  Item* next_free() { return &items[static_cast<uint32_t>(entered) % Capacity]; }
-  void enqueue() { entered = static_cast<uint32_t>(entered) + 1; }
+  Item* next_free() { return &items[counter_load(entered) % Capacity]; }
+  void enqueue() { counter_store(entered, counter_load(entered) + 1); }
 
-  uint32_t stage_begin(int k) const { return static_cast<uint32_t>(left[k]); }
-  uint32_t stage_end(int k) const { return k == 0 ? static_cast<uint32_t>(entered) : static_cast<uint32_t>(left[k - 1]); }
+  uint32_t stage_begin(int k) const { return counter_load(left[k]); }
+  uint32_t stage_end(int k) const { return k == 0 ? counter_load(entered) : counter_load(left[k - 1]); }
   bool has(int k) const { return stage_end(k) != stage_begin(k); }
   Item* first(int k) { return &items[stage_begin(k) % Capacity]; }
-  void advance(int k) { left[k] = static_cast<uint32_t>(left[k]) + 1; }
+  void advance(int k) { counter_store(left[k], counter_load(left[k]) + 1); }
 };
 
 // ---- unpack queue -------------------------------------------------------------------------------------------------
@@ -167,10 +175,17 @@ struct DeviceState;
 // and at most the control buffer's worth of fragments, one SCM_DEVMEM_OFFSET control message each, splitting a
 // fragment when the byte budget ends inside it (the kernel does the same at the end of a recvmsg).
 struct DevmemSocket {
+  // Two sides.  Whoever delivers fragments appends to `arrived` under the lock; the one thread that receives on
+  // this socket works on `rx`, which nobody else touches, and takes the lock only when `rx` has run empty, to swap
+  // the two -- once per burst of deliveries instead of once per recvmsg.
   std::mutex mu;
-  std::deque<tcpxSynthFrag> rx;
-  uint32_t max_frags_per_recvmsg = 0;  // 0 = no extra limit
+  std::vector<tcpxSynthFrag> arrived;
+  std::vector<tcpxSynthFrag> rx;
+  size_t head = 0;                     // read position in rx
+  size_t payload_frags = 0;            // fragments in rx[head..] with frag_size != 0
+  std::atomic<uint32_t> max_frags_per_recvmsg{0};  // 0 = no extra limit
   DeviceState* device = nullptr;       // page accounting
+  void push(const tcpxSynthFrag* frags, size_t n);  // takes the lock
   ssize_t recvmsg(struct msghdr* msg, size_t max_bytes);
   // setsockopt(SO_DEVMEM_DONTNEED): gives page references back (src/sock/tcpx.h:299-307).
   int dontneed(const PageToken* tokens, size_t n);
@@ -249,6 +264,9 @@ struct FlowData {  // struct tcpxFdData, src/common.h:144-157 (receive-side fiel
   uint64_t bytes = 0;
   // struct tcpxSocketStats (receive side); the socket thread counts, the proxy thread reads.
   std::atomic<uint64_t> rx_ctrl_done_cnt{0}, rx_cnt{0}, rx_slow_cnt{0};
+  // Each has one writer (the proxy thread, or the thread that runs this flow's socket), so a count is a load and a
+  // store, not a locked read-modify-write.
+  static void bump(std::atomic<uint64_t>& c) { c.store(c.load(std::memory_order_relaxed) + 1, std::memory_order_relaxed); }
 };
 
 struct Comm {  // struct tcpxComm, src/common.h:159-216
@@ -259,7 +277,8 @@ struct Comm {  // struct tcpxComm, src/common.h:159-216
   FlowData flows[kMaxFlows];
   std::unique_ptr<FlowScheduler> sched;  // tcpxComm::flow_mapper: the flows whose task ring has room
   std::mutex ctrl_mu;
-  std::deque<CtrlMessage> ctrl_rx;  // the control socket's receive queue
+  std::deque<CtrlMessage> ctrl_rx;  // the control socket's receive queue: what has arrived (under ctrl_mu)
+  std::deque<CtrlMessage> ctrl_local;  // ... and what the proxy thread has taken over from it, to read without the lock
   RequestRing rq;
   UnpackQueue* queue = nullptr;
   DeviceState* device = nullptr;
@@ -357,6 +376,11 @@ extern Global g;
 
 FlowScheduler* new_flow_scheduler(int alg);  // kSchedKaty, or round robin for anything else
 int sched_alg_from_name(const char* name, bool* valid);  // "RR" / "KATY" (exact); anything else is round robin
+
+// The synthetic peer and kernel, for drivers inside the library: many control messages under one lock, and
+// fragments that the caller has already checked against the devmem contract.
+void ctrl_send_batch(Comm* comm, const CtrlMessage* messages, size_t n);
+ncclResult_t deliver_fragments(Comm* comm, uint32_t flow, const tcpxSynthFrag* frags, uint32_t n_frags);
 
 const tcpxDeviceOps* default_device_ops();  // binds libtcpxu_hip.so, or nullptr (reason logged)
 ncclResult_t device_result(int rc, const char* what);

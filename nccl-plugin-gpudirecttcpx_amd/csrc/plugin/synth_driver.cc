@@ -73,6 +73,8 @@ extern "C" ncclResult_t tcpxSynthRunRequests(void* recvComm, const tcpxSynthFrag
   };
   std::deque<Posted> posted;
   std::vector<Chunk> chunks;
+  std::vector<CtrlMessage> ctrl;
+  std::vector<tcpxSynthFrag> by_flow[kMaxFlows];
   uint32_t next = 0;
   ncclResult_t rc = ncclSuccess;
   const double t0 = now_s();
@@ -89,14 +91,21 @@ extern "C" ncclResult_t tcpxSynthRunRequests(void* recvComm, const tcpxSynthFrag
       if (r.bytes == 0) {
         rc = tcpxSynthCtrlSend(comm, TCPX_CTRL_INLINE, 0, 0, 0, 0);
       } else {
+        // The peer's control messages, one per chunk, in chunk order; then what the kernel has for each flow: the
+        // flow's fragments in arrival order (a socket keeps order only within itself, so handing each flow its
+        // fragments in one piece is what many small deliveries come to).
         chunks_of(f, r.n_descs, n_flows, &chunks);
+        ctrl.clear();
+        for (uint32_t k = 0; k < n_flows; ++k) by_flow[k].clear();
         uint32_t offset = 0;
         for (const Chunk& c : chunks) {
-          if ((rc = tcpxSynthCtrlSend(comm, TCPX_CTRL_NORMAL, static_cast<uint16_t>(c.flow), c.bytes, offset, r.bytes)) != ncclSuccess) break;
+          ctrl.push_back(CtrlMessage{TCPX_CTRL_NORMAL, static_cast<uint16_t>(c.flow), c.bytes, offset, r.bytes});
           offset += c.bytes;
+          by_flow[c.flow].insert(by_flow[c.flow].end(), f + c.first, f + c.first + c.count);
         }
-        for (size_t k = 0; rc == ncclSuccess && k < chunks.size(); ++k)
-          rc = tcpxSynthDeliver(comm, chunks[k].flow, f + chunks[k].first, chunks[k].count);
+        ctrl_send_batch(comm, ctrl.data(), ctrl.size());
+        for (uint32_t k = 0; rc == ncclSuccess && k < n_flows; ++k)
+          if (!by_flow[k].empty()) rc = deliver_fragments(comm, k, by_flow[k].data(), static_cast<uint32_t>(by_flow[k].size()));
       }
       posted.push_back(Posted{request, next, now_s()});
       ++next;

@@ -38,6 +38,7 @@ static struct tcpxuEngine g_engine;
 static emu_job g_pending[EMU_MAX_PENDING];
 static int g_n_pending = 0;
 static int g_hold = 0;
+static int g_skip_copy = 0;
 static int g_ring_full = 0;
 static uint64_t g_submitted = 0, g_mapped_live = 0, g_device_live = 0, g_arenas_live = 0, g_engine_starts = 0;
 /* "Device memory that the host can write": host memory here; the blocks are remembered so that a submission whose
@@ -49,12 +50,13 @@ static int g_visible_off = 0;
 static int in_visible(const void* p);
 
 static void run_job(const emu_job* j) {
-  if (j->n) tcpx_oracle_unpack((uint8_t*)j->dst, (const uint8_t*)j->bounce, (const tcpx_oracle_desc*)j->descs, j->n);
+  if (j->n && !g_skip_copy) tcpx_oracle_unpack((uint8_t*)j->dst, (const uint8_t*)j->bounce, (const tcpx_oracle_desc*)j->descs, j->n);
   __atomic_store_n(j->flag, j->value, __ATOMIC_RELEASE);
 }
 
 /* ---- test controls -------------------------------------------------------------------------------------------- */
 void emu_set_hold(int hold) { g_hold = hold; }
+void emu_set_skip_copy(int skip) { g_skip_copy = skip; } /* completes submissions without moving bytes: for timing the host code alone */
 void emu_set_ring_full(int full) { g_ring_full = full; }
 void emu_set_visible_off(int off) { g_visible_off = off; } /* allocations of host-visible device memory fail */
 int emu_pending(void) { return g_n_pending; }

@@ -172,12 +172,15 @@ def test_recvmsg_finding_nothing_is_watched_and_counted(pkg):
         mh = s.comm.reg(ptr, 8192)
         rc, req = s.comm.irecv(ptr, 8192, mh)
         s.comm.ctrl(2, 8192, 0, 8192)
-        assert s.comm.test(req)[:2] == (0, 0)  # takes the control message and creates the task; no recvmsg yet
+        # takes the control message, creates the task and, in the pass that follows at once, looks at the socket for
+        # the first time (nothing there yet)
+        assert s.comm.test(req)[:2] == (0, 0)
         assert s.flow_stats(2).rx_ctrl_done_cnt == 1 and s.flow_stats(0).rx_ctrl_done_cnt == 0
         calls0 = s.flow_stats(2).rx_cnt
-        assert calls0 == 0
+        assert calls0 == 1
         watch_reports = []
         watch = host_logic.SlownessWatch(THRESHOLD_NS, FREQUENCY_NS)
+        assert watch.should_warn(s.now) == (False, None)  # the task's first look only notes the time
         rng = np.random.default_rng(2)
         for i in range(40):
             s.now += int(rng.integers(0, 700_000))
