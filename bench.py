@@ -25,9 +25,10 @@ therefore carries: an untimed fill of at least two queues' worth of steps (never
 windows of exactly K steps each, back to back, then an untimed tail of one queue's worth that keeps the queues
 full while the last window finishes.  Every completion is stamped by the host poller; a window is timed from the
 completion of the step before it to the completion of its last step; `ms_per_step` x K is the MEDIAN window and
-`value` the payload of K steps over it.  R is at least 50 and large enough that the launch carries 2000 steps or
-more, so that the launch's own duration (HIP events on the engine's stream: `roofline`) is the rate too, with
-launch, ramp and stop below 2 % of it.
+`value` the payload of K steps over it.  R is at least 50 and large enough that the launch carries 20000 steps or
+more (60 ms), so that the launch's own duration (HIP events on the engine's stream: `roofline`) is the rate too,
+with launch, ramp and stop well below 1 % of it; an untimed launch of the same length comes first, because the GPU
+takes some milliseconds of load to reach the rate it then sustains.
 
 Prints ONE JSON line: payload GB/s (`value`), the HBM roofline of the dominant kernel, p50/p99 request
 completion latency, and a memcpy-per-descriptor CPU baseline timed on this machine's host cores.
@@ -49,6 +50,10 @@ import __graft_entry__ as graft
 # (`--calibrate-copy 256`); the summary with the counter values is profiles/unpack_engine_kernel_8MiB_chunk_pmc_traffic.txt.
 TRAFFIC_PER_ALGORITHMIC_BYTE = 1.0060
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+# Steps in the untimed launch that precedes the measured one, and the least steps the windows of the measured launch
+# add up to (60 ms each way): the rate the engine sustains shows only after some milliseconds of load.
+WARM_LAUNCH_STEPS = 20000
+MIN_TIMED_STEPS = 20000
 CHUNK_CONFIG = 2
 
 
@@ -210,7 +215,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=400, help="K: steps in one timed window")
     ap.add_argument("--warmup", type=int, default=64, help="W: untimed steps before the first window (at least two queues' worth are run whatever W says)")
-    ap.add_argument("--windows", type=int, default=0, help="R: timed windows of K steps in the launch; 0 = max(50, ceil(2000 / K))")
+    ap.add_argument("--windows", type=int, default=0, help="R: timed windows of K steps in the launch; 0 = max(50, ceil(20000 / K))")
     ap.add_argument(
         "--chunks",
         type=int,
@@ -353,21 +358,24 @@ def main():
     # ---- fill, R windows of exactly K steps, tail: all inside ONE launch of the persistent kernel ---------------
     queue_steps = (args.comms * args.depth + slots_per_step - 1) // slots_per_step  # steps that fill every queue once
     fill_steps = max(args.warmup, 2 * queue_steps)
-    windows = args.windows if args.windows > 0 else max(50, (2000 + args.steps - 1) // args.steps)
+    windows = args.windows if args.windows > 0 else max(50, (MIN_TIMED_STEPS + args.steps - 1) // args.steps)
     tail_steps = queue_steps
     steps_per_launch = fill_steps + windows * args.steps + tail_steps
     all_items = item_array(0, steps_per_launch)
-    # An untimed launch first: brings the clocks up from idle and loads the library's code onto the GPU.  Where the
+    # An untimed launch first: brings the GPU from idle to the state it is in under sustained load (a measured launch
+    # of 2096 steps shows 70.2 % of the roofline after 64 untimed steps, 70.8 % after 2000 and 71.4 % after 20000) and
+    # loads the library's code onto the GPU.  Where the
     # process may launch the engine kernel only once (--one-launch, for a profiler), other kernels do that instead:
-    # the launch-per-batch kernel (the same code object) on one chunk and the plain copy kernel over 1 GiB.
+    # the launch-per-batch kernel (the same code object) on one chunk and the plain copy kernel, 150 times over half the
+    # destination ring (60 ms).
     if not args.one_launch:
-        run(item_array(0, fill_steps), args.comms * args.depth)
+        run(item_array(0, max(fill_steps, WARM_LAUNCH_STEPS)), args.comms * args.depth)
     else:
         us = ctypes.c_double()
         d0 = torch.from_numpy(np.ascontiguousarray(workloads[0].descs).view(np.uint8)).to("cuda:0")
         pkg.check(benchlib.tcpxuUnpackBatchTimed(dev, pool_d.data_ptr(), dst_base, d0.data_ptr(), workloads[0].info.n_descs, 2, 3, ctypes.byref(us)), "batch timed")
         n_warm = min(1 << 30, args.chunks * int(chunk_bytes) // 2 // 16 * 16)
-        pkg.check(benchlib.tcpxuCopyKernelTimed(dev, dst_base + n_warm, dst_base, n_warm, 2, 10, ctypes.byref(us)), "copy timed")
+        pkg.check(benchlib.tcpxuCopyKernelTimed(dev, dst_base + n_warm, dst_base, n_warm, 2, 150, ctypes.byref(us)), "copy timed")  # 60 ms of load
         del d0
     torch.cuda.synchronize()
     t0 = time.perf_counter()
