@@ -50,6 +50,19 @@ ncclResult_t tcpxCloseListen(void* listenComm);                                 
 ncclResult_t tcpxGetDeviceMr(void* comm, void* mhandle, void** dptr_mhandle);      /* src/net_tcpx.cc:1473-1475 */
 ncclResult_t tcpxIrecvConsumed(void* recvComm, int n, void* request);              /* src/net_tcpx.cc:1477-1543 */
 
+/* Who copies is chosen at tcpxInit by NCCL_GPUDIRECTTCPX_AMD_DEVICE_TYPE:
+ *   "host" (default)  the plugin's GPU engine unpacks every request; tcpxTest reports done after the copy;
+ *                     tcpxGetProperties / tcpxAccept_v5 say NCCL_NET_DEVICE_HOST (version 0, no device handle), so
+ *                     that no consumer kernel copies the same bytes a second time;
+ *   "unpack"          the reference's division of labour (src/net_tcpx.cc:725-744,1354-1357,1452-1471): they say
+ *                     NCCL_NET_DEVICE_UNPACK version 7 and hand out the 24-byte device unpackNetDeviceHandle;
+ *                     tcpxTest reports done once the descriptor count is published; the engine is never started
+ *                     and whoever holds the handle copies.
+ * tcpxListen writes the listener's identity into the 128-byte handle; tcpxConnect_v5 with that handle joins the
+ * listener's backlog (ncclSystemError if the listener is closed, ncclInternalError for a handle tcpxListen did not
+ * write); tcpxAccept_v5 returns success with *recvComm = NULL until a connection is waiting
+ * (src/net_tcpx.cc:761-769). */
+
 /* Undoes tcpxInit: stops the engines, frees arenas and cached queue memory.  Comms must be closed first.
  * The reference has no counterpart (NCCL never unloads it); a persistent kernel needs an orderly stop. */
 ncclResult_t tcpxFinalize(void);
