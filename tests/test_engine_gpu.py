@@ -574,3 +574,39 @@ def test_other_kernels_run_beside_the_engine(pkg, hip, oracle, benchlib):
     assert torch.equal(out, src)
     got = dst_d.cpu().numpy()
     assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
+
+
+@pytest.mark.parametrize("per_ticket", [0, 3, 16, 64])
+def test_engine_alternating_one_byte_whole_page_and_empty_fragments(pkg, hip, oracle, per_ticket):
+    """Fragments of 1, 4096 and 0 bytes in turn, contiguous in the destination from an odd byte offset, through the
+    engine in slots of 700 descriptors and through the entry point that allocates nothing: destination lines shared
+    by fragments of very different kinds, ticket boundaries falling anywhere among them."""
+    from test_unpack_gpu import alternating_fragments, seeded_pool
+
+    pool = seeded_pool(1 << 20, 17)
+    descs, dst_bytes = alternating_fragments(401, 3, seed=18)
+    expect = oracle_expected(oracle, pool, descs, dst_bytes, 0)
+    g = GpuBuffers(pool, descs, dst_bytes, 0)
+    slots = [(f, min(700, len(descs) - f)) for f in range(0, len(descs), 700)]
+    m = Mapped(pkg, hip, np.ascontiguousarray(descs), len(slots))
+    e = Engine(pkg, hip, descs_per_ticket=per_ticket)
+    print("engine alternating case: %d descriptors, %d slots, tickets of %d" % (len(descs), len(slots), per_ticket), flush=True)
+    e.start()
+    try:
+        for i, (first, n) in enumerate(slots):
+            e.submit(g.pool.data_ptr(), g.dst_base, m.desc_dev(first), n, m.flag_dev(i), i + 1)
+        for i in range(len(slots)):
+            m.wait(i, i + 1)
+    finally:
+        e.stop()
+    got = g.result()
+    e.destroy()
+    assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
+    if per_ticket == 0:
+        g.reset()
+        for i, (first, n) in enumerate(slots):
+            pkg.check(hip.tcpxuUnpackSlotNoAlloc(0, g.pool.data_ptr(), g.dst_base, m.desc_dev(first), n, None, 0, None), "tcpxuUnpackSlotNoAlloc")
+        pkg.check(hip.tcpxuDeviceSynchronize(0), "tcpxuDeviceSynchronize")
+        got = g.result()
+        assert first_difference(got, expect) is None, "no-alloc: first (index, got, want, count): %r" % (first_difference(got, expect),)
+    m.free()

@@ -256,3 +256,27 @@ def test_descriptors_in_host_visible_device_memory(pkg, hip, oracle):
     pkg.check(hip.tcpxuVisibleFree(0, again_h), "tcpxuVisibleFree")
     assert hip.tcpxuVisibleAlloc(0, 0, ctypes.byref(host), ctypes.byref(dev)) == pkg.INVALID_ARGUMENT
     assert hip.tcpxuVisibleAlloc(0, 65 << 20, ctypes.byref(host), ctypes.byref(dev)) == pkg.INVALID_ARGUMENT
+
+
+def alternating_fragments(n_groups, dst_base_offset, seed):
+    """Fragments of 1, 4096 and 0 bytes in turn (and, every fourth group, 300 and 200 bytes: one that may share a
+    line with its neighbours and one too short to), contiguous in the destination from an arbitrary byte offset:
+    one-byte and empty fragments sit between whole pages, so that destination lines are shared by up to four
+    fragments of very different kinds."""
+    rng = np.random.default_rng(seed)
+    rows, dst = [], dst_base_offset
+    for g in range(n_groups):
+        lens = [1, 4096, 0] if g % 4 else [1, 4096, 0, 300, 200]
+        for ln in lens:
+            page = int(rng.integers(0, 250))
+            in_page = int(rng.integers(0, 4096 - ln + 1))
+            rows.append((page * 4096 + in_page, ln, dst))
+            dst += ln
+    return make_descs(rows), dst + 64
+
+
+@pytest.mark.parametrize("offset", [0, 1, 127, 4095])
+def test_alternating_one_byte_whole_page_and_empty_fragments(pkg, hip, oracle, offset):
+    pool = seeded_pool(1 << 20, 7)
+    descs, dst_bytes = alternating_fragments(301, offset, seed=8 + offset)
+    run_batch(pkg, hip, oracle, pool, descs, dst_bytes)
