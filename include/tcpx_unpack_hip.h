@@ -116,7 +116,7 @@ typedef struct tcpxuEngineConfig {
   uint32_t descs_per_ticket;/* descriptors one workgroup takes at a time (1..64); 0 = chosen per submission from
                                the backlog of descriptors not yet unpacked: 8 when the engine is idle (lowest
                                latency), 12, then 16 when every workgroup has work queued (highest throughput), and
-                               with a payload hint that tells of short fragments as many as make 64 KiB, up to 64;
+                               with a payload hint that tells of short fragments 32, 48 or 64;
                                a submission of at most 32 descriptors stays whole once 8 or more are in flight */
   uint32_t spin_limit;      /* the kernel leaves by itself after this many consecutive empty polls of the ring
                                (about 1.2 us each) and is launched again by the next submission, so that a
@@ -142,8 +142,8 @@ int tcpxuEngineSubmit(tcpxuEngine* engine, const void* bounce_base, void* dst_ba
                       uint32_t n_descs, void* done_flag_dev, uint64_t done_value);
 /* The same with a hint: `payload_bytes` = the sum of the descriptors' lengths (the size of the request, which the
  * caller of src/net_tcpx.cc:1354-1357 has at hand in tcpxRequest::offset), 0 = unknown.  The engine hands out a
- * slot's descriptors in tickets of about 64 KiB, 16 fragments of a page; with the hint, a slot of shorter
- * fragments gets tickets of more descriptors (up to 64).  Without it fragments are taken to be whole pages. */
+ * slot's descriptors in tickets of 16 fragments of a page; with the hint, a slot of shorter fragments gets tickets
+ * of more descriptors (32, 48, up to 64).  Without it fragments are taken to be whole pages. */
 int tcpxuEngineSubmitSized(tcpxuEngine* engine, const void* bounce_base, void* dst_base, const void* descs_dev,
                            uint32_t n_descs, uint64_t payload_bytes, void* done_flag_dev, uint64_t done_value);
 

@@ -72,22 +72,19 @@ __host__ __device__ __forceinline__ uint32_t ticket_size_for(uint32_t backlog, u
 // at 8 in flight, 17.5 -> 9.3 us at 32, where the leader's loop had become the queue.)
 //
 // `bytes` is the submission's payload if the caller said (0 = unknown: whole pages).  The largest step, 16, stands
-// for 64 KiB: a submission of shorter fragments gets as many descriptors per ticket as make 64 KiB, in multiples
-// of 8 so that the copy wavefronts' shares come out even, up to 64 (fragments of 2 KiB on average, 64 slots in
-// flight: 52.9 % of the roofline in tickets of 16, 59.1 % in tickets of 32, 61.4 % in tickets of 64).  Written
-// as comparisons: the leader runs this for every submission and a division costs it forty instructions.
+// for whole pages: a submission of shorter fragments gets more descriptors per ticket, in multiples of 16 so that
+// the copy wavefronts' shares come out even, up to 64 (full_ticket_size).  Written as comparisons: the leader runs
+// this for every submission and a division costs it forty instructions.
 constexpr uint32_t kManyInFlight = 8, kSmallSubmission = 32;
 constexpr uint32_t kFullTicket = 16;
 __host__ __device__ __forceinline__ uint32_t full_ticket_size(uint32_t bytes, uint32_t n) {
-  static_assert(kFullTicket == 16 && kMaxDescsPerTicket == 64, "the steps below: 64 KiB / (bytes / n), in eights");
+  static_assert(kFullTicket == 16 && kMaxDescsPerTicket == 64, "the steps below");
   const uint64_t b = bytes;  // n <= 2^20: the products need more than 32 bits
-  return bytes == 0 || b >= 2731ull * n ? 16u
-         : b >= 2048ull * n             ? 24u
-         : b >= 1639ull * n             ? 32u
-         : b >= 1366ull * n             ? 40u
-         : b >= 1171ull * n             ? 48u
-         : b >= 1024ull * n             ? 56u
-                                        : 64u;
+  // Whole pages (or no hint): 16.  Shorter fragments: 32 from two thirds of a page down, 48 from half a page down,
+  // 64 below a third -- about 96 KiB a ticket rather than 64, because a round of a short fragment costs a wavefront
+  // nearly what a whole page costs and only a larger share per pick-up makes up for it (fragments of 1.8 KiB on
+  // average, 64 slots in flight: 59.6 % of the roofline in tickets of 32, 60.6 % in 40, 61.1 % in 48, 61.3 % in 64).
+  return bytes == 0 || b >= 2731ull * n ? 16u : b >= 2048ull * n ? 32u : b >= 1366ull * n ? 48u : 64u;
 }
 __host__ __device__ __forceinline__ uint32_t ticket_size_for_submission(uint32_t in_flight, uint32_t n,
                                                                         uint32_t bytes, uint32_t workers) {

@@ -73,10 +73,11 @@ def test_ticket_plan_arithmetic(pkg):
     assert plan(769, 0, 1, 1078) == (0, 8, 135, 524288)
     assert plan(769, 0, 10, 1078)[1:3] == (12, 90)  # 10780 in flight: 14.04 per worker
     assert plan(769, 0, 64, 1078)[1:3] == (16, 68)
-    # with the payload hint, short fragments get 64 KiB of descriptors per ticket, in eights, at most 64
+    # with the payload hint, short fragments get more descriptors per ticket: 32, 48, at most 64
     assert plan(769, 0, 64, 2048, 2048 * 4096)[1] == 16
-    assert plan(769, 0, 64, 2048, 2048 * 2048)[1] == 24
-    assert plan(769, 0, 64, 2048, 2048 * 2047)[1] == 32
+    assert plan(769, 0, 64, 2048, 2048 * 2731)[1] == 16 and plan(769, 0, 64, 2048, 2048 * 2730)[1] == 32
+    assert plan(769, 0, 64, 2048, 2048 * 2048)[1] == 32 and plan(769, 0, 64, 2048, 2048 * 2047)[1] == 48
+    assert plan(769, 0, 64, 2048, 2048 * 1366)[1] == 48 and plan(769, 0, 64, 2048, 2048 * 1365)[1] == 64
     assert plan(769, 0, 64, 2048, 2048 * 100)[1:3] == (64, 32)
     # a small submission among many stays one ticket
     assert plan(769, 0, 8, 32)[1:3] == (32, 1) and plan(769, 0, 7, 32)[1:3] == (8, 4)

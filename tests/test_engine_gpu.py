@@ -503,8 +503,14 @@ def test_engine_run_window_times_the_middle_of_a_stream(pkg, hip, oracle, benchl
 
 def test_other_kernels_run_beside_the_engine(pkg, hip, oracle, benchlib):
     """The engine takes two workgroups of nine wavefronts per compute unit and leaves the rest of each to others:
-    while it streams 64 slots of 4 MiB on its own stream, copy kernels launched on another stream must start and
-    finish (each within a deadline), their bytes must be right, and the unpack must still be byte-exact."""
+    while it streams 64 slots of 4 MiB on its own stream, copy kernels launched on other streams must start and
+    finish (each within a deadline), their bytes must be right, and the unpack must still be byte-exact.
+    Four other streams carry the copies.  Each has run one copy before the engine starts: a stream's first launch
+    sets up its hardware queue, and the kernel's first launch loads its code, both of which take milliseconds
+    when the device is busy, as long as the whole engine launch measured here.  The runtime spreads a process's
+    streams over a few hardware queues (four by default) and a queue starts its kernels in order, so a stream that
+    shares the engine's queue gets its turn when the engine kernel leaves; the others must make progress beside
+    it, which is what is asserted: copies finish on at least two of the four streams while the engine runs."""
     import threading
 
     import torch
@@ -534,7 +540,12 @@ def test_other_kernels_run_beside_the_engine(pkg, hip, oracle, benchlib):
     n_copy = 64 << 20
     src = torch.randint(0, 256, (n_copy,), dtype=torch.uint8, device="cuda:0")
     out = torch.zeros(n_copy, dtype=torch.uint8, device="cuda:0")
-    side = torch.cuda.Stream()
+    sides = [torch.cuda.Stream() for _ in range(4)]
+    for side in sides:
+        pkg.check(benchlib.tcpxuCopyKernelLaunch(0, out.data_ptr(), src.data_ptr(), n_copy, side.cuda_stream), "tcpxuCopyKernelLaunch")
+    torch.cuda.synchronize()
+    assert torch.equal(out, src)
+    out.zero_()
     torch.cuda.synchronize()
     e = Engine(pkg, hip)
     cfg = pkg.EngineConfig()
@@ -546,7 +557,9 @@ def test_other_kernels_run_beside_the_engine(pkg, hip, oracle, benchlib):
 
     def stream_all():
         wall, kern = ctypes.c_double(), ctypes.c_double()
+        result["t0"] = time.perf_counter()
         result["rc"] = benchlib.tcpxuEngineRunTimed(e.h, items, len(flat), 0, 64, 20000, ctypes.byref(wall), ctypes.byref(kern), None)
+        result["t1"] = time.perf_counter()
         result["kernel_us"] = kern.value
 
     print("co-residency case: %d slots on the engine, copies of %d MiB beside it" % (len(flat), n_copy >> 20), flush=True)
@@ -554,21 +567,28 @@ def test_other_kernels_run_beside_the_engine(pkg, hip, oracle, benchlib):
     t.start()
     while not e.running() and t.is_alive():  # the launch is the thread's first act
         time.sleep(20e-6)
-    copies_while_running = 0
+    finished = [[] for _ in sides]  # when each stream's copies were seen finished
+    pending = [None] * len(sides)
     while t.is_alive():
-        pkg.check(benchlib.tcpxuCopyKernelLaunch(0, out.data_ptr(), src.data_ptr(), n_copy, side.cuda_stream), "tcpxuCopyKernelLaunch")
-        done = torch.cuda.Event()
-        done.record(side)
-        deadline = time.time() + 10
-        while not done.query():
-            assert time.time() < deadline, "a copy kernel did not finish while the engine was running"
-        if t.is_alive() and e.running():
-            copies_while_running += 1
+        for k, side in enumerate(sides):
+            if pending[k] is None:
+                pkg.check(benchlib.tcpxuCopyKernelLaunch(0, out.data_ptr(), src.data_ptr(), n_copy, side.cuda_stream), "tcpxuCopyKernelLaunch")
+                pending[k] = torch.cuda.Event()
+                pending[k].record(side)
+            elif pending[k].query():
+                pending[k] = None
+                finished[k].append(time.perf_counter())
     t.join(timeout=30)
     assert not t.is_alive() and result["rc"] == 0
-    side.synchronize()
-    print("co-residency case: %d copies finished while the engine streamed (%.0f us launch)" % (copies_while_running, result["kernel_us"]), flush=True)
-    assert copies_while_running >= 1, "no copy kernel finished while the engine kernel was running"
+    deadline = time.time() + 10
+    for side in sides:  # a copy that shared the engine's hardware queue runs now
+        while not side.query():
+            assert time.time() < deadline, "a copy kernel did not finish after the engine had stopped"
+    # a copy counts if it was seen finished well before the engine's launch ended (the launch is over 4 ms long)
+    beside = [sum(1 for x in f if result["t0"] < x < result["t1"] - 5e-4) for f in finished]
+    copies_while_running = sum(beside)
+    print("co-residency case: copies finished while the engine streamed, per stream: %r (%.0f us launch)" % (beside, result["kernel_us"]), flush=True)
+    assert copies_while_running >= 1 and sum(b > 0 for b in beside) >= 2, "copy kernels on other streams must run while the engine kernel is running"
     assert e.completed() == len(flat)
     e.destroy()
     assert torch.equal(out, src)
