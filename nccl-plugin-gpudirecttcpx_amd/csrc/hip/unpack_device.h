@@ -133,30 +133,28 @@ struct CopyRegs {
 };
 constexpr uint32_t kLineVecs = kLineBytes / 16;  // lanes that take part in the shared line
 
-// What a lane below kLineVecs does for the shared last line: vector `lane` of the line is bytes [shift, shift+16)
-// of A:B with A = 16 bytes at src_frag + off_a and B = 16 bytes at src_next + off_b.
-struct LineLane {
-  uint32_t off_a, off_b, shift, dst_off;
+// The shared last line, lanes 0..7, one 16-byte vector each.  The fragment (A) has `rem` = frag_len - line_off bytes
+// in the line (1..127), the next fragment (B) the rest.  Where the boundary falls is the same for the whole
+// wavefront, so nothing here is worked out per lane beyond an address:
+//   vectors before the boundary are 16 bytes of A, vectors after it 16 bytes of B, each loaded where it lies
+//   (any alignment) and stored as loaded;
+//   the one vector the boundary cuts (none if rem is a multiple of 16) is the last `cut` bytes of A followed by
+//   the first 16 - cut bytes of B: its lane loads A's last 16 bytes and B's first 16 and takes bytes
+//   [16 - cut, 32 - cut) of the two, a shift by a wave-uniform amount.
+// Both neighbours are at least kShareMinLen long, so every one of these loads stays inside its fragment.
+// (An earlier form gave every lane two loads and a shift of its own, by a per-lane amount: some sixty vector
+// instructions a line instead of some twenty, a sixth of the time of a round of a 2 KiB fragment.)
+struct LinePlan {
+  uint32_t rem;       // bytes of this fragment in the line
+  uint32_t cut_lane;  // the vector the boundary falls in
+  uint32_t cut;       // bytes of this fragment in that vector, 0 = the boundary falls between two vectors
 };
-__device__ __forceinline__ LineLane line_lane(const CopyRound& c, uint32_t lane) {
-  LineLane l;
-  const uint32_t x = c.line_off + ((lane & (kLineVecs - 1)) << 4);  // this vector's offset from the fragment's start
-  const int32_t own = static_cast<int32_t>(c.frag_len) - static_cast<int32_t>(x);  // bytes still in this fragment
-  l.dst_off = x;
-  if (own >= 16) {  // entirely this fragment
-    l.off_a = x;
-    l.off_b = 0;
-    l.shift = 0;
-  } else if (own <= 0) {  // entirely the next fragment
-    l.off_a = c.frag_len - 16u;
-    l.off_b = static_cast<uint32_t>(-own);
-    l.shift = 16;
-  } else {  // the last `own` bytes of this fragment, then the first bytes of the next
-    l.off_a = c.frag_len - 16u;
-    l.off_b = 0;
-    l.shift = 16u - static_cast<uint32_t>(own);
-  }
-  return l;
+__device__ __forceinline__ LinePlan line_plan(const CopyRound& c) {
+  LinePlan p;
+  p.rem = c.frag_len - c.line_off;
+  p.cut_lane = p.rem >> 4;
+  p.cut = p.rem & 15u;
+  return p;
 }
 
 // Source realignment.  A 16-byte load whose address is not a multiple of 4 is split by the memory pipeline and
@@ -193,10 +191,15 @@ __device__ __forceinline__ void round_load(const CopyRound& c, CopyRegs& x, uint
     if (lane == 0) x.tail_dword = load_dword_sys(base4 + (c.nvec << 4));
   }
   if (c.share_next) {
+    const LinePlan p = line_plan(c);
     if (lane < kLineVecs) {
-      const LineLane l = line_lane(c, lane);
-      x.line_a = load_vec_sys(c.src_frag + l.off_a);
-      x.line_b = load_vec_sys(c.src_next + l.off_b);
+      const uint32_t off = lane << 4;
+      const uint8_t* from = lane < p.cut_lane ? c.src_frag + c.line_off + off : c.src_next + (off - p.rem);
+      if (p.cut != 0 && lane == p.cut_lane) from = c.src_frag + c.frag_len - 16u;
+      x.line_a = load_vec_sys(from);
+    }
+    if (p.cut != 0) {
+      if (lane == p.cut_lane) x.line_b = load_vec_sys(c.src_next);
     }
   }
 }
@@ -239,10 +242,13 @@ __device__ __forceinline__ void round_store_loaded(const CopyRound& c, CopyRegs&
     if (v < c.nvec) store_vec_stream(c.dst_vec + (v << 4), out);
   }
   if (c.share_next) {
-    if (lane < kLineVecs) {
-      const LineLane l = line_lane(c, lane);
-      store_vec_stream(c.dst_frag + l.dst_off, extract16(x.line_a, x.line_b, l.shift));
+    const LinePlan p = line_plan(c);
+    u32x4 line = x.line_a;
+    if (p.cut != 0) {
+      const u32x4 cut_vector = extract16(x.line_a, x.line_b, 16u - p.cut);
+      if (lane == p.cut_lane) line = cut_vector;
     }
+    if (lane < kLineVecs) store_vec_stream(c.dst_frag + c.line_off + (lane << 4), line);
   }
   if (c.has_edge) {
     if (c.edge_off != kNoEdge) store_byte_sys(c.dst_frag + c.edge_off, static_cast<uint8_t>(x.edge_byte));
@@ -432,9 +438,11 @@ __device__ __forceinline__ void wave_copy_descriptors(const tcpxuLoadMeta* descs
   if (!cursor.produce(r, r, lane, on_take)) return;
   for (;;) {
     round_load(r, x, lane);
-    round_store(r, x, lane);
+    // The next round is worked out while this one's loads are on their way.
     CopyRound nxt;
-    if (!cursor.produce(nxt, r, lane, on_take)) return;
+    const bool more = cursor.produce(nxt, r, lane, on_take);
+    round_store(r, x, lane);
+    if (!more) return;
     r = nxt;
   }
 }

@@ -630,3 +630,35 @@ def test_engine_alternating_one_byte_whole_page_and_empty_fragments(pkg, hip, or
         got = g.result()
         assert first_difference(got, expect) is None, "no-alloc: first (index, got, want, count): %r" % (first_difference(got, expect),)
     m.free()
+
+
+@pytest.mark.parametrize("per_ticket", [0, 3, 64])
+def test_engine_every_boundary_position_inside_a_shared_line(pkg, hip, oracle, per_ticket):
+    """Runs of three contiguous fragments with their boundaries at every offset inside a 128-byte line, through the
+    engine (tickets of 3 descriptors hold exactly one run, the adaptive size and 64 cut runs anywhere) and through
+    the entry point that allocates nothing."""
+    from test_unpack_gpu import boundary_runs, seeded_pool
+
+    pool = seeded_pool(1 << 20, 31)
+    descs, dst_bytes = boundary_runs(32 + per_ticket)
+    expect = oracle_expected(oracle, pool, descs, dst_bytes, 0)
+    g = GpuBuffers(pool, descs, dst_bytes, 0)
+    m = Mapped(pkg, hip, np.ascontiguousarray(descs), 1)
+    e = Engine(pkg, hip, descs_per_ticket=per_ticket)
+    print("engine boundary case: %d descriptors, tickets of %d" % (len(descs), per_ticket), flush=True)
+    e.start()
+    try:
+        e.submit(g.pool.data_ptr(), g.dst_base, m.desc_dev(0), len(descs), m.flag_dev(0), 1)
+        m.wait(0, 1)
+    finally:
+        e.stop()
+    got = g.result()
+    e.destroy()
+    assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
+    if per_ticket == 0:
+        g.reset()
+        pkg.check(hip.tcpxuUnpackSlotNoAlloc(0, g.pool.data_ptr(), g.dst_base, m.desc_dev(0), len(descs), None, 0, None), "tcpxuUnpackSlotNoAlloc")
+        pkg.check(hip.tcpxuDeviceSynchronize(0), "tcpxuDeviceSynchronize")
+        got = g.result()
+        assert first_difference(got, expect) is None, "no-alloc: first (index, got, want, count): %r" % (first_difference(got, expect),)
+    m.free()

@@ -280,3 +280,46 @@ def test_alternating_one_byte_whole_page_and_empty_fragments(pkg, hip, oracle, o
     pool = seeded_pool(1 << 20, 7)
     descs, dst_bytes = alternating_fragments(301, offset, seed=8 + offset)
     run_batch(pkg, hip, oracle, pool, descs, dst_bytes)
+
+
+def boundary_runs(seed, pool_bytes=1 << 20):
+    """Runs of three fragments that continue each other in the destination, every fragment at least 256 bytes (long
+    enough to share a line with its neighbour), with the two boundaries of each run at chosen offsets inside a
+    128-byte line: all 128 offsets occur as a first boundary, each with a different second one.  Sources have any
+    byte alignment; in every fourth run the first fragment ends exactly at the end of its bounce page, in every
+    eighth at the end of the pool, with the next fragment at the start of a page.  Runs are separated by a byte
+    that must survive; in every third run an empty descriptor sits between the first two fragments."""
+    rng = np.random.default_rng(seed)
+    pages = pool_bytes // 4096
+    rows, dst = [], 0
+    for b1 in range(128):
+        b2 = (b1 * 7 + 13) % 128
+        start = int(rng.integers(0, 128))
+        dst = (dst + 127) // 128 * 128 + start
+        len_a = 256 + int(rng.integers(0, 12)) * 128 + (b1 - start - 256) % 128
+        len_b = 256 + int(rng.integers(0, 12)) * 128 + (b2 - b1 - 256) % 128
+        len_c = 256 + int(rng.integers(0, 3000))
+        assert (dst + len_a) % 128 == b1 and (dst + len_a + len_b) % 128 == b2
+        for i, ln in enumerate((len_a, len_b, len_c)):
+            page = int(rng.integers(0, pages))
+            in_page = int(rng.integers(0, 4096 - ln + 1))
+            if i == 0 and b1 % 4 == 0:
+                in_page = 4096 - ln
+                if b1 % 8 == 0:
+                    page = pages - 1
+            if i == 1 and b1 % 4 == 0:
+                in_page = 0
+            rows.append((page * 4096 + in_page, ln, dst))
+            dst += ln
+            if i == 0 and b1 % 3 == 0:
+                rows.append((page * 4096, 0, dst))  # an empty descriptor between two that continue each other
+        dst += 1
+    return make_descs(rows), dst + 64
+
+
+def test_every_boundary_position_inside_a_shared_line(pkg, hip, oracle):
+    pool = seeded_pool(1 << 20, 21)
+    for seed in (22, 23):
+        descs, dst_bytes = boundary_runs(seed)
+        run_batch(pkg, hip, oracle, pool, descs, dst_bytes)
+        run_batch(pkg, hip, oracle, pool, descs, dst_bytes, misalign=5)
