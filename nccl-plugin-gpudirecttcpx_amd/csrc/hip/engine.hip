@@ -834,16 +834,18 @@ int tcpxuEngineCreate(int device, const tcpxuEngineConfig* config, tcpxuEngine**
   const uint32_t cus = static_cast<uint32_t>(std::max(1, device_compute_units(device)));
   if (cfg.workgroups == 0) {
     // Two worker workgroups per compute unit: 18 of a compute unit's 32 wavefront slots, so that other kernels
-    // (copies, the caller's own work) are scheduled beside the engine while it runs.  More buys nothing: the
-    // memory system is full with two (8 MiB chunks, 64 slots in flight: 70.8 % of the HBM roofline with two, 70.7 %
-    // with three; one is not enough, 59 %), and requests/s of small requests is the same or better with two.
-    // (Fixed rather than asked of the occupancy query: the kernel needs 56 vector registers and 6.2 KiB of LDS,
-    // three of its workgroups fit a compute unit, and the query has answered "one" in a process that had launched
-    // other kernels before.  A grid larger than what is resident would still be correct -- no workgroup waits for
-    // another worker -- only pointless.)
+    // (copies, the caller's own work) are scheduled beside the engine while it runs.  One is not enough (8 MiB
+    // chunks, 64 slots in flight: 59 % of the HBM roofline against 71 %; fragments of 2 KiB: 41 % against 66 %).
+    // Two is also all that is ever resident: the nine wavefronts of a workgroup go to the four SIMDs as 3+2+2+2,
+    // a third workgroup would need a ninth slot on the first SIMD, and the hardware counters show a grid of
+    // three per compute unit running exactly the wavefront-cycles of two.  (Workgroups of twelve wavefronts, two
+    // per compute unit, do fit: 22 copy wavefronts instead of 16 move short fragments 1 % faster and whole pages
+    // no faster, and leave other kernels 8 slots instead of 14.)  The occupancy query is not asked: it has answered
+    // "one" in a process that had launched other kernels before.  A grid larger than what is resident would still
+    // be correct -- no workgroup waits for another worker -- only pointless.
     uint32_t per_cu = 2;
-    const char* v = getenv("TCPXU_ENGINE_WGS_PER_CU");  // tuning aid: 1..3
-    if (v && *v) per_cu = std::min(std::max(static_cast<uint32_t>(atoi(v)), 1u), 3u);
+    const char* v = getenv("TCPXU_ENGINE_WGS_PER_CU");  // tuning aid: 1 or 2
+    if (v && *v) per_cu = std::min(std::max(static_cast<uint32_t>(atoi(v)), 1u), 2u);
     cfg.workgroups = cus * per_cu + 1;
   }
   if (cfg.workgroups < 2 || cfg.workgroups > (1u << 16)) {
