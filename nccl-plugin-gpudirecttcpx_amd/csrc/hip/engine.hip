@@ -76,6 +76,7 @@ __host__ __device__ __forceinline__ uint32_t ticket_size_for(uint32_t backlog, u
 // the copy wavefronts' shares come out even, up to 64 (full_ticket_size).  Written as comparisons: the leader runs
 // this for every submission and a division costs it forty instructions.
 constexpr uint32_t kManyInFlight = 8, kSmallSubmission = 32;
+constexpr uint32_t kLeaderBehind = 8;  // entries waiting in one poll from which the leader counts as the bottleneck
 constexpr uint32_t kFullTicket = 16;
 __host__ __device__ __forceinline__ uint32_t full_ticket_size(uint32_t bytes, uint32_t n) {
   static_assert(kFullTicket == 16 && kMaxDescsPerTicket == 64, "the steps below");
@@ -224,6 +225,12 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
 
     const uint32_t expect = static_cast<uint32_t>(s + k_of_lane + 1);
     const uint64_t ok_mask = __ballot(sect.w == expect);
+    // Entries of this poll that are there, counted from the first: lane 4k tells whether all four sectors of entry
+    // k are.  Eight or more mean that submissions queue up at the leader itself.
+    const uint64_t whole = ok_mask & (ok_mask >> 1) & (ok_mask >> 2) & (ok_mask >> 3) & 0x1111111111111111ull;
+    const uint64_t missing = ~whole & 0x1111111111111111ull;
+    const uint32_t ready = missing != 0 ? static_cast<uint32_t>(__builtin_ctzll(missing)) >> 2 : kPollEntries;
+    const bool leader_behind = ready >= kLeaderBehind;
     const uint32_t tickets_done = lane_value(aux, kAuxTicketsDone);
     const uint32_t jobs_completed = lane_value(aux, kAuxJobsCompleted);
     // Payload word i of entry k: component i % 3 of sector i / 3, held by lane 4k + i / 3.
@@ -289,9 +296,15 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
       } else {
         // Submissions not yet completed, this one included, taken to be as long as this one.
         const uint32_t in_flight = static_cast<uint32_t>(s + k) - jobs_completed + 1u;
-        const uint32_t per_ticket = fixed_per_ticket != 0
-                                        ? fixed_per_ticket
-                                        : ticket_size_for_submission(in_flight, n, payload_of(fl, 11), gridDim.x - 1);
+        uint32_t per_ticket = fixed_per_ticket != 0
+                                  ? fixed_per_ticket
+                                  : ticket_size_for_submission(in_flight, n, payload_of(fl, 11), gridDim.x - 1);
+        // Small tickets spread a small backlog over many workgroups, at the price of more tickets to write.  When
+        // submissions queue up at the leader, its time per submission is what limits the engine, not the spread:
+        // a stream of 1 MiB requests of 256 whole pages, 64 in flight, is served at 1.44 M/s in tickets of 8 (which
+        // the backlog alone asks for: the workers empty it as fast as it comes), at 1.96 M/s in tickets of 16, and at
+        // 1.64 M/s with this rule, which holds for part of the time.
+        if (fixed_per_ticket == 0 && leader_behind && per_ticket < kFullTicket) per_ticket = kFullTicket;
         const uint32_t nt = (n + per_ticket - 1) / per_ticket;
         const uint32_t slot = static_cast<uint32_t>(s + k) & ring_mask;
         const uint32_t done_now = lane_value(aux, k);
