@@ -558,7 +558,12 @@ def main():
 
     if not args.skip_extras and not args.one_launch:
         result["plugin_path"] = plugin_path(pkg, hip, torch, workloads[: min(8, args.chunks)], pool)
-        result["plugin_path"]["with_socket_thread"] = plugin_path(pkg, hip, torch, workloads[: min(8, args.chunks)], pool, helper_thread=True)
+        # Two threads that hand every fragment run to each other: the figure depends on where the machine puts them
+        # (on the virtual CPUs of the test boxes it comes out near 46 GB/s in most runs and near 11 GB/s in some,
+        # with nothing else different), so the leg runs three times and reports the median beside all three.
+        legs = [plugin_path(pkg, hip, torch, workloads[: min(8, args.chunks)], pool, helper_thread=True) for _ in range(3)]
+        legs.sort(key=lambda leg: leg.get("payload_GBps", 0.0))
+        result["plugin_path"]["with_socket_thread"] = dict(legs[1], payload_GBps_of_three_runs=[leg.get("payload_GBps") for leg in legs])
 
     # ---- CPU baseline on this machine's host cores: rank 0, bounded sample ---------------------------------
     # Threads: the cores this process may run on.  A GPU box shows every core of the host to os.cpu_count() while a

@@ -200,7 +200,21 @@ ncclResult_t flow_progress(Comm* comm, int flow) {
   return ncclSuccess;
 }
 
+// A pass of the socket thread that found nothing to do: wait a moment without leaving the CPU while work may be
+// on its way (tasks arrive every few microseconds under load, and a system call per empty pass costs more than
+// that on some machines), give the CPU away once the comm has been quiet for a while.
+inline void idle_pass(uint32_t* quiet_passes) {
+  if (++*quiet_passes < 4096) {
+#if defined(__x86_64__) || defined(__i386__)
+    __builtin_ia32_pause();
+#endif
+  } else {
+    sched_yield();
+  }
+}
+
 void helper_main(Comm* comm) {  // persistentSocketThread, src/net_tcpx.cc:252-384 (receive part)
+  uint32_t quiet_passes = 0;
   while (!comm->helper_stop.load(std::memory_order_acquire)) {
     bool idle = true;
     for (int f = 0; f < comm->num_flows; ++f) {
@@ -210,7 +224,8 @@ void helper_main(Comm* comm) {  // persistentSocketThread, src/net_tcpx.cc:252-3
         idle = false;
       }
     }
-    if (idle) sched_yield();
+    if (idle) idle_pass(&quiet_passes);
+    else quiet_passes = 0;
   }
 }
 
