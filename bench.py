@@ -163,7 +163,7 @@ def batch_kernel_line(pkg, benchlib, torch, dev, chunks=128, pools=15, warmup=3,
     }
 
 
-def other_configs(pkg, torch, run):
+def other_configs(pkg, torch, run, only=None):
     """The other workloads of the measurement contract through the same engine, 64 slots in flight.  A pass re-reads
     the pages of the pass `pool_copies` before it, so the copies are as many as it takes for 2 GiB of traffic to pass
     in between (eight times the Infinity Cache), except for config 1, which is cache-resident by construction.
@@ -174,6 +174,8 @@ def other_configs(pkg, torch, run):
         (5, 512, 32, "adversarial: 32 MiB, fragment lengths uniform in 1..4096, 10% empty descriptors, destination offset by 3 bytes"),
         (1, 2048, 1, "one 1 MiB message of 256 page-aligned fragments from a 16 MiB pool: cache-resident by construction"),
     ):
+        if only is not None and cfg != only:
+            continue
         wl = pkg.Workload(cfg, seed=0xC0FFEE00 + cfg)
         info = wl.info
         pool_bytes, dst_bytes = int(info.pool_bytes), int(info.dst_bytes)
@@ -206,6 +208,8 @@ def other_configs(pkg, torch, run):
             "payload_GBps": round(payload / (wall_us * 1e-6) / 1e9, 1),
             "rw_frac_of_hbm_peak": round(2.0 * payload / (wall_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
         }
+        if only is not None:  # the whole launch, first pass included, as a profiler sees it
+            out["config_%d" % cfg].update(passes=passes, bytes_per_launch=2.0 * float(info.payload_bytes) * passes, launch_us=round(kernel_us, 1))
         del pool_d, dst_d
     return out
 
@@ -235,6 +239,7 @@ def main():
         help="exactly one launch of the engine kernel in the process (no untimed launch before it, no single-comm run, "
         "no extras): what a kernel trace or a counter run of the headline should see",
     )
+    ap.add_argument("--one-config", type=int, default=0, choices=[0, 1, 4, 5], help="exactly one launch of the engine kernel over this other workload of the contract (1, 4 or 5), 64 slots in flight, and exit: for a profiler")
     ap.add_argument(
         "--calibrate-copy",
         type=int,
@@ -276,6 +281,30 @@ def main():
         return
     if args.batch_kernel:
         print(json.dumps(batch_kernel_line(pkg, benchlib, torch, dev)))
+        return
+    if args.one_config:
+        # One launch of the engine kernel over one of the other workloads, after 150 launches of the plain copy kernel
+        # (60 ms of load, so that the GPU is in the state it sustains).
+        n = 512 << 20
+        a = torch.empty(n, dtype=torch.uint8, device="cuda:0").random_(0, 256)
+        b = torch.empty(n, dtype=torch.uint8, device="cuda:0")
+        torch.cuda.synchronize()
+        us = ctypes.c_double()
+        pkg.check(benchlib.tcpxuCopyKernelTimed(dev, b.data_ptr(), a.data_ptr(), n, 0, 150, ctypes.byref(us)), "tcpxuCopyKernelTimed")
+        del a, b
+        engine = ctypes.c_void_p()
+        cfg = pkg.EngineConfig(0, 0, 0, 0)
+        pkg.check(hip.tcpxuEngineCreate(dev, ctypes.byref(cfg), ctypes.byref(engine)), "tcpxuEngineCreate")
+
+        def run_once(items, depth, warmup_items=0):
+            wall, kern = ctypes.c_double(), ctypes.c_double()
+            rc = benchlib.tcpxuEngineRunTimed(engine, items, len(items), warmup_items, depth, 20000, ctypes.byref(wall), ctypes.byref(kern), None)
+            pkg.check(rc, "tcpxuEngineRunTimed")
+            return wall.value, kern.value, None
+
+        out = other_configs(pkg, torch, run_once, only=args.one_config)
+        pkg.check(hip.tcpxuEngineDestroy(engine), "tcpxuEngineDestroy")
+        print(json.dumps(dict(out["config_%d" % args.one_config], kernel="unpack_engine_kernel", slots_in_flight=64)))
         return
     name = ctypes.create_string_buffer(256)
     cus = ctypes.c_int()

@@ -81,3 +81,9 @@ def test_bench_extras_report_latency_and_the_storm_sweep():
     assert r["launch_per_batch_1GiB"]["kernel"] == "unpack_batch_kernel" and r["launch_per_batch_1GiB"]["rw_GBps"] > 0
     yard = r["hbm_yardsticks"]
     assert yard["read_only_GBps"] > 0 and yard["write_only_GBps"] > 0 and yard["copy_bound_rw_GBps"] > 0
+
+
+def test_one_config_mode_launches_the_engine_once_over_another_workload():
+    r = run_bench(["--one-config", "1"], timeout=300)
+    assert r["kernel"] == "unpack_engine_kernel" and r["slots_in_flight"] == 64 and r["requests_per_pass"] == 1
+    assert r["bytes_per_launch"] == 2.0 * (1 << 20) * r["passes"] and r["launch_us"] > 0 and r["payload_GBps"] > 0
