@@ -662,3 +662,48 @@ def test_engine_every_boundary_position_inside_a_shared_line(pkg, hip, oracle, p
         got = g.result()
         assert first_difference(got, expect) is None, "no-alloc: first (index, got, want, count): %r" % (first_difference(got, expect),)
     m.free()
+
+
+@pytest.mark.parametrize("seed", range(200, 212))
+def test_engine_random_mixtures_of_fragment_kinds(pkg, hip, oracle, seed):
+    """Descriptor lists drawn from a seed (every kind of fragment beside every other, gaps now and then), in slots of
+    a random size, through the engine at a ticket size drawn from the seed, and through the entry point that
+    allocates nothing."""
+    from test_unpack_gpu import random_mixture, seeded_pool
+
+    rng = np.random.default_rng(seed)
+    pool = seeded_pool(1 << 20, seed)
+    descs, dst_bytes = random_mixture(seed)
+    per_ticket = int(rng.choice([0, 0, 1, 5, 16, 33, 64]))
+    slot = int(rng.integers(1, 2049))
+    expect = oracle_expected(oracle, pool, descs, dst_bytes, 0)
+    g = GpuBuffers(pool, descs, dst_bytes, 0)
+    slots = [(f, min(slot, len(descs) - f)) for f in range(0, len(descs), slot)]
+    m = Mapped(pkg, hip, np.ascontiguousarray(descs), len(slots))
+    e = Engine(pkg, hip, descs_per_ticket=per_ticket)
+    print("engine mixture case: seed %d, %d descriptors, slots of %d, tickets of %d" % (seed, len(descs), slot, per_ticket), flush=True)
+    e.start()
+    try:
+        for i, (first, n) in enumerate(slots):
+            nbytes = int(descs["len"][first : first + n].sum()) if seed % 2 else 0  # with and without the payload hint
+            deadline = time.time() + 20
+            while True:
+                rc = hip.tcpxuEngineSubmitSized(e.h, g.pool.data_ptr(), g.dst_base, m.desc_dev(first), n, min(nbytes, 0xFFFFFFFF), m.flag_dev(i), i + 1)
+                if rc != pkg.IN_PROGRESS:
+                    break
+                assert time.time() < deadline, "submission ring stayed full"
+            pkg.check(rc, "tcpxuEngineSubmitSized")
+        for i in range(len(slots)):
+            m.wait(i, i + 1)
+    finally:
+        e.stop()
+    got = g.result()
+    e.destroy()
+    assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
+    g.reset()
+    for first, n in slots:
+        pkg.check(hip.tcpxuUnpackSlotNoAlloc(0, g.pool.data_ptr(), g.dst_base, m.desc_dev(first), n, None, 0, None), "tcpxuUnpackSlotNoAlloc")
+    pkg.check(hip.tcpxuDeviceSynchronize(0), "tcpxuDeviceSynchronize")
+    got = g.result()
+    assert first_difference(got, expect) is None, "no-alloc: first (index, got, want, count): %r" % (first_difference(got, expect),)
+    m.free()

@@ -323,3 +323,31 @@ def test_every_boundary_position_inside_a_shared_line(pkg, hip, oracle):
         descs, dst_bytes = boundary_runs(seed)
         run_batch(pkg, hip, oracle, pool, descs, dst_bytes)
         run_batch(pkg, hip, oracle, pool, descs, dst_bytes, misalign=5)
+
+
+def random_mixture(seed, pool_bytes=1 << 20, max_descs=3000):
+    """A descriptor list drawn from a seed: empty, tiny, short, medium, whole-page and longer-than-a-page fragments in
+    random order, mostly continuing each other in the destination (so that lines are shared by every kind of
+    neighbour) with gaps now and then, sources at any byte offset."""
+    rng = np.random.default_rng(seed)
+    n = int(rng.integers(1, max_descs + 1))
+    kinds = rng.choice(6, size=n, p=[0.10, 0.10, 0.25, 0.30, 0.20, 0.05])
+    rows, dst = [], int(rng.integers(0, 256))
+    for kind in kinds:
+        ln = (0, int(rng.integers(1, 31)), int(rng.integers(31, 601)), int(rng.integers(601, 4096)), 4096, int(rng.integers(4097, 20001)))[kind]
+        if ln <= 4096:
+            src = int(rng.integers(0, pool_bytes // 4096)) * 4096 + int(rng.integers(0, 4096 - ln + 1))
+        else:
+            src = int(rng.integers(0, pool_bytes - ln + 1))
+        if rng.random() < 0.2:
+            dst += int(rng.integers(1, 301))
+        rows.append((src, ln, dst))
+        dst += ln
+    return make_descs(rows), dst + 64
+
+
+@pytest.mark.parametrize("seed", range(100, 112))
+def test_random_mixtures_of_fragment_kinds(pkg, hip, oracle, seed):
+    pool = seeded_pool(1 << 20, seed)
+    descs, dst_bytes = random_mixture(seed)
+    run_batch(pkg, hip, oracle, pool, descs, dst_bytes, misalign=seed % 16)
