@@ -156,6 +156,8 @@ int tcpxuEngineSubmitSized(tcpxuEngine* engine, const void* bounce_base, void* d
  * the given descs_per_ticket (0 = by backlog), a submission of n_descs descriptors and payload_bytes (0 = unknown)
  * with `in_flight` submissions not yet completed (itself included) is handed out in *n_tickets tickets of
  * *per_ticket descriptors; *max_descs is the most descriptors a submission may carry.  Outputs may be NULL.
+ * (One more rule lives in the kernel alone, because it depends on what the leader finds at run time: while eight or
+ * more submissions wait in one of its polls, tickets sized by backlog are at least 16 descriptors.)
  * TCPXU_INVALID_ARGUMENT for an n_descs beyond that limit. */
 int tcpxuEngineTicketPlan(uint32_t workgroups, uint32_t descs_per_ticket, uint32_t in_flight, uint32_t n_descs,
                           uint64_t payload_bytes, uint32_t* per_ticket, uint32_t* n_tickets, uint32_t* max_descs);
