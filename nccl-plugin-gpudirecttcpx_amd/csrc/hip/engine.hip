@@ -76,6 +76,7 @@ __host__ __device__ __forceinline__ uint32_t ticket_size_for(uint32_t backlog, u
 // the copy wavefronts' shares come out even, up to 64 (full_ticket_size).  Written as comparisons: the leader runs
 // this for every submission and a division costs it forty instructions.
 constexpr uint32_t kManyInFlight = 8, kSmallSubmission = 32;
+constexpr uint32_t kLaneTickets = 32;  // tickets of one submission that the lanes holding its entry still write themselves
 constexpr uint32_t kLeaderBehind = 8;  // entries waiting in one poll from which the leader counts as the bottleneck
 constexpr uint32_t kFullTicket = 16;
 __host__ __device__ __forceinline__ uint32_t full_ticket_size(uint32_t bytes, uint32_t n) {
@@ -197,8 +198,14 @@ __device__ __forceinline__ uint32_t lane_value(uint32_t v, uint32_t src_lane) {
 __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uint32_t* job_target,
                             uint32_t ring_mask, uint32_t fixed_per_ticket, uint32_t spin_limit) {
   const uint32_t lane = threadIdx.x;
-  uint64_t s = sys_load(&st->sub_head);
-  uint64_t tickets_out = sys_load(&st->tickets_out);
+  // The leader's positions are the same in every lane: said outright, so that they stay in scalar registers (in
+  // vector registers the compiler waits for the leader's own stores at the top of every pass).
+  auto same_in_all_lanes = [](uint64_t v) {
+    return (static_cast<uint64_t>(static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(v >> 32)))) << 32) |
+           static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(v)));
+  };
+  uint64_t s = same_in_all_lanes(sys_load(&st->sub_head));
+  uint64_t tickets_out = same_in_all_lanes(sys_load(&st->tickets_out));
   uint64_t mirrored = ~0ull;
   uint64_t idle = 0;
   uint32_t reason = 0;
@@ -239,33 +246,45 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
       return lane_value(i % 3 == 0 ? sect.x : i % 3 == 1 ? sect.y : sect.z, src);
     };
 
-    // Sixteen at a stroke.  A submission that fits one ticket becomes that ticket almost unchanged -- the two
-    // records share their layout up to the last sector -- so the four lanes that hold an entry's sectors write
-    // its ticket themselves: the leading run of such entries costs one store instruction, not a pass of the
-    // loop below each (which took about 0.6 us per entry and capped a storm of small requests at 1.6 M/s).
+    // Sixteen at a stroke.  The four lanes that hold an entry's sectors hold nearly all of its tickets' words
+    // already -- the two records share their layout up to the descriptor pointer and the last sector -- so they
+    // write the entry's tickets themselves, ticket i of every entry of the leading run in pass i of one short loop:
+    // sixteen submissions of sixteen tickets cost sixteen store instructions, where a pass of the loop below for
+    // each (it fetches an entry's words from their lanes into scalars first: about half a microsecond) capped a
+    // stream of 1 MiB requests at 2 M/s and a storm of 64 KiB requests at 1.6 M/s.  Taken when the run has some
+    // width: a lone entry of many tickets is written faster by the loop below, sixteen tickets to the instruction.
+    // (Not for a lone entry of more descriptors than a ticket holds, nor for a first entry of more than 32 full
+    // tickets: nothing here would apply to them, and what is worked out per lane first would only add to their
+    // latency.)
     uint32_t consumed = 0;
-    if ((ok_mask & 0xFull) == 0xFull) {  // entry s is there
-      const uint32_t n = bcast(sect.y, lane | 3u);  // payload word 10 sits in .y of sector 3
+    const uint32_t n_first = lane_value(sect.y, 3);
+    if ((ok_mask & 0xFull) == 0xFull &&  // entry s is there
+        (n_first <= kMaxDescsPerTicket || (ready >= 2 && n_first <= kLaneTickets * kFullTicket))) {
+      const uint32_t n = bcast(sect.y, lane | 3u);      // payload word 10 sits in .y of sector 3
+      const uint32_t bytes = bcast(sect.z, lane | 3u);  // payload word 11 sits in .z of sector 3
       const bool all_sectors = ((ok_mask >> (4 * k_of_lane)) & 0xFull) == 0xFull;
-      const bool small = all_sectors && n - 1u < kSmallSubmission;  // 1 .. kSmallSubmission descriptors
-      if ((__ballot(small) & 1ull) != 0) {
-        const uint32_t done_now = bcast(aux, k_of_lane);
-        const uint32_t target_prev = bcast(aux, kPollEntries + k_of_lane);
-        const uint32_t in_flight = static_cast<uint32_t>(s + k_of_lane) - jobs_completed + 1u;
-        const uint32_t bytes = bcast(sect.z, lane | 3u);  // payload word 11 sits in .z of sector 3
-        const uint32_t per_ticket =
-            fixed_per_ticket != 0 ? fixed_per_ticket : ticket_size_for_submission(in_flight, n, bytes, gridDim.x - 1);
-        const bool one_ticket = small && n <= per_ticket && done_now == target_prev;
-        const uint64_t not_fast = ~__ballot(one_ticket);
-        uint32_t run = not_fast == 0 ? kPollEntries : static_cast<uint32_t>(__builtin_ctzll(not_fast)) >> 2;
-        const uint32_t room = kTicketRing - (static_cast<uint32_t>(tickets_out) - tickets_done);
+      const uint32_t done_now = bcast(aux, k_of_lane);
+      const uint32_t target_prev = bcast(aux, kPollEntries + k_of_lane);
+      const uint32_t in_flight = static_cast<uint32_t>(s + k_of_lane) - jobs_completed + 1u;
+      uint32_t per_ticket =
+          fixed_per_ticket != 0 ? fixed_per_ticket : ticket_size_for_submission(in_flight, n, bytes, gridDim.x - 1);
+      if (fixed_per_ticket == 0 && leader_behind && per_ticket < kFullTicket) per_ticket = kFullTicket;  // see below
+      const bool sane = all_sectors && n - 1u < kMaxDescsPerSubmission;  // 1 .. 2^20 descriptors
+      const bool slot_free = done_now == target_prev;  // every ticket ever issued for the job slot has been counted
+      // The ticket ring has room while fewer than its size are outstanding (32-bit wrapping arithmetic).
+      const uint32_t room = kTicketRing - (static_cast<uint32_t>(tickets_out) - tickets_done);
+      const uint32_t sector = lane & 3u;
+      const uint32_t slot = static_cast<uint32_t>(s + k_of_lane) & ring_mask;
+      if (__ballot(sane && n > per_ticket) == 0) {
+        // Every entry that is there fits one ticket (a storm of small requests): the leading run of them becomes
+        // tickets in one store instruction.
+        const uint64_t not_now = ~__ballot(sane && slot_free);
+        uint32_t run = not_now == 0 ? kPollEntries : static_cast<uint32_t>(__builtin_ctzll(not_now)) >> 2;
         run = std::min(run, room);
         if (run != 0) {
           if (k_of_lane < run) {
-            const uint32_t sector = lane & 3u;
             const uint64_t t = tickets_out + k_of_lane;
             const uint32_t stamp = static_cast<uint32_t>(t + 1);
-            const uint32_t slot = static_cast<uint32_t>(s + k_of_lane) & ring_mask;
             const uint32_t target = target_prev + 1u;
             u32x4 v{sect.x, sect.y, sect.z, stamp};
             if (sector == 3) {
@@ -277,6 +296,55 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
           }
           tickets_out += run;
           consumed = run;
+        }
+      } else if (ready >= 2 && n_first <= kLaneTickets * lane_value(per_ticket, 0)) {
+        // Several entries, some of more than one ticket, the first of them not too many.  (The statement keeps the compiler from working this
+        // block's division and lane exchanges out ahead of the branch, where every poll would pay for them.)
+        uint32_t n_here = n, per_here = per_ticket;
+        asm volatile("" : "+v"(n_here), "+v"(per_here));
+        const uint32_t nt = sane ? (n_here + per_here - 1) / per_here : 0u;
+        const bool regular = sane && nt <= kLaneTickets && slot_free;
+        const uint64_t irregular = ~__ballot(regular);
+        const uint32_t run_regular = irregular == 0 ? kPollEntries : static_cast<uint32_t>(__builtin_ctzll(irregular)) >> 2;
+        // Tickets of the entries before this one and up to this one (the four lanes of an entry hold the same values).
+        const uint32_t mine = k_of_lane < run_regular ? nt : 0u;
+        uint32_t upto = mine, most = mine;
+#pragma unroll
+        for (uint32_t d = 4; d < kWaveLanes; d <<= 1) {
+          const uint32_t below = static_cast<uint32_t>(__shfl_up(static_cast<int>(upto), d, kWaveLanes));
+          if (lane >= d) upto += below;
+          most = std::max(most, static_cast<uint32_t>(__shfl_xor(static_cast<int>(most), static_cast<int>(d), kWaveLanes)));
+        }
+        const uint64_t no_room = ~__ballot(k_of_lane < run_regular && upto <= room);
+        const uint32_t run = no_room == 0 ? kPollEntries : static_cast<uint32_t>(__builtin_ctzll(no_room)) >> 2;
+        const uint32_t total = run != 0 ? lane_value(upto, 4 * run - 4) : 0u;
+        // Taken when the run has some width (`most` is over the regular run, which the room may have cut: an upper
+        // bound, good enough for the choice): a lone entry of many tickets is written faster by the loop below.
+        if (run != 0 && total >= 2 * most) {
+          const uint32_t target = target_prev + nt;
+          const uint64_t first_ticket = tickets_out + (upto - mine);
+          const bool takes_part = k_of_lane < run;
+          for (uint32_t i = 0; __ballot(takes_part && i < nt) != 0; ++i) {
+            if (takes_part && i < nt) {
+              const uint64_t t = first_ticket + i;
+              const uint32_t stamp = static_cast<uint32_t>(t + 1);
+              u32x4 v{sect.x, sect.y, sect.z, stamp};
+              if (sector == 1) {  // dst_hi, then where this ticket's descriptors start
+                const uint64_t d = ((static_cast<uint64_t>(sect.z) << 32) | sect.y) +
+                                   static_cast<uint64_t>(i) * per_ticket * sizeof(tcpxuLoadMeta);
+                v.y = static_cast<uint32_t>(d);
+                v.z = static_cast<uint32_t>(d >> 32);
+              }
+              if (sector == 3) {  // val_hi, then the ticket's own words
+                v.y = std::min(per_ticket, n - i * per_ticket) | (slot << 8) | (nt == 1 ? kOnlyTicket : 0u);
+                v.z = target;
+              }
+              store_vec_sys(reinterpret_cast<uint8_t*>(&st->tickets[t & (kTicketRing - 1)]) + 16 * sector, v);
+            }
+          }
+          if (takes_part && sector == 3) sys_store(&job_target[slot], target);
+          tickets_out += static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(total)));
+          consumed = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(run)));
         }
       }
     }

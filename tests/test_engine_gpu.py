@@ -707,3 +707,42 @@ def test_engine_random_mixtures_of_fragment_kinds(pkg, hip, oracle, seed):
     got = g.result()
     assert first_difference(got, expect) is None, "no-alloc: first (index, got, want, count): %r" % (first_difference(got, expect),)
     m.free()
+
+
+@pytest.mark.parametrize("per_ticket", [0, 7, 16])
+def test_engine_many_mid_size_submissions_waiting_at_once(pkg, hip, oracle, per_ticket):
+    """A backlog the leader finds sixteen entries deep at its first look: 300 submissions of 1 to 520 descriptors (one
+    ticket, a few, up to the most the leader's lanes write themselves, and beyond), empty ones in between, queued
+    before the kernel is launched.  Every poll then hands out the tickets of several submissions at once."""
+    from test_unpack_gpu import seeded_pool
+
+    rng = np.random.default_rng(900 + per_ticket)
+    pool = seeded_pool(1 << 20, 901)
+    sizes = [int(x) for x in rng.choice([1, 8, 16, 17, 33, 64, 100, 256, 257, 512, 520, 0], size=300)]
+    rows, dst = [], 5
+    for n in sizes:
+        for _ in range(n):
+            ln = int(rng.integers(1, 1500))
+            rows.append((int(rng.integers(0, 255)) * 4096 + int(rng.integers(0, 4096 - ln + 1)), ln, dst))
+            dst += ln
+    descs = make_descs(rows)
+    expect = oracle_expected(oracle, pool, descs, dst + 64, 0)
+    g = GpuBuffers(pool, descs, dst + 64, 0)
+    m = Mapped(pkg, hip, np.ascontiguousarray(descs), len(sizes))
+    e = Engine(pkg, hip, descs_per_ticket=per_ticket)
+    print("engine backlog case: %d submissions, %d descriptors, tickets of %d" % (len(sizes), len(descs), per_ticket), flush=True)
+    first = 0
+    for i, n in enumerate(sizes):
+        e.submit(g.pool.data_ptr(), g.dst_base, m.desc_dev(first), n, m.flag_dev(i), i + 1)
+        first += n
+    e.start()
+    try:
+        for i in range(len(sizes)):
+            m.wait(i, i + 1)
+    finally:
+        e.stop()
+    assert e.completed() == len(sizes)
+    got = g.result()
+    e.destroy()
+    m.free()
+    assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
