@@ -75,6 +75,19 @@ __host__ __device__ __forceinline__ uint32_t ticket_size_for(uint32_t backlog, u
 // for whole pages: a submission of shorter fragments gets more descriptors per ticket, in multiples of 16 so that
 // the copy wavefronts' shares come out even, up to 64 (full_ticket_size).  Written as comparisons: the leader runs
 // this for every submission and a division costs it forty instructions.
+// ceil(n / per_ticket) for 1 <= n <= 2^20 and 1 <= per_ticket <= 64 without the forty-odd instructions of a general
+// 32-bit division: the quotient estimated in floating point (both operands are exact there) and put right by at most one.
+__host__ __device__ __forceinline__ uint32_t tickets_for(uint32_t n, uint32_t per_ticket) {
+  const uint32_t x = n + per_ticket - 1;
+#if defined(__HIP_DEVICE_COMPILE__)
+  uint32_t q = static_cast<uint32_t>(static_cast<float>(x) * __builtin_amdgcn_rcpf(static_cast<float>(per_ticket)));
+#else
+  uint32_t q = static_cast<uint32_t>(static_cast<float>(x) / static_cast<float>(per_ticket));
+#endif
+  while (q * per_ticket > x) --q;
+  while (x - q * per_ticket >= per_ticket) ++q;
+  return q;
+}
 constexpr uint32_t kManyInFlight = 8, kSmallSubmission = 32;
 constexpr uint32_t kLaneTickets = 32;  // tickets of one submission that the lanes holding its entry still write themselves
 constexpr uint32_t kLeaderBehind = 8;  // entries waiting in one poll from which the leader counts as the bottleneck
@@ -207,6 +220,8 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
   uint64_t s = same_in_all_lanes(sys_load(&st->sub_head));
   uint64_t tickets_out = same_in_all_lanes(sys_load(&st->tickets_out));
   uint64_t mirrored = ~0ull;
+  // Read once: the grid's size comes from the dispatch packet, a scalar load with a wait behind it wherever it is asked.
+  const uint32_t workers = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(gridDim.x - 1)));
   uint64_t idle = 0;
   uint32_t reason = 0;
   // Fixed per-lane roles in the auxiliary load (second load of every poll), so that both loads of a poll are
@@ -267,7 +282,7 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
       const uint32_t target_prev = bcast(aux, kPollEntries + k_of_lane);
       const uint32_t in_flight = static_cast<uint32_t>(s + k_of_lane) - jobs_completed + 1u;
       uint32_t per_ticket =
-          fixed_per_ticket != 0 ? fixed_per_ticket : ticket_size_for_submission(in_flight, n, bytes, gridDim.x - 1);
+          fixed_per_ticket != 0 ? fixed_per_ticket : ticket_size_for_submission(in_flight, n, bytes, workers);
       if (fixed_per_ticket == 0 && leader_behind && per_ticket < kFullTicket) per_ticket = kFullTicket;  // see below
       const bool sane = all_sectors && n - 1u < kMaxDescsPerSubmission;  // 1 .. 2^20 descriptors
       const bool slot_free = done_now == target_prev;  // every ticket ever issued for the job slot has been counted
@@ -302,7 +317,7 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
         // block's division and lane exchanges out ahead of the branch, where every poll would pay for them.)
         uint32_t n_here = n, per_here = per_ticket;
         asm volatile("" : "+v"(n_here), "+v"(per_here));
-        const uint32_t nt = sane ? (n_here + per_here - 1) / per_here : 0u;
+        const uint32_t nt = sane ? tickets_for(n_here, per_here) : 0u;
         const bool regular = sane && nt <= kLaneTickets && slot_free;
         const uint64_t irregular = ~__ballot(regular);
         const uint32_t run_regular = irregular == 0 ? kPollEntries : static_cast<uint32_t>(__builtin_ctzll(irregular)) >> 2;
@@ -366,14 +381,14 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
         const uint32_t in_flight = static_cast<uint32_t>(s + k) - jobs_completed + 1u;
         uint32_t per_ticket = fixed_per_ticket != 0
                                   ? fixed_per_ticket
-                                  : ticket_size_for_submission(in_flight, n, payload_of(fl, 11), gridDim.x - 1);
+                                  : ticket_size_for_submission(in_flight, n, payload_of(fl, 11), workers);
         // Small tickets spread a small backlog over many workgroups, at the price of more tickets to write.  When
         // submissions queue up at the leader, its time per submission is what limits the engine, not the spread:
         // a stream of 1 MiB requests of 256 whole pages, 64 in flight, is served at 1.44 M/s in tickets of 8 (which
         // the backlog alone asks for: the workers empty it as fast as it comes), at 1.96 M/s in tickets of 16, and at
         // 1.64 M/s with this rule, which holds for part of the time.
         if (fixed_per_ticket == 0 && leader_behind && per_ticket < kFullTicket) per_ticket = kFullTicket;
-        const uint32_t nt = (n + per_ticket - 1) / per_ticket;
+        const uint32_t nt = tickets_for(n, per_ticket);
         const uint32_t slot = static_cast<uint32_t>(s + k) & ring_mask;
         const uint32_t done_now = lane_value(aux, k);
         const uint32_t target_prev = lane_value(aux, kPollEntries + k);
@@ -389,17 +404,33 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
         const uint64_t descs = (static_cast<uint64_t>(payload_of(fl, 5)) << 32) | payload_of(fl, 4);
         // Four neighbouring lanes write the four sectors of one ticket, so that one store instruction of the
         // wavefront fills 16 consecutive tickets (1 KiB of whole lines).
+        // What changes from one pass to the next is kept running, per lane, instead of being worked out from the
+        // ticket's index each time (the leader spends three quarters of its time on a stream of 4 MiB requests in
+        // this loop and the lines before it).
         const uint32_t sector = lane & 3u;
-        for (uint32_t i = lane >> 2; i < nt; i += kWaveLanes / 4) {
-          const uint64_t d = descs + static_cast<uint64_t>(i) * per_ticket * sizeof(tcpxuLoadMeta);
-          const uint32_t count = std::min(per_ticket, n - i * per_ticket);
-          const uint64_t t = tickets_out + i;
-          const uint32_t stamp = static_cast<uint32_t>(t + 1);
-          u32x4 v{bounce_lo, bounce_hi, dst_lo, stamp};
-          if (sector == 1) v = u32x4{dst_hi, static_cast<uint32_t>(d), static_cast<uint32_t>(d >> 32), stamp};
-          if (sector == 2) v = u32x4{flag_lo, flag_hi, val_lo, stamp};
-          if (sector == 3) v = u32x4{val_hi, count | (slot << 8) | (nt == 1 ? kOnlyTicket : 0u), target, stamp};
-          store_vec_sys(reinterpret_cast<uint8_t*>(&st->tickets[t & (kTicketRing - 1)]) + 16 * sector, v);
+        const uint32_t first = lane >> 2;
+        constexpr uint32_t kPerPass = kWaveLanes / 4;
+        u32x4 v{bounce_lo, bounce_hi, dst_lo, 0u};  // sector 0
+        if (sector == 1) v = u32x4{dst_hi, 0u, 0u, 0u};
+        if (sector == 2) v = u32x4{flag_lo, flag_hi, val_lo, 0u};
+        if (sector == 3) v = u32x4{val_hi, 0u, target, 0u};
+        const uint32_t tail_bits = (slot << 8) | (nt == 1 ? kOnlyTicket : 0u);
+        uint64_t d = descs + static_cast<uint64_t>(first) * per_ticket * sizeof(tcpxuLoadMeta);
+        const uint64_t d_step = static_cast<uint64_t>(kPerPass) * per_ticket * sizeof(tcpxuLoadMeta);
+        uint32_t left = n - first * per_ticket;  // descriptors from this lane's ticket on (meaningless beyond nt)
+        uint32_t at = static_cast<uint32_t>(tickets_out) + first;  // low word of the ticket number
+        uint8_t* const ring = reinterpret_cast<uint8_t*>(st->tickets) + 16 * sector;
+        for (uint32_t i = first; i < nt; i += kPerPass) {
+          v.w = at + 1u;  // the stamp
+          if (sector == 1) {
+            v.y = static_cast<uint32_t>(d);
+            v.z = static_cast<uint32_t>(d >> 32);
+          }
+          if (sector == 3) v.y = std::min(per_ticket, left) | tail_bits;
+          store_vec_sys(ring + static_cast<size_t>(at & (kTicketRing - 1)) * sizeof(Record), v);
+          d += d_step;
+          left -= kPerPass * per_ticket;
+          at += kPerPass;
         }
         tickets_out += nt;
       }
