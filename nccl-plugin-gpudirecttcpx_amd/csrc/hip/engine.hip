@@ -368,9 +368,9 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
       if (((ok_mask >> (4 * k)) & 0xFull) != 0xFull) break;
       const uint32_t fl = 4 * k;  // first lane of entry k
       const uint32_t n = payload_of(fl, 10);
-      const uint32_t flag_lo = payload_of(fl, 6), flag_hi = payload_of(fl, 7);
-      const uint32_t val_lo = payload_of(fl, 8), val_hi = payload_of(fl, 9);
       if (n == 0) {
+        const uint32_t flag_lo = payload_of(fl, 6), flag_hi = payload_of(fl, 7);
+        const uint32_t val_lo = payload_of(fl, 8), val_hi = payload_of(fl, 9);
         if (lane == 0) {
           sys_store(reinterpret_cast<uint64_t*>((static_cast<uint64_t>(flag_hi) << 32) | flag_lo),
                     (static_cast<uint64_t>(val_hi) << 32) | val_lo);
@@ -399,21 +399,20 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
         if (static_cast<uint32_t>(tickets_out) + nt - tickets_done > kTicketRing) break;
         const uint32_t target = target_prev + nt;
         if (lane == 0) sys_store(&job_target[slot], target);
-        const uint32_t bounce_lo = payload_of(fl, 0), bounce_hi = payload_of(fl, 1);
-        const uint32_t dst_lo = payload_of(fl, 2), dst_hi = payload_of(fl, 3);
-        const uint64_t descs = (static_cast<uint64_t>(payload_of(fl, 5)) << 32) | payload_of(fl, 4);
         // Four neighbouring lanes write the four sectors of one ticket, so that one store instruction of the
-        // wavefront fills 16 consecutive tickets (1 KiB of whole lines).
+        // wavefront fills 16 consecutive tickets (1 KiB of whole lines).  A ticket's sector differs from the entry's
+        // in two places only, so every lane fetches the entry's sector of its own kind from the lane that holds it
+        // (three lane exchanges, where fetching the twelve words one by one into scalars took twelve).
         // What changes from one pass to the next is kept running, per lane, instead of being worked out from the
         // ticket's index each time (the leader spends three quarters of its time on a stream of 4 MiB requests in
         // this loop and the lines before it).
         const uint32_t sector = lane & 3u;
         const uint32_t first = lane >> 2;
         constexpr uint32_t kPerPass = kWaveLanes / 4;
-        u32x4 v{bounce_lo, bounce_hi, dst_lo, 0u};  // sector 0
-        if (sector == 1) v = u32x4{dst_hi, 0u, 0u, 0u};
-        if (sector == 2) v = u32x4{flag_lo, flag_hi, val_lo, 0u};
-        if (sector == 3) v = u32x4{val_hi, 0u, target, 0u};
+        const uint32_t holder = fl + sector;
+        u32x4 v{bcast(sect.x, holder), bcast(sect.y, holder), bcast(sect.z, holder), 0u};
+        const uint64_t descs = (static_cast<uint64_t>(v.z) << 32) | v.y;  // in the lanes of sector 1: dst_hi, descs
+        if (sector == 3) v.z = target;                                     // in the lanes of sector 3: val_hi, n, bytes
         const uint32_t tail_bits = (slot << 8) | (nt == 1 ? kOnlyTicket : 0u);
         uint64_t d = descs + static_cast<uint64_t>(first) * per_ticket * sizeof(tcpxuLoadMeta);
         const uint64_t d_step = static_cast<uint64_t>(kPerPass) * per_ticket * sizeof(tcpxuLoadMeta);
