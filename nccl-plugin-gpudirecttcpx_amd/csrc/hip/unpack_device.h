@@ -77,10 +77,15 @@ __device__ __forceinline__ void store_byte_sys(uint8_t* p, uint8_t v) {
 // starts at B's first full line.  Every line inside a run of fragments is then written whole, by one wavefront.
 // Both owners decide with the same inputs whether the rule applies to a boundary:
 constexpr uint32_t kLineBytes = 128;
-constexpr uint32_t kShareMinLen = 256;  // shorter fragments keep their own partial lines
+// The line must hold nothing but the end of A and the beginning of B -- A reaches back to the line's first byte, B
+// on to its last -- and each of the two must be long enough for a 16-byte load of its own bytes and not be one of
+// the tiny fragments that are copied bytewise.
+__device__ __forceinline__ bool fragment_is_tiny(const uint8_t* dst, uint32_t len);
 __device__ __forceinline__ bool shares_line(uint64_t dst_a, uint32_t len_a, uint64_t dst_b, uint32_t len_b) {
-  return dst_a + len_a == dst_b && len_a >= kShareMinLen && len_b >= kShareMinLen &&
-         ((dst_a + len_a) & (kLineBytes - 1)) != 0;
+  const uint32_t in_line = static_cast<uint32_t>(dst_a + len_a) & (kLineBytes - 1);  // bytes of A in the line
+  return dst_a + len_a == dst_b && in_line != 0 && len_a >= in_line && len_a >= 16u && len_b >= kLineBytes - in_line &&
+         len_b >= 16u && !fragment_is_tiny(reinterpret_cast<const uint8_t*>(dst_a), len_a) &&
+         !fragment_is_tiny(reinterpret_cast<const uint8_t*>(dst_b), len_b);
 }
 
 // 16 bytes starting at byte `shift` (0..16) of the 32 bytes a:b.
@@ -116,7 +121,7 @@ struct CopyRound {
   const uint8_t* src_frag;  // first byte of the fragment
   uint8_t* dst_frag;
   const uint8_t* src_next;  // first byte of the next fragment's source if the last line is shared, else src_frag
-  uint32_t nvec;            // vectors in this round, 1..kVecPerRound
+  uint32_t nvec;            // vectors in this round, 0..kVecPerRound (0: nothing but a shared line or edge bytes)
   uint32_t frag_len;
   uint32_t line_off;        // offset of the shared last line from dst_frag
   bool share_next;          // this round completes the fragment's last line out of the next fragment
@@ -141,7 +146,7 @@ constexpr uint32_t kLineVecs = kLineBytes / 16;  // lanes that take part in the 
 //   the one vector the boundary cuts (none if rem is a multiple of 16) is the last `cut` bytes of A followed by
 //   the first 16 - cut bytes of B: its lane loads A's last 16 bytes and B's first 16 and takes bytes
 //   [16 - cut, 32 - cut) of the two, a shift by a wave-uniform amount.
-// Both neighbours are at least kShareMinLen long, so every one of these loads stays inside its fragment.
+// shares_line has seen to it that every one of these loads stays inside its fragment.
 // (An earlier form gave every lane two loads and a shift of its own, by a per-lane amount: some sixty vector
 // instructions a line instead of some twenty, a sixth of the time of a round of a 2 KiB fragment.)
 struct LinePlan {
@@ -187,7 +192,7 @@ __device__ __forceinline__ void round_load(const CopyRound& c, CopyRegs& x, uint
     const uint32_t v = static_cast<uint32_t>(k) * kWaveLanes + lane;
     if (v < c.nvec) x.r[k] = load_vec_sys(base4 + (v << 4));
   }
-  if (skew != 0) {
+  if (skew != 0 && c.nvec != 0) {
     if (lane == 0) x.tail_dword = load_dword_sys(base4 + (c.nvec << 4));
   }
   if (c.share_next) {
@@ -277,7 +282,7 @@ struct FragmentPlan {
   uint32_t start_off;  // offset of vector 0 from the fragment's first byte
   uint32_t end_off;    // offset of the end of the last vector (where the shared last line starts, if there is one)
   uint32_t head, tail; // edge bytes before vector 0 and after the last vector, each fewer than 16
-  uint32_t nvec;       // vectors in all, at least 1
+  uint32_t nvec;       // vectors in all; none where a short fragment lies in the shared lines of its two neighbours
 };
 __device__ __forceinline__ FragmentPlan plan_fragment(uint64_t dst_addr, uint32_t len, bool share_prev, bool share_next) {
   FragmentPlan p;

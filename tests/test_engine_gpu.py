@@ -632,15 +632,17 @@ def test_engine_alternating_one_byte_whole_page_and_empty_fragments(pkg, hip, or
     m.free()
 
 
+@pytest.mark.parametrize("kind", ["long", "short"])
 @pytest.mark.parametrize("per_ticket", [0, 3, 64])
-def test_engine_every_boundary_position_inside_a_shared_line(pkg, hip, oracle, per_ticket):
-    """Runs of three contiguous fragments with their boundaries at every offset inside a 128-byte line, through the
-    engine (tickets of 3 descriptors hold exactly one run, the adaptive size and 64 cut runs anywhere) and through
-    the entry point that allocates nothing."""
-    from test_unpack_gpu import boundary_runs, seeded_pool
+def test_engine_every_boundary_position_inside_a_shared_line(pkg, hip, oracle, per_ticket, kind):
+    """Runs of three contiguous fragments with their boundaries at every offset inside a 128-byte line ("long"), and
+    runs of short fragments that lie in the lines they share with their neighbours ("short"), through the engine
+    (tickets of 3 descriptors, the adaptive size and 64 cut the runs anywhere) and through the entry point that
+    allocates nothing."""
+    from test_unpack_gpu import boundary_runs, seeded_pool, short_runs
 
     pool = seeded_pool(1 << 20, 31)
-    descs, dst_bytes = boundary_runs(32 + per_ticket)
+    descs, dst_bytes = boundary_runs(32 + per_ticket) if kind == "long" else short_runs(52 + per_ticket)
     expect = oracle_expected(oracle, pool, descs, dst_bytes, 0)
     g = GpuBuffers(pool, descs, dst_bytes, 0)
     m = Mapped(pkg, hip, np.ascontiguousarray(descs), 1)

@@ -351,3 +351,30 @@ def test_random_mixtures_of_fragment_kinds(pkg, hip, oracle, seed):
     pool = seeded_pool(1 << 20, seed)
     descs, dst_bytes = random_mixture(seed)
     run_batch(pkg, hip, oracle, pool, descs, dst_bytes, misalign=seed % 16)
+
+
+def short_runs(seed, pool_bytes=1 << 20):
+    """Runs of short fragments (16 to 300 bytes, in random order) that continue each other in the destination between
+    two longer ones, one run from every offset in a 128-byte line: a short fragment may lie entirely in the lines it
+    shares with its two neighbours, or fill a line together with one of them, or be too short to reach the line's
+    end, in which case three fragments meet in one line and nothing is shared."""
+    rng = np.random.default_rng(seed)
+    lengths = [16, 17, 31, 32, 47, 64, 100, 127, 128, 129, 200, 255, 256, 300]
+    rows, dst = [], 0
+    for start in range(128):
+        dst = (dst + 127) // 128 * 128 + start
+        run = [1000] + [int(x) for x in rng.permutation(lengths)[: int(rng.integers(3, len(lengths) + 1))]] + [1000]
+        for ln in run:
+            page = int(rng.integers(0, pool_bytes // 4096))
+            rows.append((page * 4096 + int(rng.integers(0, 4096 - ln + 1)), ln, dst))
+            dst += ln
+        dst += 1
+    return make_descs(rows), dst + 64
+
+
+def test_short_fragments_in_the_shared_lines_of_their_neighbours(pkg, hip, oracle):
+    pool = seeded_pool(1 << 20, 41)
+    for seed in (42, 43):
+        descs, dst_bytes = short_runs(seed)
+        run_batch(pkg, hip, oracle, pool, descs, dst_bytes)
+        run_batch(pkg, hip, oracle, pool, descs, dst_bytes, misalign=9)
