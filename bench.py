@@ -48,7 +48,7 @@ import __graft_entry__ as graft
 # the hardware counters FETCH_SIZE and WRITE_SIZE of one launch of `bench.py --one-launch --steps 20 --warmup 5`
 # (two rocprofv3 --pmc runs), each scaled by what the same counter reads for the plain copy kernel of known size
 # (`--calibrate-copy 256`); the summary with the counter values is profiles/unpack_engine_kernel_8MiB_chunk_pmc_traffic.txt.
-TRAFFIC_PER_ALGORITHMIC_BYTE = 1.0060
+TRAFFIC_PER_ALGORITHMIC_BYTE = 1.0080
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # Steps in the untimed launch that precedes the measured one, and the least steps the windows of the measured launch
 # add up to (60 ms each way): the rate the engine sustains shows only after some milliseconds of load.

@@ -132,9 +132,27 @@ constexpr int kPayloadWords = 12;
 __host__ __device__ constexpr int payload_slot(int i) { return (i / 3) * 4 + (i % 3); }
 // Submission payload: 0-1 bounce, 2-3 dst, 4-5 descs, 6-7 done_flag, 8-9 done_value, 10 n_descs, 11 payload bytes
 //                     (0 = not given).
-// Ticket payload:     0-1 bounce, 2-3 dst, 4-5 descs, 6-7 done_flag, 8-9 done_value, 10 n | job << 8 | only << 31,
-//                     11 target.  `only`: the submission's only ticket (the job slot index is below 2^16).
+// Ticket payload:     0-1 bounce, 2-3 dst, 4-5 descs, 6-7 done_flag, 8-9 done_value,
+//                     10 n | job << 8 | before << 29 | after << 30 | only << 31, 11 target.
+// `only`: the submission's only ticket (the job slot index is below 2^16); `before` / `after`: the submission has
+// descriptors before this ticket's first / after its last (in the same array: the fetcher looks at the nearest one
+// to decide whether the destination line at that end of the ticket is shared with the neighbouring ticket).
 constexpr uint32_t kOnlyTicket = 1u << 31;
+constexpr uint32_t kMoreAfter = 1u << 30, kMoreBefore = 1u << 29;
+__host__ __device__ __forceinline__ uint32_t neighbour_bits(uint32_t i, uint32_t nt, bool across) {
+  return (nt == 1 ? kOnlyTicket : 0u) | (across && i != 0 ? kMoreBefore : 0u) | (across && i + 1 < nt ? kMoreAfter : 0u);
+}
+// Whether a submission's tickets share destination lines across their ends.  It saves two partial writes of a line
+// per ticket boundary and costs every ticket's pick-up two more descriptors to read and look at: worth it when the
+// engine is busy (8 MiB workload +0.3 points of the roofline, fragments of 1.8 KiB +0.4), not for a request that is
+// alone (4 MiB: 0.3 us more), and pointless where whole pages land on line boundaries anyway (1 MiB requests of
+// whole pages: 0.90 -> 0.84 of the roofline with it).  Decided by the leader for the whole submission, so that the
+// two tickets at a boundary always agree.
+__host__ __device__ __forceinline__ bool shares_across_tickets(uint32_t in_flight, uint32_t n, uint32_t bytes,
+                                                               uint32_t dst_lo) {
+  const bool whole_pages_on_lines = bytes == n * TCPXU_PAGE_SIZE && (dst_lo & 127u) == 0;
+  return in_flight >= kManyInFlight && !whole_pages_on_lines;
+}
 
 struct HostCtl {  // mapped host memory
   alignas(64) uint64_t tail;       // host -> GPU: submissions published so far
@@ -337,6 +355,7 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
         // bound, good enough for the choice): a lone entry of many tickets is written faster by the loop below.
         if (run != 0 && total >= 2 * most) {
           const uint32_t target = target_prev + nt;
+          const bool across = shares_across_tickets(in_flight, n, bytes, bcast(sect.z, lane & ~3u));  // dst_lo: .z of sector 0
           const uint64_t first_ticket = tickets_out + (upto - mine);
           const bool takes_part = k_of_lane < run;
           for (uint32_t i = 0; __ballot(takes_part && i < nt) != 0; ++i) {
@@ -351,7 +370,7 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
                 v.z = static_cast<uint32_t>(d >> 32);
               }
               if (sector == 3) {  // val_hi, then the ticket's own words
-                v.y = std::min(per_ticket, n - i * per_ticket) | (slot << 8) | (nt == 1 ? kOnlyTicket : 0u);
+                v.y = std::min(per_ticket, n - i * per_ticket) | (slot << 8) | neighbour_bits(i, nt, across);
                 v.z = target;
               }
               store_vec_sys(reinterpret_cast<uint8_t*>(&st->tickets[t & (kTicketRing - 1)]) + 16 * sector, v);
@@ -409,23 +428,30 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
         const uint32_t sector = lane & 3u;
         const uint32_t first = lane >> 2;
         constexpr uint32_t kPerPass = kWaveLanes / 4;
+        // (asked in this order: a request that is alone pays for nothing but the first comparison)
+        const bool across = in_flight >= kManyInFlight && shares_across_tickets(in_flight, n, payload_of(fl, 11), payload_of(fl, 2));
         const uint32_t holder = fl + sector;
         u32x4 v{bcast(sect.x, holder), bcast(sect.y, holder), bcast(sect.z, holder), 0u};
         const uint64_t descs = (static_cast<uint64_t>(v.z) << 32) | v.y;  // in the lanes of sector 1: dst_hi, descs
         if (sector == 3) v.z = target;                                     // in the lanes of sector 3: val_hi, n, bytes
-        const uint32_t tail_bits = (slot << 8) | (nt == 1 ? kOnlyTicket : 0u);
         uint64_t d = descs + static_cast<uint64_t>(first) * per_ticket * sizeof(tcpxuLoadMeta);
         const uint64_t d_step = static_cast<uint64_t>(kPerPass) * per_ticket * sizeof(tcpxuLoadMeta);
         uint32_t left = n - first * per_ticket;  // descriptors from this lane's ticket on (meaningless beyond nt)
         uint32_t at = static_cast<uint32_t>(tickets_out) + first;  // low word of the ticket number
         uint8_t* const ring = reinterpret_cast<uint8_t*>(st->tickets) + 16 * sector;
+        // The ticket's own word: count | job slot | whether the submission has tickets before and after this one
+        // (the last ticket is the one that takes all that is left).
+        const uint32_t across_bits = across ? kMoreBefore | kMoreAfter : 0u;
+        const uint32_t fixed_bits = (slot << 8) | (nt == 1 ? kOnlyTicket : 0u), after_bit = across_bits & kMoreAfter;
+        uint32_t before_bit = first != 0 ? across_bits & kMoreBefore : 0u;
         for (uint32_t i = first; i < nt; i += kPerPass) {
           v.w = at + 1u;  // the stamp
           if (sector == 1) {
             v.y = static_cast<uint32_t>(d);
             v.z = static_cast<uint32_t>(d >> 32);
           }
-          if (sector == 3) v.y = std::min(per_ticket, left) | tail_bits;
+          if (sector == 3) v.y = std::min(per_ticket, left) | fixed_bits | (left > per_ticket ? after_bit : 0u) | before_bit;
+          before_bit = across_bits & kMoreBefore;  // every ticket but the submission's first
           store_vec_sys(ring + static_cast<size_t>(at & (kTicketRing - 1)) * sizeof(Record), v);
           d += d_step;
           left -= kPerPass * per_ticket;
@@ -553,25 +579,48 @@ __device__ uint32_t try_fetch_ticket(State* st, const uint32_t* stop_word, uint6
     return (static_cast<uint64_t>(bcast(word, payload_slot(lo + 1))) << 32) | bcast(word, payload_slot(lo));
   };
   const uint64_t bounce = word64(0), dst = word64(2), descs_addr = word64(4);
-  const uint32_t n = bcast(word, payload_slot(10)) & 0xFFu;
+  const uint32_t ticket_bits = bcast(word, payload_slot(10));
+  const uint32_t n = ticket_bits & 0xFFu;
   // One 16-byte descriptor per lane straight from where the submission keeps them (system scope: never a cached
   // copy); lanes past the end repeat the last one and write no record.
   const uint32_t mine = lane < n ? lane : (n != 0 ? n - 1u : 0u);  // a ticket has at least one descriptor
   const u32x4 d = load_vec_sys(reinterpret_cast<const uint8_t*>(descs_addr) + 16 * mine);
   const uint32_t so = d[0], len = d[1];
   const uint64_t doff = (static_cast<uint64_t>(d[3]) << 32) | d[2];
+  // The descriptor before the ticket's first and the one after its last, where the submission has them (lanes 0
+  // and 1, in the same round trip): the neighbouring tickets' fetchers look at the same pairs from the other side.
+  const bool more_before = (ticket_bits & kMoreBefore) != 0, more_after = (ticket_bits & kMoreAfter) != 0;
+  uint32_t before_len = 0, before_dlo = 0, before_dhi = 0, after_so = 0, after_len = 0, after_dlo = 0, after_dhi = 0;
+  if (more_before || more_after) {  // wave-uniform: a ticket without such neighbours pays nothing here
+    u32x4 outer = {0u, 0u, 0u, 0u};
+    if ((lane == 0 && more_before) || (lane == 1 && more_after)) {
+      const uint64_t at = lane == 0 ? descs_addr - sizeof(tcpxuLoadMeta) : descs_addr + sizeof(tcpxuLoadMeta) * n;
+      outer = load_vec_sys(reinterpret_cast<const uint8_t*>(at));
+    }
+    auto from_lane = [](uint32_t v, int src) { return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), src)); };
+    before_len = from_lane(outer[1], 0), before_dlo = from_lane(outer[2], 0), before_dhi = from_lane(outer[3], 0);
+    after_so = from_lane(outer[0], 1), after_len = from_lane(outer[1], 1);
+    after_dlo = from_lane(outer[2], 1), after_dhi = from_lane(outer[3], 1);
+  }
   // The neighbours' descriptors decide which destination lines are shared with them.  A fragment's neighbours are
   // the nearest descriptors of the ticket that are not empty: an empty descriptor between two fragments (a
   // zero-length control message's, a fragment cut to nothing) leaves them back to back in the destination.
   const uint64_t live = __ballot(lane < n && len != 0);
   const uint64_t below = live & ((1ull << lane) - 1ull);
   const uint64_t above = lane < 63u ? live & ~((2ull << lane) - 1ull) : 0ull;
-  const bool has_prev = below != 0, has_next = above != 0;
-  const uint32_t prev_lane = has_prev ? 63u - static_cast<uint32_t>(__builtin_clzll(below)) : lane;
-  const uint32_t next_lane = has_next ? static_cast<uint32_t>(__builtin_ctzll(above)) : lane;
-  const uint32_t p_len = lane_shift(len, prev_lane), p_dlo = lane_shift(d[2], prev_lane), p_dhi = lane_shift(d[3], prev_lane);
-  const uint32_t q_len = lane_shift(len, next_lane), q_dlo = lane_shift(d[2], next_lane), q_dhi = lane_shift(d[3], next_lane);
-  const uint32_t q_so = lane_shift(so, next_lane);
+  const bool prev_inside = below != 0, next_inside = above != 0;
+  // Across a ticket's ends only the very first and the very last descriptor have a neighbour, and only one that
+  // is not empty: that is the pair the other ticket sees too.
+  const bool prev_outside = !prev_inside && lane == 0 && before_len != 0;
+  const bool next_outside = !next_inside && lane + 1 == n && after_len != 0;
+  const bool has_prev = prev_inside || prev_outside, has_next = next_inside || next_outside;
+  const uint32_t prev_lane = prev_inside ? 63u - static_cast<uint32_t>(__builtin_clzll(below)) : lane;
+  const uint32_t next_lane = next_inside ? static_cast<uint32_t>(__builtin_ctzll(above)) : lane;
+  uint32_t p_len = lane_shift(len, prev_lane), p_dlo = lane_shift(d[2], prev_lane), p_dhi = lane_shift(d[3], prev_lane);
+  uint32_t q_len = lane_shift(len, next_lane), q_dlo = lane_shift(d[2], next_lane), q_dhi = lane_shift(d[3], next_lane);
+  uint32_t q_so = lane_shift(so, next_lane);
+  if (prev_outside) p_len = before_len, p_dlo = before_dlo, p_dhi = before_dhi;
+  if (next_outside) q_len = after_len, q_dlo = after_dlo, q_dhi = after_dhi, q_so = after_so;
   const uint64_t fdst = dst + doff, fsrc = bounce + so;
   const uint64_t p_dst = dst + ((static_cast<uint64_t>(p_dhi) << 32) | p_dlo);
   const uint64_t q_dst = dst + ((static_cast<uint64_t>(q_dhi) << 32) | q_dlo);
@@ -607,7 +656,7 @@ __device__ uint32_t try_fetch_ticket(State* st, const uint32_t* stop_word, uint6
 template <typename State>
 __device__ void retire_ticket(State* st, uint32_t* jobs_done, const Stage* stage, uint32_t lane) {
   if (lane == 0) {
-    const uint32_t job = (stage->payload[10] & ~kOnlyTicket) >> 8;
+    const uint32_t job = (stage->payload[10] >> 8) & 0xFFFFu;
     const uint32_t target = stage->payload[11];
     const uint64_t done_flag = (static_cast<uint64_t>(stage->payload[7]) << 32) | stage->payload[6];
     const uint64_t done_value = (static_cast<uint64_t>(stage->payload[9]) << 32) | stage->payload[8];
@@ -853,7 +902,7 @@ __global__ __launch_bounds__(kOneShotTickets) void oneshot_prepare_kernel(OneSho
       static_cast<uint32_t>(bounce),    static_cast<uint32_t>(bounce >> 32),    static_cast<uint32_t>(dst),
       static_cast<uint32_t>(dst >> 32), static_cast<uint32_t>(d),               static_cast<uint32_t>(d >> 32),
       static_cast<uint32_t>(done_flag), static_cast<uint32_t>(done_flag >> 32), static_cast<uint32_t>(done_value),
-      static_cast<uint32_t>(done_value >> 32), count | (nt == 1 ? kOnlyTicket : 0u) /* job slot 0 */, nt};
+      static_cast<uint32_t>(done_value >> 32), count | neighbour_bits(t, nt, true) /* job slot 0 */, nt};
   const uint32_t stamp = t + 1u;
   uint8_t* rec = reinterpret_cast<uint8_t*>(&st->tickets[t]);
 #pragma unroll
