@@ -748,3 +748,38 @@ def test_engine_many_mid_size_submissions_waiting_at_once(pkg, hip, oracle, per_
     e.destroy()
     m.free()
     assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
+
+
+@pytest.mark.parametrize("per_ticket", [0, 5, 16])
+def test_engine_lines_shared_across_the_ends_of_tickets(pkg, hip, oracle, per_ticket):
+    """With eight or more submissions in flight the tickets of a submission share destination lines across their
+    ends: runs of fragments with boundaries at every offset inside a line, and runs of short fragments, in slots of
+    37 descriptors all submitted at once, so that ticket ends fall anywhere in the runs and most slots are handed out
+    while many are in flight (the first few are not, and keep their ends to themselves)."""
+    from test_unpack_gpu import boundary_runs, seeded_pool, short_runs
+
+    pool = seeded_pool(1 << 20, 61)
+    a, a_bytes = boundary_runs(62 + per_ticket)
+    b, b_bytes = short_runs(63 + per_ticket)
+    b = b.copy()
+    b["dst_off"] += a_bytes
+    descs = np.concatenate([a, b])
+    dst_bytes = a_bytes + b_bytes
+    expect = oracle_expected(oracle, pool, descs, dst_bytes, 0)
+    g = GpuBuffers(pool, descs, dst_bytes, 0)
+    slots = [(f, min(37, len(descs) - f)) for f in range(0, len(descs), 37)]
+    m = Mapped(pkg, hip, np.ascontiguousarray(descs), len(slots))
+    e = Engine(pkg, hip, descs_per_ticket=per_ticket)
+    print("engine ticket-ends case: %d descriptors, %d slots, tickets of %d" % (len(descs), len(slots), per_ticket), flush=True)
+    for i, (first, n) in enumerate(slots):  # queued before the kernel starts: all in flight together
+        e.submit(g.pool.data_ptr(), g.dst_base, m.desc_dev(first), n, m.flag_dev(i), i + 1)
+    e.start()
+    try:
+        for i in range(len(slots)):
+            m.wait(i, i + 1)
+    finally:
+        e.stop()
+    got = g.result()
+    e.destroy()
+    m.free()
+    assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
