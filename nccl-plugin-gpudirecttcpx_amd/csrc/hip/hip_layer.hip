@@ -48,7 +48,10 @@ __global__ __launch_bounds__(kBatchThreads) void unpack_batch_kernel(const uint8
                                                                    const tcpxuLoadMeta* __restrict__ descs,
                                                                    uint64_t n_descs, uint32_t descs_per_wg,
                                                                    uint64_t n_batches) {
-  __shared__ tcpxuLoadMeta staged[2][kMaxDescsPerWg];
+  // A stage holds the batch at [1, cnt] and, around it, the last descriptor of the batch before and the first of the
+  // batch after (where the list has them): the fragments at the two ends of a batch share destination lines with
+  // them like any other neighbours, and the workgroup that copies the neighbouring batch sees the same pairs.
+  __shared__ tcpxuLoadMeta staged[2][kMaxDescsPerWg + 2];
   const uint32_t tid = threadIdx.x;
   const uint32_t lane = tid & (kWaveLanes - 1);
   const uint32_t wave = tid / kWaveLanes;
@@ -62,21 +65,25 @@ __global__ __launch_bounds__(kBatchThreads) void unpack_batch_kernel(const uint8
     *first = batch * descs_per_wg;
     return static_cast<uint32_t>(std::min<uint64_t>(descs_per_wg, n_descs - *first));
   };
-  auto fetch = [&](uint64_t first, uint32_t cnt) -> u32x4 {
-    return tid < cnt ? *reinterpret_cast<const u32x4*>(descs + first + tid) : u32x4{0, 0, 0, 0};
+  auto fetch = [&](uint64_t first, uint32_t cnt) -> u32x4 {  // thread t: descriptor first - 1 + t
+    const uint64_t one_past = first + tid;
+    const bool there = cnt != 0 && tid < cnt + 2 && one_past >= 1 && one_past <= n_descs;
+    return there ? *reinterpret_cast<const u32x4*>(descs + one_past - 1) : u32x4{0, 0, 0, 0};
   };
 
   uint64_t wg = blockIdx.x, first = 0;
   uint32_t cnt = batch_of(wg, &first);
   u32x4 raw = fetch(first, cnt);
   for (uint32_t stage = 0; wg < n_slots; stage ^= 1u) {
-    if (tid < cnt) *reinterpret_cast<u32x4*>(&staged[stage][tid]) = raw;
+    if (tid < cnt + 2) *reinterpret_cast<u32x4*>(&staged[stage][tid]) = raw;
     const uint32_t cnt_now = cnt;
+    const bool has_before = first > 0, has_after = first + cnt < n_descs;
     wg += gridDim.x;
     cnt = batch_of(wg, &first);
     raw = fetch(first, cnt);  // in flight while this batch is copied
     __syncthreads();          // the stage is complete; every wavefront has left the stage written two batches ago
-    wave_copy_descriptors(staged[stage], cnt_now, wave, kBatchWaves, cnt_now, bounce, dst, lane, [] {});
+    wave_copy_descriptors(staged[stage] + 1, cnt_now, wave, kBatchWaves, cnt_now, bounce, dst, lane, [] {}, has_before,
+                          has_after);
   }
 }
 

@@ -356,9 +356,13 @@ struct FragmentRounds {
 // a list of n.  Neighbours in the list (whoever copies them) decide which destination lines are shared.
 // Everything that describes a fragment is wave-uniform; saying so keeps it in scalar registers and leaves the
 // vector registers to the payload in flight.  `bounce` and `dst` must be wave-uniform.
+// `before` / `after`: the list has a valid descriptor at index -1 / at index n (the last of the batch before, the
+// first of the batch after, staged with it), which the first and the last fragment of the list may share a line with:
+// the wavefront that copies the neighbouring batch looks at the same pair from the other side.
 struct ShareCursor {
   const tcpxuLoadMeta* descs;
   uint32_t n, j, end, stride;
+  bool before, after;
   const uint8_t* bounce;
   uint8_t* dst;
   FragmentRounds fr;
@@ -370,9 +374,12 @@ struct ShareCursor {
     return (static_cast<uint64_t>(uniform(static_cast<uint32_t>(v >> 32))) << 32) | uniform(static_cast<uint32_t>(v));
   }
   __device__ __forceinline__ void open(const tcpxuLoadMeta* list, uint32_t count, uint32_t first, uint32_t step,
-                                       uint32_t stop, const uint8_t* bounce_base, uint8_t* dst_base) {
+                                       uint32_t stop, const uint8_t* bounce_base, uint8_t* dst_base,
+                                       bool has_before, bool has_after) {
     descs = list;
     n = count;
+    before = has_before;
+    after = has_after;
     j = uniform(first);
     end = uniform(stop);
     stride = step;
@@ -407,11 +414,11 @@ struct ShareCursor {
       }
       bool share_prev = false, share_next = false;
       const uint8_t* src_next = fsrc;
-      if (cur > 0) {
-        const tcpxuLoadMeta p = descs[cur - 1];
+      if (cur > 0 || before) {
+        const tcpxuLoadMeta p = descs[static_cast<int32_t>(cur) - 1];
         share_prev = shares_line(dst_addr + uniform64(p.dst_off), uniform(p.len), dst_addr + doff, len);
       }
-      if (cur + 1 < n) {
+      if (cur + 1 < n || after) {
         const tcpxuLoadMeta q = descs[cur + 1];
         share_next = shares_line(dst_addr + doff, len, dst_addr + uniform64(q.dst_off), uniform(q.len));
         if (share_next) src_next = bounce + uniform(q.src_off);
@@ -431,9 +438,10 @@ template <typename OnLastFragment>
 __device__ __forceinline__ void wave_copy_descriptors(const tcpxuLoadMeta* descs, uint32_t n, uint32_t first,
                                                       uint32_t stride, uint32_t end, const uint8_t* bounce,
                                                       uint8_t* dst, uint32_t lane,
-                                                      OnLastFragment&& on_last_fragment) {
+                                                      OnLastFragment&& on_last_fragment, bool has_before = false,
+                                                      bool has_after = false) {
   ShareCursor cursor;
-  cursor.open(descs, n, first, stride, end, bounce, dst);
+  cursor.open(descs, n, first, stride, end, bounce, dst, has_before, has_after);
   if (cursor.j >= cursor.end) on_last_fragment();
   auto on_take = [&] {
     if (cursor.j >= cursor.end) on_last_fragment();
