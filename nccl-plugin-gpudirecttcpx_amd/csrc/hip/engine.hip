@@ -3,13 +3,16 @@
 //
 // Roles inside the one kernel launch
 //   workgroup 0, wavefront 0  "leader": polls the submission ring over PCIe (sixteen entries per round trip),
-//                             cuts each submission into tickets of 8 to 16 consecutive descriptors (by backlog,
-//                             or of the fixed `descs_per_ticket`) and writes them into a device-memory ticket
-//                             ring.  It never copies payload.
+//                             cuts each submission into tickets of 8 to 16 consecutive descriptors (by backlog;
+//                             up to 64 where the payload says the fragments are short; or of the fixed
+//                             `descs_per_ticket`) and writes them into a device-memory ticket ring: several
+//                             waiting submissions at once where it can.  It never copies payload.
 //   every other workgroup     "worker": one fetcher wavefront claims the next ticket number with one atomic,
 //                             polls that ticket's slot until its stamps match, reads the ticket's descriptors
 //                             (one per lane) and leaves in LDS, per fragment, a record of what the copy needs
-//                             to know about it; the copy wavefronts copy the fragments from those records,
+//                             to know about it (which destination lines it shares with its neighbours, in
+//                             the ticket and, when the engine is busy, in the tickets before and after);
+//                             the copy wavefronts copy the fragments from those records,
 //                             and the last of them to finish counts the ticket done.  Whoever counts the last
 //                             ticket of a submission writes the completion word that the host poller reads.
 //
