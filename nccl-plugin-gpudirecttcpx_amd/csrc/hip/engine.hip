@@ -68,16 +68,6 @@ constexpr uint32_t kMaxDescsPerTicket = 64;
 __host__ __device__ __forceinline__ uint32_t ticket_size_for(uint32_t backlog, uint32_t workers) {
   return backlog < 13u * workers ? 8u : backlog < 18u * workers ? 12u : 16u;
 }
-// Ticket size for one submission of n descriptors when `in_flight` submissions (this one included) are not yet
-// completed; each is taken to be as long as this one.  A small submission among many stays whole: with 8 or
-// more in flight the parallelism is in the submissions, and a submission that is one ticket costs the leader
-// one store instead of a pass of its loop.  (64 KiB requests of 16 fragments, p50 publish -> done: 8.7 -> 9.1 us
-// at 8 in flight, 17.5 -> 9.3 us at 32, where the leader's loop had become the queue.)
-//
-// `bytes` is the submission's payload if the caller said (0 = unknown: whole pages).  The largest step, 16, stands
-// for whole pages: a submission of shorter fragments gets more descriptors per ticket, in multiples of 16 so that
-// the copy wavefronts' shares come out even, up to 64 (full_ticket_size).  Written as comparisons: the leader runs
-// this for every submission and a division costs it forty instructions.
 // ceil(n / per_ticket) for 1 <= n <= 2^20 and 1 <= per_ticket <= 64 without the forty-odd instructions of a general
 // 32-bit division: the quotient estimated in floating point (both operands are exact there) and put right by at most one.
 __host__ __device__ __forceinline__ uint32_t tickets_for(uint32_t n, uint32_t per_ticket) {
@@ -91,6 +81,16 @@ __host__ __device__ __forceinline__ uint32_t tickets_for(uint32_t n, uint32_t pe
   while (x - q * per_ticket >= per_ticket) ++q;
   return q;
 }
+// Ticket size for one submission of n descriptors when `in_flight` submissions (this one included) are not yet
+// completed; each is taken to be as long as this one.  A small submission among many stays whole: with 8 or
+// more in flight the parallelism is in the submissions, and a submission that is one ticket costs the leader
+// one store instead of a pass of its loop.  (64 KiB requests of 16 fragments, p50 publish -> done: 8.7 -> 9.1 us
+// at 8 in flight, 17.5 -> 9.3 us at 32, where the leader's loop had become the queue.)
+//
+// `bytes` is the submission's payload if the caller said (0 = unknown: whole pages).  The largest step, 16, stands
+// for whole pages: a submission of shorter fragments gets more descriptors per ticket, in multiples of 16 so that
+// the copy wavefronts' shares come out even, up to 64 (full_ticket_size).  Written as comparisons: the leader runs
+// this for every submission and a division costs it forty instructions.
 constexpr uint32_t kManyInFlight = 8, kSmallSubmission = 32;
 constexpr uint32_t kLaneTickets = 32;  // tickets of one submission that the lanes holding its entry still write themselves
 constexpr uint32_t kLeaderBehind = 8;  // entries waiting in one poll from which the leader counts as the bottleneck
@@ -334,8 +334,9 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
           consumed = run;
         }
       } else if (ready >= 2 && n_first <= kLaneTickets * lane_value(per_ticket, 0)) {
-        // Several entries, some of more than one ticket, the first of them not too many.  (The statement keeps the compiler from working this
-        // block's division and lane exchanges out ahead of the branch, where every poll would pay for them.)
+        // Several entries, some of more than one ticket, the first of them not too many.  (The empty statement keeps
+        // the compiler from working this block's division and lane exchanges out ahead of the branch, where every
+        // poll would pay for them.)
         uint32_t n_here = n, per_here = per_ticket;
         asm volatile("" : "+v"(n_here), "+v"(per_here));
         const uint32_t nt = sane ? tickets_for(n_here, per_here) : 0u;
