@@ -571,9 +571,23 @@ def main():
         read_gbps = 2 * n_copy / us.value / 1e3
         pkg.check(benchlib.tcpxuCopyKernelTimed(dev, scratch.data_ptr(), None, 2 * n_copy, 3, 20, ctypes.byref(us)), "fill timed")
         write_gbps = 2 * n_copy / us.value / 1e3
+        # The runtime's own device-to-device copy of the same gigabyte (torch's copy_ of a contiguous tensor is one
+        # hipMemcpyDtoDAsync), timed with events on torch's stream.
+        lo, hi = scratch[:n_copy], scratch[n_copy:]
+        for _ in range(3):
+            hi.copy_(lo)
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for _ in range(20):
+            hi.copy_(lo)
+        ev1.record()
+        ev1.synchronize()
+        runtime_copy_gbps = 2 * n_copy * 20 / (ev0.elapsed_time(ev1) * 1e-3) / 1e9
+        del lo, hi
         result["hbm_yardsticks"] = {
             "read_only_GBps": round(read_gbps, 1),
             "write_only_GBps": round(write_gbps, 1),
+            "runtime_device_to_device_copy_rw_GBps": round(runtime_copy_gbps, 1),
             "copy_bound_rw_GBps": round(2.0 / (1.0 / read_gbps + 1.0 / write_gbps), 1),
             "note": "plain kernels over 2 GiB with the unpack kernel's load and store instructions; copy_bound is what a "
             "plain copy made of these two halves comes to (1/read + 1/write per byte), against the roofline's 8000 GB/s",
