@@ -78,25 +78,32 @@ def cpu_baseline(oracle, descs, dst_bytes, pool, threads, budget_s):
     return payload / med / 1e9, iters
 
 
-def plugin_path(pkg, hip, torch, workloads, pool, helper_thread=False):
+def plugin_path(pkg, hip, torch, workloads, pool, helper_thread=False, rx_bindings=None):
     """The same chunks through the whole plugin (libnccl-net.so): irecv -> control messages -> synthetic recvmsg
     with its control messages -> descriptor builder -> slot -> engine -> test() -> iflush -> irecvConsumed, driven by
     the request loop inside the library.  The host builds one descriptor per fragment here, so this is a host-bound
     figure: what the receive path costs per fragment on one proxy thread (or, with `helper_thread`, on the proxy
-    thread plus the plugin's socket thread, NCCL_GPUDIRECTTCPX_AMD_HELPER_THREAD=1)."""
+    thread plus the plugin's socket thread, NCCL_GPUDIRECTTCPX_AMD_HELPER_THREAD=1, which `rx_bindings` binds to
+    CPUs: the value of NCCL_GPUDIRECTTCPX_RX_BINDINGS)."""
     from nccl_plugin_gpudirecttcpx_amd import synth_driver
 
     lib = pkg.plugin_lib()
-    saved = os.environ.get("NCCL_GPUDIRECTTCPX_AMD_HELPER_THREAD")
-    os.environ["NCCL_GPUDIRECTTCPX_AMD_HELPER_THREAD"] = "1" if helper_thread else "0"
+    flags = {"NCCL_GPUDIRECTTCPX_AMD_HELPER_THREAD": "1" if helper_thread else "0", "NCCL_GPUDIRECTTCPX_RX_BINDINGS": rx_bindings}
+    saved = {k: os.environ.get(k) for k in flags}
+    for k, v in flags.items():
+        if v is None:
+            os.environ.pop(k, None)
+        else:
+            os.environ[k] = v
     try:
         if lib.tcpxInit(None) != 0:
             return {"error": "tcpxInit failed"}
     finally:
-        if saved is None:
-            os.environ.pop("NCCL_GPUDIRECTTCPX_AMD_HELPER_THREAD", None)
-        else:
-            os.environ["NCCL_GPUDIRECTTCPX_AMD_HELPER_THREAD"] = saved
+        for k, v in saved.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
     base = ctypes.c_void_p()
     assert lib.tcpxSynthArenaCreate(0, pool.nbytes, ctypes.byref(base)) == 0
     pkg.check(hip.tcpxuCopyToDevice(0, base, pool.ctypes.data, pool.nbytes), "tcpxuCopyToDevice")
@@ -601,12 +608,32 @@ def main():
 
     if not args.skip_extras and not args.one_launch:
         result["plugin_path"] = plugin_path(pkg, hip, torch, workloads[: min(8, args.chunks)], pool)
-        # Two threads that hand every fragment run to each other: the figure depends on where the machine puts them
-        # (on the virtual CPUs of the test boxes it comes out near 46 GB/s in most runs and near 11 GB/s in some,
-        # with nothing else different), so the leg runs three times and reports the median beside all three.
-        legs = [plugin_path(pkg, hip, torch, workloads[: min(8, args.chunks)], pool, helper_thread=True) for _ in range(3)]
+        # Two threads that hand every task to each other through the task rings, and in this workload (four flows
+        # interleaved fragment by fragment) every fragment is a chunk of its own, hence a task: the leg costs about one
+        # cache line there and back per fragment, and that depends on where the machine puts the two threads (the
+        # virtual CPUs of the test boxes lie 60-85 ns apart in some pairs and 400-750 ns in others, and the leg comes
+        # out near 46-57 GB/s or near 11 GB/s accordingly).  So it runs three times as the machine places the threads,
+        # median beside all three, and once each with the proxy thread on one CPU and the socket thread bound
+        # (NCCL_GPUDIRECTTCPX_RX_BINDINGS, the reference's flag for this) to the CPU nearest to it and farthest from it.
+        some = workloads[: min(8, args.chunks)]
+        legs = [plugin_path(pkg, hip, torch, some, pool, helper_thread=True) for _ in range(3)]
         legs.sort(key=lambda leg: leg.get("payload_GBps", 0.0))
         result["plugin_path"]["with_socket_thread"] = dict(legs[1], payload_GBps_of_three_runs=[leg.get("payload_GBps") for leg in legs])
+        cpus = sorted(os.sched_getaffinity(0))
+        if len(cpus) >= 2:
+            synth, ns, apart = pkg.synth_lib(), ctypes.c_double(), {}
+            for other in cpus[1:]:
+                if synth.tcpxSynthCpuRoundTripNs(cpus[0], other, 5000, ctypes.byref(ns)) == 0:
+                    apart[other] = ns.value
+            bound = {}
+            try:
+                os.sched_setaffinity(0, [cpus[0]])  # this thread is the proxy thread
+                for which, other in (("nearest", min(apart, key=apart.get)), ("farthest", max(apart, key=apart.get))) if apart else ():
+                    leg = plugin_path(pkg, hip, torch, some, pool, helper_thread=True, rx_bindings="tcpx-amd-synth0:%d-%d" % (other, other))
+                    bound[which] = {"cpus": [cpus[0], other], "cache_line_round_trip_ns": round(apart[other]), "payload_GBps": leg.get("payload_GBps"), "host_ns_per_fragment": leg.get("host_ns_per_fragment")}
+            finally:
+                os.sched_setaffinity(0, cpus)
+            result["plugin_path"]["with_socket_thread"]["socket_thread_bound_to_the_cpu"] = bound
 
     # ---- CPU baseline on this machine's host cores: rank 0, bounded sample ---------------------------------
     # Threads: the cores this process may run on.  A GPU box shows every core of the host to os.cpu_count() while a

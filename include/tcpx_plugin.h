@@ -61,7 +61,13 @@ ncclResult_t tcpxIrecvConsumed(void* recvComm, int n, void* request);           
  * tcpxListen writes the listener's identity into the 128-byte handle; tcpxConnect_v5 with that handle joins the
  * listener's backlog (ncclSystemError if the listener is closed, ncclInternalError for a handle tcpxListen did not
  * write); tcpxAccept_v5 returns success with *recvComm = NULL until a connection is waiting
- * (src/net_tcpx.cc:761-769). */
+ * (src/net_tcpx.cc:761-769).
+ *
+ * With NCCL_GPUDIRECTTCPX_AMD_HELPER_THREAD=1 a receive comm's sockets are served by a thread of its own (the receive
+ * part of persistentSocketThread, src/net_tcpx.cc:252-384).  NCCL_GPUDIRECTTCPX_RX_BINDINGS, in the reference's syntax
+ * "name:lo-hi,lo-hi;name:lo-hi" with the device names that tcpxGetProperties reports, names the CPUs that thread may
+ * run on (parseCoreRanges, src/common.cc:65-130; sched_setaffinity over all of them, src/net_tcpx.cc:300-307):
+ * the two threads hand every task to each other, so how far apart their CPUs are is what that mode costs. */
 
 /* Undoes tcpxInit: stops the engines, frees arenas and cached queue memory.  Comms must be closed first.
  * The reference has no counterpart (NCCL never unloads it); a persistent kernel needs an orderly stop. */
@@ -180,6 +186,7 @@ typedef struct tcpxCommStats {
   uint64_t unpack_slow_cnt;  /* slowness reports while the GPU held a slot (no counterpart in the reference) */
   uint64_t unpack_ns;        /* publish -> completion word seen by tcpxTest, summed over unpack_cnt slots */
   uint64_t trace_dropped;    /* tracepoint events lost because nobody drained the buffer */
+  uint64_t socket_thread_cpus; /* CPUs the comm's socket thread may run on (NCCL_GPUDIRECTTCPX_RX_BINDINGS), 0 = no such thread */
 } tcpxCommStats;
 
 ncclResult_t tcpxGetFlowStats(void* recvComm, uint32_t flow, tcpxFlowStats* stats);

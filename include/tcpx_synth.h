@@ -78,6 +78,13 @@ const tcpxSynthRequest* tcpxSynthRequests(const tcpxSynthWorkload* workload);
  * refills recycled pages.  Deterministic in (seed, window, byte position). */
 int tcpxSynthFillWindow(const tcpxSynthWorkload* workload, uint32_t window, uint8_t* pool);
 
+/* How far apart two CPUs are: nanoseconds for a cache line to go from `cpu_a` to `cpu_b` and back, averaged over
+ * `rounds`, measured by two threads of this call, one pinned to each.  Two threads that hand work to each other (a
+ * proxy thread and the plugin's socket thread) cost this per hand-over, and on a host whose CPUs span sockets it
+ * varies tenfold between pairs; a measurement says which pair it ran on.  Returns 0; 4 for bad arguments; 2 if a
+ * CPU cannot be used. */
+int tcpxSynthCpuRoundTripNs(int cpu_a, int cpu_b, uint32_t rounds, double* ns);
+
 #ifdef __cplusplus
 }
 #endif

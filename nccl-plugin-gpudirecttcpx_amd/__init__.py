@@ -296,6 +296,7 @@ _SYNTH_PROTOTYPES = {
     "tcpxSynthFrags": (ctypes.POINTER(SynthFrag), [ctypes.c_void_p]),
     "tcpxSynthRequests": (ctypes.POINTER(SynthRequest), [ctypes.c_void_p]),
     "tcpxSynthFillWindow": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_uint32, ctypes.c_void_p]),
+    "tcpxSynthCpuRoundTripNs": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_uint32, ctypes.POINTER(ctypes.c_double)]),
 }
 
 
@@ -352,6 +353,7 @@ class CommStats(ctypes.Structure):
         ("unpack_slow_cnt", ctypes.c_uint64),
         ("unpack_ns", ctypes.c_uint64),
         ("trace_dropped", ctypes.c_uint64),
+        ("socket_thread_cpus", ctypes.c_uint64),
     ]
 
 

@@ -18,6 +18,8 @@
 #include <chrono>
 #include <cstdarg>
 #include <cstdio>
+#include <cstring>
+#include <string>
 
 #include "plugin_internal.h"
 
@@ -128,6 +130,61 @@ void parse_device_type() {
   INFO(NCCL_INIT, "device type %s", g.device_type == kDeviceUnpack ? "unpack (the caller's kernel copies)" : "host (the plugin's engine copies)");
 }
 
+// NCCL_GPUDIRECTTCPX_RX_BINDINGS: the CPUs a receive comm's socket thread may run on, per network device, in the
+// reference's syntax "name:lo-hi,lo-hi;name:lo-hi" (parseCoreRanges, src/common.cc:65-130; the names are the ones
+// getProperties reports).  A device that is not named keeps the CPUs the process may use (the reference's default is
+// the NIC's NUMA node, src/net_tcpx.cc:592-611; a synthetic device has none).  A malformed entry is reported and
+// skipped, as there.  Called once the device names exist.
+void parse_rx_bindings() {
+  for (int d = 0; d < kMaxDevices; ++d) {
+    CPU_ZERO(&g.rx_cpus[d]);
+    g.rx_bound[d] = false;
+  }
+  const char* v = getenv("NCCL_GPUDIRECTTCPX_RX_BINDINGS");
+  if (!v || !*v) return;
+  INFO(NCCL_INIT, "NCCL_GPUDIRECTTCPX_RX_BINDINGS %s", v);
+  const std::string all(v);
+  size_t at = 0;
+  while (at < all.size()) {
+    size_t end = all.find(';', at);
+    if (end == std::string::npos) end = all.size();
+    const std::string phrase = all.substr(at, end - at);
+    at = end + 1;
+    const size_t colon = phrase.find(':');
+    if (colon == std::string::npos) continue;
+    const std::string name = phrase.substr(0, colon);
+    int dev = -1;
+    for (int d = 0; d < g.n_devices; ++d) {
+      if (name == g.dev_names[d]) dev = d;
+    }
+    if (dev < 0) {
+      INFO(NCCL_NET, "%s not a device of this run", name.c_str());
+      continue;
+    }
+    cpu_set_t set;
+    CPU_ZERO(&set);
+    bool ok = true;
+    size_t r = colon + 1;
+    while (ok && r <= phrase.size()) {
+      size_t comma = phrase.find(',', r);
+      if (comma == std::string::npos) comma = phrase.size();
+      const std::string range = phrase.substr(r, comma - r);
+      r = comma + 1;
+      int lo = -1, hi = -1;
+      char tail = 0;
+      if (sscanf(range.c_str(), "%d-%d%c", &lo, &hi, &tail) != 2 || lo < 0 || hi < lo || hi >= CPU_SETSIZE) {
+        WARN("invalid range %s", range.c_str());
+        ok = false;
+        break;
+      }
+      for (int c = lo; c <= hi; ++c) CPU_SET(c, &set);
+    }
+    if (!ok || CPU_COUNT(&set) == 0) continue;
+    g.rx_cpus[dev] = set;
+    g.rx_bound[dev] = true;
+  }
+}
+
 // Timestamp of a tracepoint: the wall clock like the reference's exporter lines, or the injected clock.
 int64_t trace_timestamp() {
   if (g.clock_injected) return static_cast<int64_t>(g.clock());
@@ -214,6 +271,14 @@ inline void idle_pass(uint32_t* quiet_passes) {
 }
 
 void helper_main(Comm* comm) {  // persistentSocketThread, src/net_tcpx.cc:252-384 (receive part)
+  // The thread runs on the CPUs bound to its device, all of them (src/net_tcpx.cc:300-307); a refusal (a CPU the
+  // process may not use) leaves it where it was.  What it ends up with is kept for tcpxGetCommStats.
+  if (g.rx_bound[comm->dev] && sched_setaffinity(0, sizeof(cpu_set_t), &g.rx_cpus[comm->dev]) != 0) {
+    WARN("Comm %p dev %d: binding the socket thread failed: %s", static_cast<void*>(comm), comm->dev, strerror(errno));
+  }
+  cpu_set_t now;
+  CPU_ZERO(&now);
+  if (sched_getaffinity(0, sizeof now, &now) == 0) comm->helper_cpus.store(static_cast<uint64_t>(CPU_COUNT(&now)), std::memory_order_relaxed);
   uint32_t quiet_passes = 0;
   while (!comm->helper_stop.load(std::memory_order_acquire)) {
     bool idle = true;
@@ -522,6 +587,7 @@ ncclResult_t tcpxInit(ncclDebugLogger_t logFunction) {
     snprintf(g.dev_names[d], sizeof g.dev_names[d], "tcpx-amd-synth%d", d);
     snprintf(g.pci_paths[d], sizeof g.pci_paths[d], "/sys/class/net/tcpx-amd-synth%d/device", d);
   }
+  parse_rx_bindings();
   g.initialized = true;
   INFO(NCCL_INIT | NCCL_NET, "NET/GPUDirectTCPX-AMD initialised: %d device(s), %d flows per comm", g.n_devices,
        g.flows_per_comm);
@@ -1061,6 +1127,7 @@ ncclResult_t tcpxGetCommStats(void* recvComm, tcpxCommStats* stats) {
   stats->unpack_slow_cnt = comm->unpack_slow_cnt;
   stats->unpack_ns = comm->unpack_ns;
   stats->trace_dropped = comm->trace ? comm->trace->dropped() : 0;
+  stats->socket_thread_cpus = comm->helper_cpus.load(std::memory_order_relaxed);
   return ncclSuccess;
 }
 

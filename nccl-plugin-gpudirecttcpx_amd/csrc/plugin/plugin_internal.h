@@ -15,6 +15,7 @@
 #ifndef TCPX_AMD_PLUGIN_INTERNAL_H_
 #define TCPX_AMD_PLUGIN_INTERNAL_H_
 
+#include <sched.h>
 #include <sys/socket.h>
 #include <sys/uio.h>
 
@@ -289,6 +290,7 @@ struct Comm {  // struct tcpxComm, src/common.h:159-216
   // Optional socket thread (persistentSocketThread, src/net_tcpx.cc:252-384).
   std::thread helper;
   std::atomic<bool> helper_stop{false};
+  std::atomic<uint64_t> helper_cpus{0};  // CPUs the socket thread may run on, as it found them when it started
   bool use_helper = false;
 };
 
@@ -369,6 +371,9 @@ struct Global {
   int task_stats = 0;
   int request_stats = 0;
   int sampling_factor = 1;
+  // NCCL_GPUDIRECTTCPX_RX_BINDINGS (struct tcpxBindings, src/common.h): CPUs for the socket threads of a device's comms.
+  cpu_set_t rx_cpus[kMaxDevices];
+  bool rx_bound[kMaxDevices] = {};
   char dev_names[kMaxDevices][32];
   char pci_paths[kMaxDevices][64];
 };

@@ -4,10 +4,16 @@
 // are derived from the seed, so changing how one quantity is drawn does not disturb the others.
 // Payload bytes are a counter-based function of (seed, window, 8-byte word index): any part of the pool can be
 // produced on its own and in any order.
+#include <pthread.h>
+#include <sched.h>
+
 #include <algorithm>
+#include <atomic>
+#include <chrono>
 #include <cstdint>
 #include <cstring>
 #include <new>
+#include <thread>
 #include <vector>
 
 #include "tcpx_synth.h"
@@ -242,6 +248,45 @@ int tcpxSynthFillWindow(const tcpxSynthWorkload* w, uint32_t window, uint8_t* po
     for (uint64_t i = r.first_desc; i < r.first_desc + r.n_descs; ++i)
       fill_words(static_cast<uint64_t>(w->frags[i].frag_token) * (kPage / 8), kPage / 8);
   }
+  return 0;
+}
+
+// Two threads, one pinned to each CPU, pass a cache line back and forth.
+int tcpxSynthCpuRoundTripNs(int cpu_a, int cpu_b, uint32_t rounds, double* ns) {
+  if (!ns || rounds == 0 || cpu_a < 0 || cpu_b < 0 || cpu_a >= CPU_SETSIZE || cpu_b >= CPU_SETSIZE || cpu_a == cpu_b) return 4;
+  struct alignas(64) Ball {
+    std::atomic<uint64_t> v{0};
+  } ball;
+  std::atomic<int> failed{0};
+  auto pin = [&](int cpu) {
+    cpu_set_t set;
+    CPU_ZERO(&set);
+    CPU_SET(cpu, &set);
+    if (pthread_setaffinity_np(pthread_self(), sizeof set, &set) != 0) failed.store(1);
+  };
+  double seconds = 0;
+  std::thread a([&] {
+    pin(cpu_a);
+    const auto t0 = std::chrono::steady_clock::now();
+    for (uint64_t i = 0; i < rounds && !failed.load(std::memory_order_relaxed); ++i) {
+      ball.v.store(2 * i + 1, std::memory_order_release);
+      while (ball.v.load(std::memory_order_acquire) != 2 * i + 2 && !failed.load(std::memory_order_relaxed)) {
+      }
+    }
+    seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+  });
+  std::thread b([&] {
+    pin(cpu_b);
+    for (uint64_t i = 0; i < rounds && !failed.load(std::memory_order_relaxed); ++i) {
+      while (ball.v.load(std::memory_order_acquire) != 2 * i + 1 && !failed.load(std::memory_order_relaxed)) {
+      }
+      ball.v.store(2 * i + 2, std::memory_order_release);
+    }
+  });
+  a.join();
+  b.join();
+  if (failed.load()) return 2;
+  *ns = seconds / rounds * 1e9;
   return 0;
 }
 

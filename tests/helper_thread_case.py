@@ -1,5 +1,6 @@
-"""Run by test_plugin_host.py (test_socket_thread_mode, test_katy_scheduler_receives_the_same_bytes) in its own
-process: the flags are read at tcpxInit."""
+"""Run by test_plugin_host.py (test_socket_thread_mode, test_socket_thread_binding,
+test_katy_scheduler_receives_the_same_bytes) in its own process: the flags are read at tcpxInit.  Arguments, if any,
+name the configs to run."""
 import ctypes
 import os
 import sys
@@ -22,7 +23,10 @@ assert lib.tcpxSynthArenaCreate(0, arena_bytes, ctypes.byref(base)) == 0
 arena = np.frombuffer((ctypes.c_uint8 * arena_bytes).from_address(base.value), dtype=np.uint8)
 from nccl_plugin_gpudirecttcpx_amd import synth_driver  # noqa: E402
 
-for config, shrink in ((4, 4), (2, 2), (5, 3)):
+cases = ((4, 4), (2, 2), (5, 3))
+if len(sys.argv) > 1:  # only these configs
+    cases = tuple(c for c in cases if str(c[0]) in sys.argv[1:])
+for config, shrink in cases:
     wl = pkg.Workload(config, seed=31 + config, shrink=shrink)
     pool = arena[: wl.info.pool_bytes]
     wl.fill_window(0, pool)
@@ -31,6 +35,9 @@ for config, shrink in ((4, 4), (2, 2), (5, 3)):
     synth_driver.run_workload(comm, wl, buf.ctypes.data, n_flows=8, window=8)
     assert np.array_equal(buf, expected_bytes(pool, wl.frags, wl.requests, int(wl.info.dst_bytes))), config
     assert comm.outstanding_pages() == 0
+    stats = pkg.CommStats()
+    assert lib.tcpxGetCommStats(comm.comm, ctypes.byref(stats)) == 0
+    print("socket thread cpus", stats.socket_thread_cpus)
     comm.close()
 sched = ctypes.c_void_p()
 assert lib.tcpxFlowSchedCreate(None, ctypes.byref(sched)) == 0

@@ -504,6 +504,34 @@ def test_socket_thread_mode(tmp_path):
     assert "sched alg 0" in p.stdout
 
 
+def test_socket_thread_binding():
+    """NCCL_GPUDIRECTTCPX_RX_BINDINGS in the reference's syntax (parseCoreRanges, src/common.cc:65-130) binds a receive
+    comm's socket thread to the CPUs named for its device (src/net_tcpx.cc:300-307); entries for other devices and
+    malformed ranges leave it on the CPUs of the process."""
+    script = os.path.join(ROOT, "tests", "helper_thread_case.py")
+    allowed = sorted(os.sched_getaffinity(0))
+    one = allowed[-1]
+
+    def cpus(bindings, helper="1"):
+        env = dict(os.environ, NCCL_GPUDIRECTTCPX_AMD_HELPER_THREAD=helper, NCCL_GPUDIRECTTCPX_AMD_FLOWS="4")
+        env.pop("NCCL_GPUDIRECTTCPX_RX_BINDINGS", None)
+        if bindings is not None:
+            env["NCCL_GPUDIRECTTCPX_RX_BINDINGS"] = bindings
+        p = subprocess.run([sys.executable, script, "2"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env, timeout=300)
+        assert p.returncode == 0 and "helper-thread case ok" in p.stdout, p.stdout
+        return [int(line.split()[-1]) for line in p.stdout.splitlines() if line.startswith("socket thread cpus")]
+
+    assert cpus(None) == [len(allowed)]
+    assert cpus("tcpx-amd-synth0:%d-%d" % (one, one)) == [1]
+    assert cpus("eth9:0-1;tcpx-amd-synth0:%d-%d;" % (one, one)) == [1]
+    if len(allowed) >= 2:
+        lo, hi = allowed[0], allowed[1]
+        assert cpus("tcpx-amd-synth0:%d-%d,%d-%d" % (lo, lo, hi, hi)) == [2]
+    assert cpus("eth9:0-1") == [len(allowed)]  # another device's
+    assert cpus("tcpx-amd-synth0:%d" % one) == [len(allowed)]  # no upper end: invalid, as in the reference
+    assert cpus("tcpx-amd-synth0:%d-%d" % (one, one), helper="0") == [0]  # no socket thread
+
+
 # ---- flow scheduler (src/flow_mapper.h) -----------------------------------------------------------------------------
 def run_sched_script(lib, alg, script):
     sched = ctypes.c_void_p()

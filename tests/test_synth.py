@@ -107,3 +107,25 @@ def test_bad_arguments(pkg):
         pkg.Workload(9)
     with pytest.raises(ValueError):
         pkg.Workload(1, shrink=40)
+
+
+def test_cpu_round_trip_probe(pkg):
+    """The probe that says how far apart two CPUs are (what a hand-over between two threads costs): a plausible
+    time for a pair this process may use, errors for a pair it cannot be."""
+    import ctypes
+    import os
+
+    synth, ns = pkg.synth_lib(), ctypes.c_double(-1.0)
+    cpus = sorted(os.sched_getaffinity(0))
+    before = os.sched_getaffinity(0)
+    if len(cpus) >= 2:
+        assert synth.tcpxSynthCpuRoundTripNs(cpus[0], cpus[1], 2000, ctypes.byref(ns)) == 0
+        assert 5.0 < ns.value < 1e6  # a cache line there and back: tens of nanoseconds to a few microseconds
+    assert os.sched_getaffinity(0) == before  # the probe pins its own two threads, not the caller
+    assert synth.tcpxSynthCpuRoundTripNs(cpus[0], cpus[0], 10, ctypes.byref(ns)) == 4
+    assert synth.tcpxSynthCpuRoundTripNs(-1, cpus[0], 10, ctypes.byref(ns)) == 4
+    assert synth.tcpxSynthCpuRoundTripNs(cpus[0], cpus[-1] + 1 if len(cpus) < 2 else cpus[1], 0, ctypes.byref(ns)) == 4
+    assert synth.tcpxSynthCpuRoundTripNs(cpus[0], 100000, 10, ctypes.byref(ns)) == 4
+    not_mine = next((c for c in range(1024) if c not in before), None)
+    if not_mine is not None and not_mine < (os.cpu_count() or 0) + 64:
+        assert synth.tcpxSynthCpuRoundTripNs(cpus[0], not_mine, 10, ctypes.byref(ns)) == 2
