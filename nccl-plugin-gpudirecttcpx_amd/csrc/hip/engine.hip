@@ -1058,6 +1058,24 @@ int tcpxuEngineCreate(int device, const tcpxuEngineConfig* config, tcpxuEngine**
     }
     e->jobs_done = reinterpret_cast<uint32_t*>(reinterpret_cast<uint8_t*>(e->st) + sizeof(DevState));
     e->job_target = e->jobs_done + cfg.ring_entries;
+    // Test aid: where the engine's counts of submissions and tickets start.  Records are stamped with the low 32 bits
+    // of their sequence number, and a busy engine passes 2^32 submissions within the hour; a test that starts just
+    // below sees the crossing in milliseconds.
+    const char* vc = getenv("TCPXU_ENGINE_COUNT_FROM");
+    if (vc && *vc) {
+      const uint64_t from = strtoull(vc, nullptr, 0);
+      uint64_t* const counts[] = {&e->st->ticket_head, &e->st->tickets_done, &e->st->jobs_completed, &e->st->sub_head,
+                                  &e->st->tickets_out};  // device addresses: only computed here, never read
+      for (uint64_t* c : counts) {
+        if (hipMemcpy(c, &from, sizeof from, hipMemcpyHostToDevice) != hipSuccess) {
+          set_error("engine counters: %s", hipGetErrorString(hipGetLastError()));
+          rc = TCPXU_DEVICE_ERROR;
+          break;
+        }
+      }
+      e->tail = from;
+      e->ctl->tail = e->ctl->head = e->ctl->completed = from;
+    }
   } while (false);
   if (rc != TCPXU_SUCCESS) {
     tcpxuEngineDestroy(e);

@@ -407,17 +407,14 @@ def test_engine_bursts_around_the_idle_exit(pkg, hip, oracle):
     assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
 
 
-@pytest.mark.parametrize("depth", [3, 16, 128])
-def test_engine_storm_of_mixed_small_submissions(pkg, hip, oracle, depth, benchlib):
-    """Thousands of submissions of 0 to 300 ragged fragments in random order, `depth` of them in flight: runs of
-    submissions that the leader turns into tickets sixteen at a time are broken at every position by empty ones,
-    by ones just over the one-ticket limit and by ones that need many tickets; each submission owns a stretch of
-    the destination and every byte must be the oracle's."""
+def storm_workload(pkg, oracle, seed, n_submissions=3000):
+    """Submissions of 0 to 300 ragged fragments in random order, each owning a stretch of one destination buffer:
+    (pool on the device, sentinel-filled destination on the device, stream items, expected bytes, descriptor count)."""
     import torch
 
-    rng = np.random.default_rng(0x570A + depth)
+    rng = np.random.default_rng(seed)
     pool = np.random.default_rng(0xD00D).integers(0, 256, size=8 << 20, dtype=np.uint8)
-    sizes = rng.choice([0, 1, 2, 7, 8, 9, 15, 16, 17, 31, 32, 33, 40, 64, 65, 300], size=3000,
+    sizes = rng.choice([0, 1, 2, 7, 8, 9, 15, 16, 17, 31, 32, 33, 40, 64, 65, 300], size=n_submissions,
                        p=[.05, .1, .05, .05, .1, .05, .05, .2, .05, .05, .1, .03, .03, .03, .03, .03])
     rows, subs, dst_off = [], [], 0
     for n in sizes:
@@ -447,15 +444,49 @@ def test_engine_storm_of_mixed_small_submissions(pkg, hip, oracle, depth, benchl
         items[i].dst_base = dst_d.data_ptr() + GUARD + base
         items[i].descs_host = descs.ctypes.data + 16 * first
         items[i].n_descs = n
+    return pool_d, dst_d, items, expect, descs
+
+
+@pytest.mark.parametrize("depth", [3, 16, 128])
+def test_engine_storm_of_mixed_small_submissions(pkg, hip, oracle, depth, benchlib):
+    """Thousands of submissions of 0 to 300 ragged fragments in random order, `depth` of them in flight: runs of
+    submissions that the leader turns into tickets sixteen at a time are broken at every position by empty ones,
+    by ones just over the one-ticket limit and by ones that need many tickets; each submission owns a stretch of
+    the destination and every byte must be the oracle's."""
+    pool_d, dst_d, items, expect, descs = storm_workload(pkg, oracle, 0x570A + depth)
     e = Engine(pkg, hip)
-    print("engine storm case: depth=%d submissions=%d descriptors=%d" % (depth, len(subs), len(descs)), flush=True)
+    print("engine storm case: depth=%d submissions=%d descriptors=%d" % (depth, len(items), len(descs)), flush=True)
     wall, kern = ctypes.c_double(), ctypes.c_double()
-    lat = (ctypes.c_double * len(subs))()
-    pkg.check(benchlib.tcpxuEngineRunTimed(e.h, items, len(subs), 0, depth, 20000, ctypes.byref(wall), ctypes.byref(kern), lat), "tcpxuEngineRunTimed")
-    assert e.completed() == len(subs) and min(lat) > 0
+    lat = (ctypes.c_double * len(items))()
+    pkg.check(benchlib.tcpxuEngineRunTimed(e.h, items, len(items), 0, depth, 20000, ctypes.byref(wall), ctypes.byref(kern), lat), "tcpxuEngineRunTimed")
+    assert e.completed() == len(items) and min(lat) > 0
     e.destroy()
     got = dst_d.cpu().numpy()
     assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
+
+
+def test_engine_sequence_numbers_cross_2_to_the_32(pkg, hip, oracle, benchlib, monkeypatch):
+    """Submission entries and tickets are stamped with the low 32 bits of their sequence numbers, and the leader's
+    ring arithmetic runs on low words: an engine that starts 70000 below 2^32 (TCPXU_ENGINE_COUNT_FROM) crosses it
+    with its tickets first (after more than one lap of the ticket ring) and with its submissions later, under the
+    storm of mixed submissions, launch after launch; every launch's bytes must be the oracle's."""
+    start = (1 << 32) - 70000
+    pool_d, dst_d, items, expect, descs = storm_workload(pkg, oracle, 0xC2055)
+    monkeypatch.setenv("TCPXU_ENGINE_COUNT_FROM", str(start))
+    e = Engine(pkg, hip)
+    monkeypatch.delenv("TCPXU_ENGINE_COUNT_FROM")
+    assert e.completed() == start
+    launches = 70000 // len(items) + 4
+    print("engine sequence case: start=%d launches=%d submissions each=%d" % (start, launches, len(items)), flush=True)
+    wall, kern = ctypes.c_double(), ctypes.c_double()
+    for launch in range(launches):
+        dst_d.fill_(SENTINEL)
+        pkg.check(benchlib.tcpxuEngineRunTimed(e.h, items, len(items), 0, 64, 20000, ctypes.byref(wall), ctypes.byref(kern), None), "tcpxuEngineRunTimed")
+        assert e.completed() == start + (launch + 1) * len(items), launch
+        got = dst_d.cpu().numpy()
+        assert first_difference(got, expect) is None, "launch %d, first (index, got, want, count): %r" % (launch, first_difference(got, expect))
+    assert e.completed() > (1 << 32)
+    e.destroy()
 
 
 def test_engine_run_window_times_the_middle_of_a_stream(pkg, hip, oracle, benchlib):
