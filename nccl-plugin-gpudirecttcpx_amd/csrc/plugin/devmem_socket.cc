@@ -216,7 +216,10 @@ ssize_t devmem_recv(DevmemSocket* sock, int size, int offset, DataPipe* p, uint6
 }
 
 TaskRing::TaskRing() {
-  for (int i = 0; i < kMaxTasks; ++i) items[i].pipe = new DataPipe;
+  for (int i = 0; i < kMaxTasks; ++i) {
+    items[i].pipe = new DataPipe;
+    scatter[i] = items[i].pipe->scatter_list.data();
+  }
 }
 TaskRing::~TaskRing() {
   for (int i = 0; i < kMaxTasks; ++i) delete items[i].pipe;

@@ -224,6 +224,14 @@ ncclResult_t flow_progress(Comm* comm, int flow) {
   for (int served = 0; served < kMaxTasks; ++served) {
     if (tasks->has(kTaskActive)) {
       Task* t = tasks->first(kTaskActive);
+      if (t->offset == 0) {
+        // Nothing received for this task yet: its pipe starts empty.  (Done here, by the thread that serves the
+        // socket, where the reference has the thread that enqueues do it: the pipe then never leaves this thread.)
+        t->pipe->cnt_cache = 0;
+        t->pipe->bytes_cnt = 0;
+        t->pipe->pgtoks = t->pgtoks;
+        t->pipe->pgtok_cnt = t->pgtok_cnt;
+      }
       ncclResult_t res = ncclSuccess;
       const ssize_t bytes = devmem_recv(&fd->sock, t->size, t->offset, t->pipe, static_cast<uint64_t>(t->request_offset), &res);
       if (res != ncclSuccess) {
@@ -248,7 +256,10 @@ ncclResult_t flow_progress(Comm* comm, int flow) {
         t->offset += static_cast<int>(bytes);
         fd->bytes += static_cast<uint64_t>(bytes);
       }
-      if (t->offset == t->size) task_advance(comm, tasks, kTaskActive);  // ACTIVE -> COMPLETING
+      if (t->offset == t->size) {
+        t->cnt = static_cast<uint32_t>(t->pipe->cnt_cache);
+        task_advance(comm, tasks, kTaskActive);  // ACTIVE -> COMPLETING
+      }
     }
     if (!tasks->has(kTaskCompleting)) break;  // the active task, if any, is still waiting for bytes
     // The reference asks gpu_inline_test here, which always answers "done" (src/devcomm/nccl/inline.cu:55-60).
@@ -301,22 +312,23 @@ void enqueue_task(Comm* comm, Request* r) {
   const int sz = r->next_size;
   TaskRing* tasks = &comm->flows[flow].tasks;
   Task* t = tasks->next_free();
-  t->op = r->op;
+  t->op = static_cast<uint16_t>(r->op);
   t->data = static_cast<char*>(r->data) + r->offset;
   t->r = r;
   t->result = ncclSuccess;
   t->offset = 0;
   t->request_offset = r->offset;
   t->size = sz;
-  t->flow = flow;
+  t->flow = static_cast<uint16_t>(flow);
+  t->cnt = 0;
   t->watch.configure(static_cast<uint64_t>(g.timeout_threshold_ns), static_cast<uint64_t>(g.timeout_frequency_ns));
-  t->pipe->cnt_cache = 0;
-  t->pipe->bytes_cnt = 0;
+  t->pgtoks = nullptr;
+  t->pgtok_cnt = nullptr;
   if (comm->passive) {
     UnpackSlot* u = &r->slot;
     u->flows[flow] = flow;
-    t->pipe->pgtoks = &u->pgtoks[static_cast<size_t>(flow) * kSlotPages];
-    t->pipe->pgtok_cnt = &u->pgtok_cnts[flow];
+    t->pgtoks = &u->pgtoks[static_cast<size_t>(flow) * kSlotPages];
+    t->pgtok_cnt = &u->pgtok_cnts[flow];
     // Unlike the reference, the count is not zeroed here: a request may put several chunks on the same flow, and
     // every chunk's pages must be given back when the request is consumed.  It is zeroed when the slot is taken.
   }
@@ -340,13 +352,12 @@ ncclResult_t reap_tasks(Comm* comm) {
       t->r->size_pending -= t->size;
       if (t->op == kOpRecv && t->size > 0) {
         UnpackSlot* u = &t->r->slot;
-        if (u->cnt_cache + t->pipe->cnt_cache > static_cast<uint64_t>(kSlotPages)) {  // src/net_tcpx.cc:1350-1353
-          WARN("request too many pages %lu, failstop", static_cast<unsigned long>(u->cnt_cache + t->pipe->cnt_cache));
+        if (u->cnt_cache + t->cnt > static_cast<uint64_t>(kSlotPages)) {  // src/net_tcpx.cc:1350-1353
+          WARN("request too many pages %lu, failstop", static_cast<unsigned long>(u->cnt_cache + t->cnt));
           return fail_stop("request needs more descriptors than a slot holds");
         }
-        memcpy(u->mem + u->cnt_cache, t->pipe->scatter_list.data(), sizeof(union loadMeta) * t->pipe->cnt_cache);
-        u->cnt_cache += t->pipe->cnt_cache;
-        t->pipe->cnt_cache = 0;
+        memcpy(u->mem + u->cnt_cache, tasks->scatter[t - tasks->items], sizeof(union loadMeta) * t->cnt);
+        u->cnt_cache += t->cnt;
       }
       task_advance(comm, tasks, kTaskInactive);  // INACTIVE -> FREE
     }

@@ -20,6 +20,7 @@
 #include <sys/uio.h>
 
 #include <atomic>
+#include <cstddef>
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
@@ -205,21 +206,31 @@ ssize_t devmem_recv(DevmemSocket* sock, int size, int offset, DataPipe* pipe, ui
 struct Comm;
 struct Request;
 
-struct Task {  // struct tcpxTask, src/work_queue.h:38-59 (receive-side fields)
-  SlownessWatch watch;  // recvmsg finding nothing, over and over (tcpxTask::timeout)
-  int op = 0;
+// A task goes from the proxy thread (which fills it in) to the thread that serves its socket and back (descriptor
+// count, result), and with a socket thread each direction is a cache line travelling between two CPUs: everything
+// that travels is in the task's first line, and neither thread touches the other's bookkeeping (the pipe, the watch)
+// on the way.
+struct alignas(64) Task {  // struct tcpxTask, src/work_queue.h:38-59 (receive-side fields)
   int size = 0;
   int offset = 0;
   int request_offset = 0;
+  uint16_t op = 0;
+  uint16_t flow = 0;
   void* data = nullptr;
   Request* r = nullptr;
   ncclResult_t result = ncclSuccess;
-  DataPipe* pipe = nullptr;
-  int flow = 0;
+  uint32_t cnt = 0;                // descriptors the task produced (the pipe's cnt_cache when its last byte arrived)
+  DataPipe* pipe = nullptr;        // the slot's own, for the life of the ring
+  PageToken* pgtoks = nullptr;     // passive side: where the task's page tokens go (the request's slot, per flow)
+  size_t* pgtok_cnt = nullptr;
+  SlownessWatch watch;  // second line; recvmsg finding nothing, over and over (tcpxTask::timeout)
 };
+static_assert(offsetof(Task, watch) == 64, "what travels between the threads is one cache line");
 
 enum TaskStage { kTaskActive = 0, kTaskCompleting = 1, kTaskInactive = 2, kTaskStages = 3 };
 struct TaskRing : StageRing<Task, kMaxTasks, kTaskStages, std::atomic<uint32_t>> {
+  // Where each slot's pipe keeps its descriptors, never written after construction: a line both threads can keep.
+  alignas(64) const union loadMeta* scatter[kMaxTasks];
   TaskRing();
   ~TaskRing();
 };
@@ -331,8 +342,10 @@ struct DeviceState {
   size_t arena_bytes = 0;
   std::unique_ptr<std::atomic<int32_t>[]> page_refs;  // references held by the plugin, per arena page
   size_t n_pages = 0;
-  std::atomic<uint64_t> pages_outstanding{0};
-  tcpxuEngine* engine = nullptr;
+  // Counted up by whoever receives (every recvmsg) and down by whoever consumes: a cache line of its own, or every
+  // count would take the line with the fields around it away from the thread that reads those at every poll.
+  alignas(64) std::atomic<uint64_t> pages_outstanding{0};
+  alignas(64) tcpxuEngine* engine = nullptr;
   bool engine_started = false;
   int comms = 0;
   std::vector<QueueBlock> free_blocks;
