@@ -293,6 +293,13 @@ void helper_main(Comm* comm) {  // persistentSocketThread, src/net_tcpx.cc:252-3
   uint32_t quiet_passes = 0;
   while (!comm->helper_stop.load(std::memory_order_acquire)) {
     bool idle = true;
+    // The same from this side: what the proxy thread has enqueued lies in its CPU's cache.
+    for (int f = 0; f < comm->num_flows; ++f) __builtin_prefetch(&comm->flows[f].tasks.entered);
+    for (int f = 0; f < comm->num_flows; ++f) {
+      TaskRing* tasks = &comm->flows[f].tasks;
+      for (uint32_t i = tasks->stage_begin(kTaskActive), end = tasks->stage_end(kTaskActive); i != end; ++i)
+        __builtin_prefetch(&tasks->items[i % kMaxTasks]);
+    }
     for (int f = 0; f < comm->num_flows; ++f) {
       TaskRing* tasks = &comm->flows[f].tasks;
       if (tasks->has(kTaskActive) || tasks->has(kTaskCompleting)) {
@@ -342,6 +349,18 @@ void enqueue_task(Comm* comm, Request* r) {
 // whose task ring has room are offered to the scheduler.
 ncclResult_t reap_tasks(Comm* comm) {
   comm->sched->reset();  // src/net_tcpx.cc:1114
+  if (comm->use_helper) {
+    // What the socket thread has finished lies in its CPU's cache: the counters first, all flows at once, then every
+    // finished task's line and its first descriptors, so that the waits overlap instead of following one another.
+    for (int f = 0; f < comm->num_flows; ++f) __builtin_prefetch(&comm->flows[f].tasks.left_[kTaskCompleting]);
+    for (int f = 0; f < comm->num_flows; ++f) {
+      TaskRing* tasks = &comm->flows[f].tasks;
+      for (uint32_t i = tasks->stage_begin(kTaskInactive), end = tasks->stage_end(kTaskInactive); i != end; ++i) {
+        __builtin_prefetch(&tasks->items[i % kMaxTasks]);
+        __builtin_prefetch(tasks->scatter[i % kMaxTasks]);
+      }
+    }
+  }
   for (int i = 0; i < comm->num_flows; ++i) {
     int idx = comm->end_flow_idx - i;
     if (idx < 0) idx += comm->num_flows;
@@ -1102,10 +1121,10 @@ ncclResult_t tcpxDebugQueueState(void* recvComm, uint64_t* head, uint64_t* tail,
   if (request_idx) {
     // In the order of the reference's idx[]: [0] dequeue cursor, [1] left TRANSMITTING, [2] left ACTIVE,
     // [3] left POSTED, [4] enqueue cursor.
-    request_idx[0] = comm->rq.left[kReqInactive];
-    request_idx[1] = comm->rq.left[kReqTransmitting];
-    request_idx[2] = comm->rq.left[kReqActive];
-    request_idx[3] = comm->rq.left[kReqPosted];
+    request_idx[0] = comm->rq.stage_begin(kReqInactive);
+    request_idx[1] = comm->rq.stage_begin(kReqTransmitting);
+    request_idx[2] = comm->rq.stage_begin(kReqActive);
+    request_idx[3] = comm->rq.stage_begin(kReqPosted);
     request_idx[4] = comm->rq.entered;
   }
   return ncclSuccess;

@@ -82,26 +82,32 @@ inline void counter_store(std::atomic<uint32_t>& c, uint32_t v) { c.store(v, std
 
 template <typename Item, int Capacity, int Stages, typename Counter>
 struct StageRing {
+  // Each counter has one writer and a cache line of its own: the stages of a task ring are advanced by two threads
+  // (the socket thread and the proxy thread), and a counter that shared its line with the other thread's would be
+  // taken away from its writer at every step of the other.
+  struct alignas(64) Line {
+    Counter v;
+  };
   alignas(64) Counter entered;
-  alignas(64) Counter left[Stages];
+  Line left_[Stages];  // left[k] of the description above
   alignas(64) Item items[Capacity];
 
   StageRing() {
     counter_store(entered, 0);
-    for (int k = 0; k < Stages; ++k) counter_store(left[k], 0);
+    for (int k = 0; k < Stages; ++k) counter_store(left_[k].v, 0);
   }
-  uint32_t in_flight() const { return counter_load(entered) - counter_load(left[Stages - 1]); }
+  uint32_t in_flight() const { return counter_load(entered) - counter_load(left_[Stages - 1].v); }
   bool empty() const { return in_flight() == 0; }
   uint32_t num_free() const { return Capacity - in_flight(); }
   bool has_free() const { return num_free() > 0; }
   Item* next_free() { return &items[counter_load(entered) % Capacity]; }
   void enqueue() { counter_store(entered, counter_load(entered) + 1); }
 
-  uint32_t stage_begin(int k) const { return counter_load(left[k]); }
-  uint32_t stage_end(int k) const { return k == 0 ? counter_load(entered) : counter_load(left[k - 1]); }
+  uint32_t stage_begin(int k) const { return counter_load(left_[k].v); }
+  uint32_t stage_end(int k) const { return k == 0 ? counter_load(entered) : counter_load(left_[k - 1].v); }
   bool has(int k) const { return stage_end(k) != stage_begin(k); }
   Item* first(int k) { return &items[stage_begin(k) % Capacity]; }
-  void advance(int k) { counter_store(left[k], counter_load(left[k]) + 1); }
+  void advance(int k) { counter_store(left_[k].v, counter_load(left_[k].v) + 1); }
 };
 
 // ---- unpack queue -------------------------------------------------------------------------------------------------
