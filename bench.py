@@ -631,8 +631,13 @@ def main():
                 for which, other in (("nearest", min(apart, key=apart.get)), ("farthest", max(apart, key=apart.get))) if apart else ():
                     leg = plugin_path(pkg, hip, torch, some, pool, helper_thread=True, rx_bindings="tcpx-amd-synth0:%d-%d" % (other, other))
                     bound[which] = {"cpus": [cpus[0], other], "cache_line_round_trip_ns": round(apart[other]), "payload_GBps": leg.get("payload_GBps"), "host_ns_per_fragment": leg.get("host_ns_per_fragment")}
+            except OSError as err:  # a machine that does not let the process choose its CPUs: the unbound runs stand alone
+                bound["error"] = str(err)
             finally:
-                os.sched_setaffinity(0, cpus)
+                try:
+                    os.sched_setaffinity(0, cpus)
+                except OSError:
+                    pass
             result["plugin_path"]["with_socket_thread"]["socket_thread_bound_to_the_cpu"] = bound
 
     # ---- CPU baseline on this machine's host cores: rank 0, bounded sample ---------------------------------
