@@ -465,7 +465,7 @@ def main():
             "device": name.value.decode(),
             "compute_units": cus.value,
             "engine_workgroups": eff.workgroups,
-            "descs_per_ticket": eff.descs_per_ticket if eff.descs_per_ticket else "8..16 by backlog (a submission of at most 32 stays whole)",
+            "descs_per_ticket": eff.descs_per_ticket if eff.descs_per_ticket else "8..16 by backlog (a submission of at most 32 stays whole; up to 64 for short fragments)",
         },
         "roofline": {
             "bound": "hbm",

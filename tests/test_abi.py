@@ -69,10 +69,13 @@ def test_ticket_plan_arithmetic(pkg):
         rc = hip.tcpxuEngineTicketPlan(wgs, fixed, in_flight, n, nbytes, ctypes.byref(per), ctypes.byref(nt), ctypes.byref(lim))
         return rc, per.value, nt.value, lim.value
 
-    # by backlog (768 workers): below 13 descriptors per worker 8, below 18 12, then 16
+    # by backlog (768 workers): below 13 descriptors per worker 8, below 18 12, below 100 14, then 16
     assert plan(769, 0, 1, 1078) == (0, 8, 135, 524288)
     assert plan(769, 0, 10, 1078)[1:3] == (12, 90)  # 10780 in flight: 14.04 per worker
-    assert plan(769, 0, 64, 1078)[1:3] == (16, 68)
+    assert plan(769, 0, 16, 1078)[1:3] == (14, 77)  # one comm's sixteen slots: 22.5 per worker
+    assert plan(769, 0, 64, 1078)[1:3] == (14, 77)  # 89.8 per worker
+    assert plan(769, 0, 72, 1078)[1:3] == (16, 68)  # 101.1 per worker
+    assert plan(513, 0, 64, 1078)[1:3] == (16, 68)  # the bench's four comms on 512 workers: 134.8 per worker
     # with the payload hint, short fragments get more descriptors per ticket: 32, 48, at most 64
     assert plan(769, 0, 64, 2048, 2048 * 4096)[1] == 16
     assert plan(769, 0, 64, 2048, 2048 * 2731)[1] == 16 and plan(769, 0, 64, 2048, 2048 * 2730)[1] == 32
