@@ -136,7 +136,7 @@ def test_engine_workloads_full_size(pkg, hip, oracle, config):
     run_requests(pkg, hip, oracle, wl, read_back_while_running=True)
 
 
-@pytest.mark.parametrize("per_ticket", [1, 4, 16, 64])
+@pytest.mark.parametrize("per_ticket", [1, 4, 14, 16, 64])
 def test_engine_ticket_sizes(pkg, hip, oracle, per_ticket):
     wl = pkg.Workload(5, seed=5, shrink=3)
     run_requests(pkg, hip, oracle, wl, read_back_while_running=True, descs_per_ticket=per_ticket)
@@ -781,7 +781,7 @@ def test_engine_many_mid_size_submissions_waiting_at_once(pkg, hip, oracle, per_
     assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
 
 
-@pytest.mark.parametrize("per_ticket", [0, 5, 16])
+@pytest.mark.parametrize("per_ticket", [0, 5, 14, 16])
 def test_engine_lines_shared_across_the_ends_of_tickets(pkg, hip, oracle, per_ticket):
     """With eight or more submissions in flight the tickets of a submission share destination lines across their
     ends: runs of fragments with boundaries at every offset inside a line, and runs of short fragments, in slots of
