@@ -49,7 +49,7 @@ __device__ __forceinline__ void store_vec_sys(uint8_t* p, u32x4 v) {
 // The bulk of the payload is stored with the non-temporal hint on top of the system scope (sc0 sc1 nt): the
 // destination is written once and not read again by this kernel, and telling the caches so keeps it from
 // displacing other data (at an 8 MiB chunk of 4 KiB fragments, all from HBM: 2.80 against 2.58 TB/s of payload).
-// The hint on the loads as well measured slower.  No builtin combines the hint with a scope, so the store is
+// The hint on the loads as well measured no faster.  No builtin combines the hint with a scope, so the store is
 // written as an instruction; the s_nop covers the wait state the hardware wants between a store of more than
 // 8 bytes and a write to its data registers, which the compiler cannot insert for an instruction it does not see.
 #ifndef TCPXU_STORE_NT
