@@ -5,9 +5,13 @@
 
 One "step" is the unpack of one 8 MiB chunk of the 4-flow workload (about 2155 descriptors of at most 4 KiB,
 byte-unaligned sources in a 256 MiB bounce pool, contiguous destination), cut into two 4 MiB requests the way
-NCCL slices an 8 MiB chunk.  The chunk goes through the persistent engine exactly as the plugin drives it:
-descriptors are copied into a slot of a 16-deep mapped ring, the slot is published, the GPU unpacks it and
-writes a completion word that the host polls -- no kernel launch per request.  One engine serves every receive
+NCCL slices an 8 MiB chunk.  The chunk goes through the persistent engine by the entry point the plugin calls
+for every completed request (tcpxuEngineSubmitSized): descriptors are copied into a slot of a 16-deep mapped
+ring, the slot is published, the GPU unpacks it and writes a completion word that the host polls -- no kernel
+launch per request.  The descriptor lists are built beforehand here; the plugin builds them from control messages
+and fragments as they arrive, one proxy thread per comm, and that whole path through ncclNet_v7 (host-bound: it
+keeps as many slots at the GPU as its one thread can build ahead, `plugin_path.max_slots_at_gpu`) is reported
+beside the headline as `plugin_path`, the drop-in figure.  One engine serves every receive
 comm of the GPU; the headline keeps `--comms` (4) comms busy, each with the reference's queue depth of 16, taking
 turns; the same run with a single comm is reported beside it (`single_comm`).  Successive steps use different
 descriptor lists, different destinations (a ring of 128 chunks = 1 GiB, four times the 256 MiB Infinity Cache:
@@ -113,18 +117,19 @@ def plugin_path(pkg, hip, torch, workloads, pool, helper_thread=False, rx_bindin
     torch.cuda.synchronize()
     seconds, frags, lat = 0.0, 0, []
     for rep in range(3):  # the first pass warms up; the other two are timed
-        for c, wl in enumerate(workloads):
-            s, l = synth_driver.run_workload_native(comm, wl, dst.data_ptr() + c * chunk_bytes, window=8)
-            if rep > 0:
-                seconds += s
-                frags += int(wl.info.n_descs)
-                lat.extend(l)
+        # every chunk's requests in one list, sixteen posted at a time (the request ring's depth, src/work_queue.h:20)
+        s, l = synth_driver.run_chunks_native(comm, workloads, dst.data_ptr(), chunk_bytes, window=16)
+        if rep > 0:
+            seconds += s
+            frags += sum(int(wl.info.n_descs) for wl in workloads)
+            lat.extend(l)
     stats = pkg.CommStats()
     lib.tcpxGetCommStats(comm.comm, ctypes.byref(stats))
     comm.close()
     assert lib.tcpxFinalize() == 0
     payload = 2 * len(workloads) * chunk_bytes
     return {
+        "max_slots_at_gpu": int(stats.max_slots_at_gpu),
         "what": "8 MiB chunks through ncclNet_v7 (irecv/test/iflush/irecvConsumed) with the synthetic devmem socket, "
         + ("the proxy thread plus the plugin's socket thread" if helper_thread else "one proxy thread"),
         "payload_GBps": round(payload / seconds / 1e9, 2),

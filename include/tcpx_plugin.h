@@ -187,6 +187,7 @@ typedef struct tcpxCommStats {
   uint64_t unpack_ns;        /* publish -> completion word seen by tcpxTest, summed over unpack_cnt slots */
   uint64_t trace_dropped;    /* tracepoint events lost because nobody drained the buffer */
   uint64_t socket_thread_cpus; /* CPUs the comm's socket thread may run on (NCCL_GPUDIRECTTCPX_RX_BINDINGS), 0 = no such thread */
+  uint64_t max_slots_at_gpu; /* most slots of this comm that were with the engine at one time (at most 16) */
 } tcpxCommStats;
 
 ncclResult_t tcpxGetFlowStats(void* recvComm, uint32_t flow, tcpxFlowStats* stats);

@@ -354,6 +354,7 @@ class CommStats(ctypes.Structure):
         ("unpack_ns", ctypes.c_uint64),
         ("trace_dropped", ctypes.c_uint64),
         ("socket_thread_cpus", ctypes.c_uint64),
+        ("max_slots_at_gpu", ctypes.c_uint64),
     ]
 
 

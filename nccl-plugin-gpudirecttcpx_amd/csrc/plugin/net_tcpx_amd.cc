@@ -387,6 +387,7 @@ ncclResult_t reap_tasks(Comm* comm) {
 }
 
 ncclResult_t take_control_messages(Comm* comm, bool* enqueued);
+ncclResult_t submit_ready_requests(Comm* comm);
 
 // tcpxCommProgress, src/net_tcpx.cc:1099-1308 (receive branch)
 ncclResult_t comm_progress(Comm* comm) {
@@ -401,6 +402,7 @@ ncclResult_t comm_progress(Comm* comm) {
       for (int f = 0; f < comm->num_flows; ++f) TCPXCHECK(flow_progress(comm, f));
     }
     TCPXCHECK(reap_tasks(comm));
+    TCPXCHECK(submit_ready_requests(comm));
     bool enqueued = false;
     TCPXCHECK(take_control_messages(comm, &enqueued));
     if (!enqueued || comm->use_helper) break;
@@ -449,6 +451,19 @@ ncclResult_t take_control_messages(Comm* comm, bool* enqueued) {
         return ncclInternalError;
       }
       if (ctrl.type != TCPX_CTRL_INLINE) FlowData::bump(comm->flows[ctrl.index].rx_ctrl_done_cnt);
+      // What the peer announces decides which bytes of the receive buffer the GPU will write.  The reference takes
+      // both numbers as they come (src/net_tcpx.cc:995-1010) and a wrong one ends in a device error there; here a
+      // message longer than the posted receive, or a chunk that runs past the message's end, is refused before any
+      // descriptor is built from it.
+      if (ar->size_pending < 0 && ctrl.total > static_cast<uint32_t>(ar->posted_size)) {
+        WARN("control message announces %u bytes for a receive of %d posted", ctrl.total, ar->posted_size);
+        return ncclInternalError;
+      }
+      const int64_t message = ar->size_pending < 0 ? static_cast<int64_t>(ctrl.total) : ar->size;
+      if (ctrl.type != TCPX_CTRL_INLINE && static_cast<int64_t>(ar->offset) + ctrl.size > message) {
+        WARN("control message: chunk of %u bytes at %d runs past the message's %ld", ctrl.size, ar->offset, static_cast<long>(message));
+        return ncclInternalError;
+      }
       ar->next_flow = ctrl.index;  // tcpxCtrlRecv, src/net_tcpx.cc:995-1014
       ar->next_size = static_cast<int>(ctrl.size);
       if (ar->size_pending < 0) ar->size_pending = ar->size = static_cast<int>(ctrl.total);
@@ -522,6 +537,72 @@ ncclResult_t ensure_engine(DeviceState* ds) {
   if (!ds->engine_started) {
     TCPXCHECK(device_result(g.ops->engine_start(ds->engine), "engine_start"));
     ds->engine_started = true;
+  }
+  return ncclSuccess;
+}
+
+
+// Publishes a completed receive request's descriptor count and hands its slot to the engine (device type "host").
+// The count and the release are the reference's publish (src/net_tcpx.cc:1350-1357); the submission is this
+// build's doorbell.  *submitted stays false when the engine's submission ring is full: the caller tries again at
+// the next poll.
+ncclResult_t publish_to_engine(Comm* comm, Request* r, bool* submitted) {
+  *submitted = false;
+  UnpackQueue* q = comm->queue;
+  if (r->slot.cnt_cache > static_cast<uint64_t>(kSlotPages)) {  // src/net_tcpx.cc:1350-1353
+    WARN("request too many pages %lu, failstop", static_cast<unsigned long>(r->slot.cnt_cache));
+    return fail_stop("request needs more descriptors than a slot holds");
+  }
+  *r->slot.cnt = r->slot.cnt_cache;
+  std::atomic_thread_fence(std::memory_order_release);
+  q->meta->done[r->slot.idx].value = 0;
+  r->done_value = ++comm->done_seq;
+  // The descriptors the engine reads: the mapped slot, or -- for a small request, of which a comm has at
+  // most 16 in flight -- a second copy in the GPU's own memory, written through the BAR ahead of the
+  // submission, which saves the GPU a PCIe round trip before it can start copying.
+  const void* descs_dev = q->meta_dev->nccl.mem[r->slot.idx];
+  if (q->stage && r->slot.cnt_cache <= kStagedDescs) {
+    union loadMeta* copy = q->stage + r->slot.idx * kStagedDescs;
+    memcpy(copy, r->slot.mem, sizeof(union loadMeta) * r->slot.cnt_cache);
+    g.ops->visible_flush();
+    descs_dev = q->stage_dev + r->slot.idx * kStagedDescs;
+  }
+  // The request's size goes along as a hint (it sizes the engine's tickets for fragments shorter than a page).
+  const uint32_t n_descs = static_cast<uint32_t>(r->slot.cnt_cache);
+  void* done_flag = &q->meta_dev->done[r->slot.idx].value;
+  const int rc = g.ops->engine_submit_sized
+                     ? g.ops->engine_submit_sized(comm->device->engine, comm->device->arena, r->data, descs_dev, n_descs,
+                                                  static_cast<uint64_t>(r->offset), done_flag, r->done_value)
+                     : g.ops->engine_submit(comm->device->engine, comm->device->arena, r->data, descs_dev, n_descs,
+                                            done_flag, r->done_value);
+  if (rc == TCPXU_IN_PROGRESS) {  // submission ring full
+    --comm->done_seq;
+    return ncclSuccess;
+  }
+  TCPXCHECK(device_result(rc, "engine_submit"));
+  r->published = true;
+  r->published_ns = g.clock();
+  r->unpack_watch.configure(static_cast<uint64_t>(g.timeout_threshold_ns), static_cast<uint64_t>(g.timeout_frequency_ns));
+  comm->unpack_cnt++;
+  comm->slots_at_gpu++;
+  comm->max_slots_at_gpu = std::max(comm->max_slots_at_gpu, comm->slots_at_gpu);
+  *submitted = true;
+  return ncclSuccess;
+}
+
+// Device type "host": every request whose last byte has been accounted for goes to the engine at once, oldest
+// first, whether or not the caller has come to test it yet.  The reference reports done=1 at publish
+// (src/net_tcpx.cc:1354-1370), so that up to sixteen slots of a comm are with the consumer together
+// (src/devcomm/nccl/unpack1.h:30-65); here done=1 waits for the copy, and submitting ahead of the test is what
+// keeps that many slots at the GPU.  Completion is still reported strictly in posting order, by tcpxTest.
+ncclResult_t submit_ready_requests(Comm* comm) {
+  if (g.device_type != kDeviceHost) return ncclSuccess;
+  for (uint32_t i = comm->rq.stage_begin(kReqTransmitting), end = comm->rq.stage_end(kReqTransmitting); i != end; ++i) {
+    Request* r = &comm->rq.items[i % kMaxRequests];
+    if (r->published || r->op != kOpRecv || r->size == 0 || !request_done(r)) continue;
+    bool submitted = false;
+    TCPXCHECK(publish_to_engine(comm, r, &submitted));
+    if (!submitted) break;  // ring full: the younger ones wait behind this one
   }
   return ncclSuccess;
 }
@@ -822,7 +903,6 @@ ncclResult_t tcpxAccept_v5(void* listenComm, void** recvComm, ncclNetDeviceHandl
 }
 
 ncclResult_t tcpxRegMr(void* ocomm, void* data, int size, int type, void** mhandle) {
-  (void)size;
   if (ocomm == nullptr) {
     WARN("regMr called with NULL communicator.");
     return ncclInternalError;
@@ -834,6 +914,7 @@ ncclResult_t tcpxRegMr(void* ocomm, void* data, int size, int type, void** mhand
   MemHandle* m = static_cast<MemHandle*>(calloc(1, sizeof *m));
   if (!m) return ncclSystemError;
   m->ptr = data;
+  m->size = size < 0 ? 0 : static_cast<size_t>(size);  // the registered range bounds what a receive may write (get_request)
   m->mem_type = type;
   *mhandle = m;
   return ncclSuccess;
@@ -858,6 +939,15 @@ static ncclResult_t get_request(Comm* comm, int op, void* data, int size, MemHan
     WARN("mhandle is null");
     return ncclInternalError;
   }
+  // A receive lies inside the memory its handle registered.  (The reference does not look,
+  // src/net_tcpx.cc:862-896; here whatever the request names is what the GPU writes.)
+  if (op == kOpRecv) {
+    const uintptr_t lo = reinterpret_cast<uintptr_t>(mh->ptr), at = reinterpret_cast<uintptr_t>(data);
+    if (size < 0 || at < lo || at - lo > mh->size || static_cast<size_t>(size) > mh->size - (at - lo)) {
+      WARN("receive of %d bytes at %p lies outside its registration [%p, +%zu)", size, data, mh->ptr, mh->size);
+      return ncclInternalError;
+    }
+  }
   if (!comm->rq.has_free()) {
     WARN("unable to allocate requests");
     return ncclInternalError;
@@ -870,6 +960,7 @@ static ncclResult_t get_request(Comm* comm, int op, void* data, int size, MemHan
   r->data = data;
   r->offset = 0;
   r->size = size;
+  r->posted_size = size;
   r->size_pending = op == kOpSend ? size : -1;
   r->comm = comm;
   r->slot = UnpackSlot{};  // cnt == nullptr: no slot yet
@@ -928,56 +1019,24 @@ ncclResult_t tcpxTest(void* request, int* done, int* size) {
   if (r->op == kOpRecv) {
     if (r->size) {
       UnpackQueue* q = comm->queue;
-      if (!r->published) {
+      if (g.device_type == kDeviceUnpack) {
         if (r->slot.cnt_cache > static_cast<uint64_t>(kSlotPages)) {  // src/net_tcpx.cc:1350-1353
           WARN("request too many pages %lu, failstop", static_cast<unsigned long>(r->slot.cnt_cache));
           return fail_stop("request needs more descriptors than a slot holds");
         }
-        // Publish: descriptor count, then a release, then the submission that makes the GPU look
-        // (src/net_tcpx.cc:1354-1357 is the count + fences; the doorbell is this build's).
+        // The reference's publish and nothing else (src/net_tcpx.cc:1354-1357): the count, a release, and the store
+        // fence that pushes it out of the write-combining buffers; whoever holds the device handle copies.  done=1
+        // means "published".
         *r->slot.cnt = r->slot.cnt_cache;
         std::atomic_thread_fence(std::memory_order_release);
-        if (g.device_type == kDeviceUnpack) {
-          // The reference's publish and nothing else: the count is visible to the device (the store fence pushes
-          // it out of the write-combining buffers, src/net_tcpx.cc:1356), and whoever holds the device handle
-          // copies.  done=1 means "published".
-          __builtin_ia32_sfence();
-          comm->unpack_cnt++;
-          request_advance(comm, kReqTransmitting);
-          *done = 1;
-          return ncclSuccess;
-        }
-        q->meta->done[r->slot.idx].value = 0;
-        r->done_value = ++comm->done_seq;
-        // The descriptors the engine reads: the mapped slot, or -- for a small request, of which a comm has at
-        // most 16 in flight -- a second copy in the GPU's own memory, written through the BAR ahead of the
-        // submission, which saves the GPU a PCIe round trip before it can start copying.
-        const void* descs_dev = q->meta_dev->nccl.mem[r->slot.idx];
-        if (q->stage && r->slot.cnt_cache <= kStagedDescs) {
-          union loadMeta* copy = q->stage + r->slot.idx * kStagedDescs;
-          memcpy(copy, r->slot.mem, sizeof(union loadMeta) * r->slot.cnt_cache);
-          g.ops->visible_flush();
-          descs_dev = q->stage_dev + r->slot.idx * kStagedDescs;
-        }
-        // The request's size goes along as a hint (it sizes the engine's tickets for fragments shorter than a page).
-        const uint32_t n_descs = static_cast<uint32_t>(r->slot.cnt_cache);
-        void* done_flag = &q->meta_dev->done[r->slot.idx].value;
-        const int rc = g.ops->engine_submit_sized
-                           ? g.ops->engine_submit_sized(comm->device->engine, comm->device->arena, r->data, descs_dev,
-                                                        n_descs, static_cast<uint64_t>(r->offset), done_flag,
-                                                        r->done_value)
-                           : g.ops->engine_submit(comm->device->engine, comm->device->arena, r->data, descs_dev, n_descs,
-                                                  done_flag, r->done_value);
-        if (rc == TCPXU_IN_PROGRESS) {  // submission ring full: try again at the next poll
-          --comm->done_seq;
-          return ncclSuccess;
-        }
-        TCPXCHECK(device_result(rc, "engine_submit"));
-        r->published = true;
-        r->published_ns = g.clock();
-        r->unpack_watch.configure(static_cast<uint64_t>(g.timeout_threshold_ns), static_cast<uint64_t>(g.timeout_frequency_ns));
+        __builtin_ia32_sfence();
         comm->unpack_cnt++;
+        request_advance(comm, kReqTransmitting);
+        *done = 1;
+        return ncclSuccess;
       }
+      // The progress call above has submitted the slot, unless the engine's submission ring was full.
+      if (!r->published) return ncclSuccess;
       const uint64_t seen =
           reinterpret_cast<std::atomic<uint64_t>*>(&q->meta->done[r->slot.idx].value)->load(std::memory_order_acquire);
       if (seen != r->done_value) {  // the GPU is still copying
@@ -995,6 +1054,7 @@ ncclResult_t tcpxTest(void* request, int* done, int* size) {
         }
         return ncclSuccess;
       }
+      comm->slots_at_gpu--;
       comm->unpack_ns += g.clock() - r->published_ns;
     } else {
       *r->slot.cnt = 0;  // src/net_tcpx.cc:1361
@@ -1158,6 +1218,7 @@ ncclResult_t tcpxGetCommStats(void* recvComm, tcpxCommStats* stats) {
   stats->unpack_ns = comm->unpack_ns;
   stats->trace_dropped = comm->trace ? comm->trace->dropped() : 0;
   stats->socket_thread_cpus = comm->helper_cpus.load(std::memory_order_relaxed);
+  stats->max_slots_at_gpu = comm->max_slots_at_gpu;
   return ncclSuccess;
 }
 

@@ -249,7 +249,8 @@ struct Request {  // struct tcpxRequest, src/work_queue.h:63-76
   int next_flow = -1;  // next_sock_id: >= 0 once a control message is pending for this request
   int next_size = 0;
   int offset = 0;
-  int size = 0;
+  int size = 0;          // the message's size once its first control message has been read; until then, posted_size
+  int posted_size = 0;   // what irecv was given: the most the message may be
   int size_pending = 0;
   UnpackSlot slot;
   // Engine hand-off: the slot has been submitted, and the value its completion word will take.
@@ -273,6 +274,7 @@ static_assert(sizeof(CtrlMessage) == 16, "control message is 16 bytes");
 
 struct MemHandle {  // struct tcpxMemHandle, src/common.h:90-98
   void* ptr;
+  size_t size;  // bytes registered (the reference does not keep it)
   int mem_type;
 };
 
@@ -301,6 +303,7 @@ struct Comm {  // struct tcpxComm, src/common.h:159-216
   UnpackQueue* queue = nullptr;
   DeviceState* device = nullptr;
   uint64_t done_seq = 0;
+  uint32_t slots_at_gpu = 0, max_slots_at_gpu = 0;  // slots submitted to the engine and not yet reported done
   SlownessWatch ctrl_watch;  // tcpxComm::ctrl_timeout
   uint64_t rx_ctrl_slow_cnt = 0, unpack_cnt = 0, unpack_slow_cnt = 0, unpack_ns = 0;
   std::unique_ptr<TraceBuffer> trace;  // tcpxComm::statsbuf; allocated when a stats level is on

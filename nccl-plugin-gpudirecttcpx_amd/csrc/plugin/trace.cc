@@ -10,7 +10,7 @@
 #include <chrono>
 
 static_assert(sizeof(tcpxTraceEvent) == 24, "tcpxTraceEvent is 24 bytes");
-static_assert(sizeof(tcpxFlowStats) == 32 && sizeof(tcpxCommStats) == 48, "stats records are plain 64-bit counters");
+static_assert(sizeof(tcpxFlowStats) == 32 && sizeof(tcpxCommStats) == 56, "stats records are plain 64-bit counters");
 
 namespace tcpx {
 

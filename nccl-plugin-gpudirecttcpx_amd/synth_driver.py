@@ -8,7 +8,7 @@ several steps in flight.  The payload must already be in the bounce arena.
 import ctypes
 import time
 
-from . import CTRL_INLINE, CTRL_NORMAL, NCCL_PTR_CUDA, NetDeviceHandle, SynthFrag, plugin_lib
+from . import CTRL_INLINE, CTRL_NORMAL, NCCL_PTR_CUDA, CommStats, NetDeviceHandle, SynthFrag, plugin_lib
 
 
 class PluginError(RuntimeError):
@@ -88,6 +88,11 @@ class RecvComm:
         n = ctypes.c_uint64()
         ok(self.lib.tcpxSynthOutstandingPages(self.comm, ctypes.byref(n)), "tcpxSynthOutstandingPages")
         return n.value
+
+    def stats(self):
+        st = CommStats()
+        ok(self.lib.tcpxGetCommStats(self.comm, ctypes.byref(st)), "tcpxGetCommStats")
+        return st
 
     def queue_state(self):
         head, tail = ctypes.c_uint64(), ctypes.c_uint64()
@@ -210,3 +215,29 @@ def run_workload_native(comm, workload, dst_ptr, window=8, timeout_ms=30000, fir
     )  # fmt: skip
     ok(rc, "tcpxSynthRunRequests")
     return seconds.value, list(lat[:count])
+
+
+def run_chunks_native(comm, workloads, dst_ptr, chunk_stride, window=16, timeout_ms=30000):
+    """Several workloads received back to back as ONE list of requests (workload c into dst_ptr + c * chunk_stride),
+    so that the request window stays full across them: tcpxSynthRunRequests over the concatenated fragment and
+    request arrays.  Returns (wall seconds, per-request latencies)."""
+    import numpy as np
+
+    frags, reqs, first = [], [], 0
+    for c, wl in enumerate(workloads):
+        r = np.array(wl.requests, copy=True)
+        r["first_desc"] += first
+        r["dst_off"] += c * chunk_stride
+        reqs.append(r)
+        frags.append(wl.frags)
+        first += len(wl.frags)
+    frags = np.ascontiguousarray(np.concatenate(frags))
+    reqs = np.ascontiguousarray(np.concatenate(reqs))
+    seconds = ctypes.c_double()
+    lat = (ctypes.c_double * max(len(reqs), 1))()
+    rc = comm.lib.tcpxSynthRunRequests(
+        comm.comm, frags.ctypes.data, reqs.ctypes.data, len(reqs), dst_ptr, len(workloads) * chunk_stride, window, timeout_ms,
+        ctypes.byref(seconds), lat,
+    )  # fmt: skip
+    ok(rc, "tcpxSynthRunRequests")
+    return seconds.value, list(lat[: len(reqs)])

@@ -70,6 +70,13 @@ int emu_release(int n) { /* completes the n oldest held submissions; returns how
   }
   return done;
 }
+int emu_release_at(int index) { /* completes the held submission at `index` (0 = oldest) ahead of the others */
+  if (index < 0 || index >= g_n_pending) return 0;
+  run_job(&g_pending[index]);
+  memmove(&g_pending[index], &g_pending[index + 1], sizeof(emu_job) * (size_t)(g_n_pending - index - 1));
+  --g_n_pending;
+  return 1;
+}
 uint64_t emu_counter(int which) {
   switch (which) {
     case 0: return g_submitted;

@@ -29,6 +29,8 @@ def load_emu():
     lib.emu_release.restype = ctypes.c_int
     lib.emu_release.argtypes = [ctypes.c_int]
     lib.emu_pending.restype = ctypes.c_int
+    lib.emu_release_at.restype = ctypes.c_int
+    lib.emu_release_at.argtypes = [ctypes.c_int]
     lib.emu_set_hold.argtypes = [ctypes.c_int]
     lib.emu_set_ring_full.argtypes = [ctypes.c_int]
     lib.emu_set_visible_off.argtypes = [ctypes.c_int]

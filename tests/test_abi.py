@@ -104,7 +104,7 @@ def test_struct_sizes_match_the_headers(pkg):
     assert ctypes.sizeof(pkg.SynthRequest) == 32 and ctypes.sizeof(pkg.SynthInfo) == 48
     assert ctypes.sizeof(pkg.EngineConfig) == 16 and ctypes.sizeof(pkg.StreamItem) == 32
     assert ctypes.sizeof(pkg.NetDeviceHandle) == 32 and ctypes.sizeof(pkg.NetProperties) == 56
-    assert ctypes.sizeof(pkg.FlowStats) == 32 and ctypes.sizeof(pkg.CommStats) == 48 and ctypes.sizeof(pkg.TraceEvent) == 24
+    assert ctypes.sizeof(pkg.FlowStats) == 32 and ctypes.sizeof(pkg.CommStats) == 56 and ctypes.sizeof(pkg.TraceEvent) == 24
 
 
 def test_missing_library_raises(pkg, monkeypatch, tmp_path):

@@ -129,6 +129,90 @@ def test_two_comms_share_one_engine(env, oracle):
         c.close()
 
 
+def test_a_comm_keeps_many_slots_at_the_gpu(env, oracle):
+    """Sixteen requests posted with all their fragments already there: polling the oldest submits every one of them
+    to the engine (the reference's consumer may hold all sixteen slots of a comm, src/devcomm/nccl/unpack1.h:30-65,
+    because its test() reports done at publish, src/net_tcpx.cc:1354-1370), done is still reported strictly in
+    posting order, and the bytes are the oracle's."""
+    import time
+
+    torch = env.torch
+    wl = env.pkg.Workload(3, seed=0x51075, shrink=5)  # 64 requests of 16 x 4 KiB
+    info = wl.info
+    pool = np.empty(info.pool_bytes, dtype=np.uint8)
+    wl.fill_window(0, pool)
+    upload(env, pool)
+    expect = np.full(GUARD + info.dst_bytes + GUARD, SENTINEL, dtype=np.uint8)
+    graft.oracle_unpack(oracle, expect[GUARD : GUARD + info.dst_bytes], pool, np.ascontiguousarray(wl.descs))
+    dst = torch.full((GUARD + info.dst_bytes + GUARD,), SENTINEL, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    comm = env.driver.RecvComm(0)
+    base = dst.data_ptr() + GUARD
+    mh = comm.reg(base, int(info.dst_bytes))
+    order = []
+    print("plugin case: 4 bursts of 16 requests of 64 KiB, all fed before the first poll", flush=True)
+    for burst in range(4):
+        posted = []
+        for k in range(16 * burst, 16 * burst + 16):
+            r = wl.requests[k]
+            first, n, total = int(r["first_desc"]), int(r["n_descs"]), int(r["bytes"])
+            rc, req = comm.irecv(base + int(r["dst_off"]), total, mh)
+            assert rc == 0
+            env.driver.feed_request(comm, wl.frags[first : first + n], total, 4)
+            posted.append((k, req))
+        assert comm.irecv(base, 4096, mh)[0] == 3, "the request ring holds sixteen (src/work_queue.h:20)"
+        deadline = time.time() + 30
+        while posted:
+            k, req = posted[0]
+            rc, done, _ = comm.test(req)
+            assert rc == 0
+            if done:
+                order.append(k)
+                assert comm.consumed(req) == 0
+                posted.pop(0)
+            else:
+                if len(posted) > 1:
+                    assert comm.test(posted[1][1])[0] == 3, "only the oldest request may be tested (src/net_tcpx.cc:1322-1328)"
+                assert time.time() < deadline, "request %d did not complete" % k
+    got = dst.cpu().numpy()
+    stats = comm.stats()
+    print("plugin case: most slots at the GPU at one time: %d" % stats.max_slots_at_gpu, flush=True)
+    assert order == list(range(64))
+    assert stats.unpack_cnt == 64 and stats.max_slots_at_gpu >= 8
+    assert comm.outstanding_pages() == 0
+    head, tail, _ = comm.queue_state()
+    assert head == tail == 64
+    comm.dereg(mh)
+    comm.close()
+    assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
+
+
+def test_native_driver_with_the_whole_request_ring_posted(env, oracle):
+    """tcpxSynthRunRequests with sixteen requests posted at a time over four 8 MiB chunks as one request list."""
+    torch = env.torch
+    wls = [env.pkg.Workload(2, seed=0xC0FFEE02 + 7919 * i) for i in range(4)]
+    info = wls[0].info
+    pool = np.empty(info.pool_bytes, dtype=np.uint8)
+    wls[0].fill_window(0, pool)
+    upload(env, pool)
+    chunk = int(info.dst_bytes)
+    expect = np.full(GUARD + 4 * chunk + GUARD, SENTINEL, dtype=np.uint8)
+    for c, wl in enumerate(wls):
+        graft.oracle_unpack(oracle, expect[GUARD + c * chunk : GUARD + (c + 1) * chunk], pool, np.ascontiguousarray(wl.descs))
+    dst = torch.full((GUARD + 4 * chunk + GUARD,), SENTINEL, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    comm = env.driver.RecvComm(0)
+    print("native plugin case: 4 chunks of 8 MiB, 16 requests posted at a time", flush=True)
+    seconds, lat = env.driver.run_chunks_native(comm, wls, dst.data_ptr() + GUARD, chunk, window=16)
+    got = dst.cpu().numpy()
+    stats = comm.stats()
+    print("native plugin case: %.1f GB/s, most slots at the GPU at one time: %d" % (4 * chunk / seconds / 1e9, stats.max_slots_at_gpu), flush=True)
+    assert comm.outstanding_pages() == 0 and len(lat) == sum(int(wl.info.n_requests) for wl in wls)
+    assert stats.unpack_cnt == len(lat) and 1 <= stats.max_slots_at_gpu <= 16
+    comm.close()
+    assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
+
+
 def test_hip_layer_is_what_init_bound(env):
     """The plugin on a GPU box runs on libtcpxu_hip.so: the device count it reports is the HIP layer's."""
     n = ctypes.c_int()

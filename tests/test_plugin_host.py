@@ -290,6 +290,129 @@ def test_done_only_after_the_copy_completed(env, comm):
     comm.dereg(mh)
 
 
+def post_and_feed(env, comm, ptr, mh, n, nbytes=8192):
+    """n receives of nbytes each, every one with its control message and fragments already there."""
+    reqs = []
+    for i in range(n):
+        rc, req = comm.irecv(ptr + i * nbytes, nbytes, mh)
+        assert rc == 0
+        comm.ctrl(i % 4, nbytes, 0, nbytes)
+        comm.deliver(i % 4, simple_request(env, comm, nbytes, page=i * (nbytes // 4096)))
+        reqs.append(req)
+    return reqs
+
+
+def test_every_complete_request_is_at_the_engine_before_it_is_tested(env, comm):
+    """A comm keeps up to sixteen slots with the consumer (src/devcomm/nccl/unpack1.h:30-65; the reference reports
+    done at publish, src/net_tcpx.cc:1354-1370): polling the OLDEST request submits every request whose bytes are
+    all there, and completion is still reported in posting order."""
+    env.emu.emu_set_hold(1)
+    buf, ptr = host_buffer(16 * 8192)
+    mh = comm.reg(ptr, 16 * 8192)
+    reqs = post_and_feed(env, comm, ptr, mh, 16)
+    submitted = env.emu.emu_counter(0)
+    for _ in range(40):
+        assert comm.test(reqs[0])[:2] == (0, 0)
+    assert env.emu.emu_counter(0) - submitted == 16 and env.emu.emu_pending() == 16
+    assert comm.stats().max_slots_at_gpu == 16
+    assert (buf == 0xA5).all()
+    for i, req in enumerate(reqs):
+        assert comm.test(req)[:2] == (0, 0)
+        if i + 1 < 16:
+            assert comm.test(reqs[i + 1])[0] == INTERNAL_ERROR  # src/net_tcpx.cc:1322-1328
+        env.emu.emu_release(1)
+        assert comm.test(req)[:2] == (0, 1)
+        assert np.array_equal(buf[: (i + 1) * 8192], env.arena_np[: (i + 1) * 8192]) and (buf[(i + 1) * 8192 :] == 0xA5).all()
+    assert env.emu.emu_counter(0) - submitted == 16, "a request is submitted to the engine exactly once"
+    for req in reqs:
+        assert comm.consumed(req) == 0
+    assert comm.outstanding_pages() == 0
+    comm.dereg(mh)
+
+
+def test_a_younger_slot_that_finishes_first_waits_for_the_older_one(env, comm):
+    """Completion words may arrive in any order; done is reported in posting order only."""
+    env.emu.emu_set_hold(1)
+    buf, ptr = host_buffer(3 * 8192)
+    mh = comm.reg(ptr, 3 * 8192)
+    r0, r1, r2 = post_and_feed(env, comm, ptr, mh, 3)
+    for _ in range(20):
+        assert comm.test(r0)[:2] == (0, 0)
+    assert env.emu.emu_pending() == 3
+    assert env.emu.emu_release_at(2) == 1 and env.emu.emu_release_at(1) == 1  # the two younger copies finish
+    assert np.array_equal(buf[8192:], env.arena_np[8192 : 3 * 8192]) and (buf[:8192] == 0xA5).all()
+    for _ in range(20):
+        assert comm.test(r0)[:2] == (0, 0), "the oldest request's own completion word gates it"
+    assert comm.test(r1)[0] == INTERNAL_ERROR and comm.test(r2)[0] == INTERNAL_ERROR
+    assert comm.consumed(r1) == INTERNAL_ERROR
+    assert env.emu.emu_release(1) == 1
+    assert comm.test(r0)[:2] == (0, 1)
+    assert comm.test(r2)[0] == INTERNAL_ERROR
+    assert comm.test(r1)[:2] == (0, 1) and comm.test(r2)[:2] == (0, 1)  # their words were there already
+    for r in (r0, r1, r2):
+        assert comm.consumed(r) == 0
+    assert np.array_equal(buf, env.arena_np[: 3 * 8192])
+    assert comm.stats().max_slots_at_gpu == 3
+    comm.dereg(mh)
+
+
+def test_submissions_behind_a_full_engine_ring_keep_their_order(env, comm):
+    buf, ptr = host_buffer(4 * 8192)
+    mh = comm.reg(ptr, 4 * 8192)
+    env.emu.emu_set_ring_full(1)
+    reqs = post_and_feed(env, comm, ptr, mh, 4)
+    submitted = env.emu.emu_counter(0)
+    for _ in range(20):
+        assert comm.test(reqs[0])[:2] == (0, 0)
+    assert env.emu.emu_counter(0) == submitted
+    env.emu.emu_set_ring_full(0)
+    for req in reqs:
+        for _ in range(20):
+            rc, done, _ = comm.test(req)
+            assert rc == 0
+            if done:
+                break
+        assert done == 1
+    assert env.emu.emu_counter(0) - submitted == 4
+    for req in reqs:
+        assert comm.consumed(req) == 0
+    assert np.array_equal(buf, env.arena_np[: 4 * 8192])
+    comm.dereg(mh)
+
+
+def test_a_receive_may_only_write_what_it_registered_and_posted(env, comm):
+    """Host-side bounds on what the GPU will be told to write (the reference checks none of them,
+    src/net_tcpx.cc:771-853, 862-896, 995-1010)."""
+    buf, ptr = host_buffer(4 * 8192)
+    mh = comm.reg(ptr + 8192, 8192)
+    assert comm.irecv(ptr, 8192, mh)[0] == INTERNAL_ERROR  # starts before the registration
+    assert comm.irecv(ptr + 8192, 8193, mh)[0] == INTERNAL_ERROR  # ends after it
+    assert comm.irecv(ptr + 12288, 8192, mh)[0] == INTERNAL_ERROR
+    assert comm.irecv(ptr + 8192, -1, mh)[0] == INTERNAL_ERROR
+    assert comm.queue_state()[2] == [0, 0, 0, 0, 0], "a refused receive takes no request"
+    # a message longer than the posted receive
+    rc, req = comm.irecv(ptr + 8192, 4096, mh)
+    assert rc == 0
+    comm.ctrl(0, 8192, 0, 8192)
+    assert comm.test(req)[0] == INTERNAL_ERROR
+    assert (buf == 0xA5).all() and env.emu.emu_pending() == 0
+
+
+def test_a_chunk_may_not_run_past_its_message(env, comm):
+    buf, ptr = host_buffer(8192)
+    mh = comm.reg(ptr, 8192)
+    rc, req = comm.irecv(ptr, 8192, mh)
+    assert rc == 0
+    comm.ctrl(0, 4096, 0, 8192)
+    comm.ctrl(1, 4097, 4096, 8192)
+    for _ in range(4):
+        rc = comm.test(req)[0]
+        if rc:
+            break
+    assert rc == INTERNAL_ERROR
+    assert (buf == 0xA5).all()
+
+
 def test_engine_ring_full_is_retried(env, comm):
     buf, ptr = host_buffer(8192)
     mh = comm.reg(ptr, 8192)
