@@ -226,6 +226,46 @@ def other_configs(pkg, torch, run, only=None):
     return out
 
 
+def storm_launch(pkg, hip, benchlib, torch, engine, in_flight, reps=64):
+    """One launch of the engine over the storm of 64 KiB requests (2048 requests of 16 whole pages from a 512 MiB
+    pool, `reps` times over, into a ring of 1 GiB of destinations), `in_flight` of them in flight."""
+    wl = pkg.Workload(3, seed=0xC0FFEE03)
+    info = wl.info
+    pool_d = torch.empty(int(info.pool_bytes), dtype=torch.uint8, device="cuda:0").random_(0, 256)
+    dst_d = torch.empty((1 << 30) + 512, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    descs = np.array(wl.descs, copy=True)
+    descs["dst_off"] %= 65536
+    n = len(wl.requests)
+    items = (pkg.StreamItem * (n * reps))()
+    for i in range(n * reps):
+        r = wl.requests[i % n]
+        items[i].bounce_base = pool_d.data_ptr()
+        items[i].dst_base = dst_d.data_ptr() + 256 + (i * 65536) % (1 << 30)
+        items[i].descs_host = descs.ctypes.data + 16 * int(r["first_desc"])
+        items[i].n_descs = int(r["n_descs"])
+        items[i].payload_bytes = int(r["bytes"])
+    wall, kern = ctypes.c_double(), ctypes.c_double()
+    pkg.check(benchlib.tcpxuEngineRunTimed(engine, items, len(items), n, in_flight, 20000, ctypes.byref(wall), ctypes.byref(kern), None), "tcpxuEngineRunTimed")
+    stats, split = pkg.EngineStats(), pkg.StreamSplit()
+    pkg.check(hip.tcpxuEngineGetStats(engine, ctypes.byref(stats)), "tcpxuEngineGetStats")
+    pkg.check(benchlib.tcpxuStreamLastSplit(ctypes.byref(split)), "tcpxuStreamLastSplit")
+    timed = n * (reps - 1)
+    return {
+        "what": "storm: %d requests of 64 KiB (16 whole pages each), %d in flight" % (n * reps, in_flight),
+        "requests": n * reps,
+        "requests_per_s": round(timed / (wall.value * 1e-6)),
+        "payload_GBps": round(timed * 65536 / (wall.value * 1e-6) / 1e9, 1),
+        "rw_frac_of_hbm_peak": round(2.0 * timed * 65536 / (wall.value * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+        "bytes_per_launch": 2.0 * 65536 * n * reps,
+        "launch_us": round(kern.value, 1),
+        "host_ns_per_publish": round(split.publish_ns / max(split.published, 1), 1),
+        "leader_entries_per_poll": round(stats.leader_entries / max(stats.leader_polls, 1), 2),
+        "leader_polls": int(stats.leader_polls),
+        "leader_polls_fetching_64": int(stats.leader_deep_polls),
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -251,7 +291,8 @@ def main():
         help="exactly one launch of the engine kernel in the process (no untimed launch before it, no single-comm run, "
         "no extras): what a kernel trace or a counter run of the headline should see",
     )
-    ap.add_argument("--one-config", type=int, default=0, choices=[0, 1, 4, 5], help="exactly one launch of the engine kernel over this other workload of the contract (1, 4 or 5), 64 slots in flight, and exit: for a profiler")
+    ap.add_argument("--one-config", type=int, default=0, choices=[0, 1, 3, 4, 5], help="exactly one launch of the engine kernel over this other workload of the contract (1, 4 or 5 with 64 slots in flight; 3, the storm of 64 KiB requests, with --in-flight), and exit: for a profiler")
+    ap.add_argument("--in-flight", type=int, default=1024, help="requests in flight for --one-config 3 (1..2048)")
     ap.add_argument(
         "--calibrate-copy",
         type=int,
@@ -314,9 +355,14 @@ def main():
             pkg.check(rc, "tcpxuEngineRunTimed")
             return wall.value, kern.value, None
 
-        out = other_configs(pkg, torch, run_once, only=args.one_config)
+        if args.one_config == 3:
+            out = {"config_3": storm_launch(pkg, hip, benchlib, torch, engine, args.in_flight)}
+            in_flight = args.in_flight
+        else:
+            out = other_configs(pkg, torch, run_once, only=args.one_config)
+            in_flight = 64
         pkg.check(hip.tcpxuEngineDestroy(engine), "tcpxuEngineDestroy")
-        print(json.dumps(dict(out["config_%d" % args.one_config], kernel="unpack_engine_kernel", slots_in_flight=64)))
+        print(json.dumps(dict(out["config_%d" % args.one_config], kernel="unpack_engine_kernel", slots_in_flight=in_flight)))
         return
     name = ctypes.create_string_buffer(256)
     cus = ctypes.c_int()
@@ -536,24 +582,51 @@ def main():
             "request_4MiB_1078_descs": {"p50": round(percentile(lat4m, 50), 2), "p99": round(percentile(lat4m, 99), 2)},
         }
         result["p50_request_us"] = result["latency_us"]["request_64KiB_16_descs"]["p50"]
-        # The small-message storm: all 2048 requests of 64 KiB (16 fragments of 4 KiB each), W of them in flight,
-        # W x 16 = 64 .. 2048 descriptors handed to the engine per pass of the host loop.
+        # The small-message storm: the 2048 requests of 64 KiB (16 fragments of 4 KiB each) sixteen times over, W of
+        # them in flight, W x 16 = 64 .. 32768 descriptors with the engine at a time; W = 2048 is the workload's
+        # "2048 concurrent requests" (the unpack queues of 128 comms).  The first 2048 are left out of the rate.
+        # Beside each rate, where the time went: the host thread's nanoseconds per publish (descriptors into the slot,
+        # the submission entry, one tail store per batch) and what the leader's polls of the submission ring found.
+        storm_reps = 16
+        many = (pkg.StreamItem * (n_storm * storm_reps))()
+        for i in range(n_storm * storm_reps):
+            src = storm_items[i % n_storm]
+            many[i].bounce_base = src.bounce_base
+            many[i].dst_base = dst_base + (i * 65536) % (storm_dst_bytes - 65536)
+            many[i].descs_host = src.descs_host
+            many[i].n_descs = src.n_descs
+            many[i].payload_bytes = src.payload_bytes
         sweep = []
-        for in_flight in (4, 8, 16, 32, 64, 128):
-            w, _, lat = run(storm_items, in_flight, want_latency=True)
+        stats0, stats1, split = pkg.EngineStats(), pkg.EngineStats(), pkg.StreamSplit()
+        for in_flight in (4, 8, 16, 32, 64, 128, 256, 512, 1024, 2048):
+            pkg.check(hip.tcpxuEngineGetStats(engine, ctypes.byref(stats0)), "tcpxuEngineGetStats")
+            w, _, lat = run(many, in_flight, warmup_items=n_storm, want_latency=True)
+            pkg.check(hip.tcpxuEngineGetStats(engine, ctypes.byref(stats1)), "tcpxuEngineGetStats")
+            pkg.check(benchlib.tcpxuStreamLastSplit(ctypes.byref(split)), "tcpxuStreamLastSplit")
+            timed = n_storm * (storm_reps - 1)
+            polls = stats1.leader_polls - stats0.leader_polls
             sweep.append(
                 {
                     "requests_in_flight": in_flight,
                     "descriptors_in_flight": 16 * in_flight,
-                    "requests_per_s": round(n_storm / (w * 1e-6)),
-                    "payload_GBps": round(n_storm * 65536 / (w * 1e-6) / 1e9, 1),
-                    "p50_us": round(percentile(lat, 50), 2),
-                    "p99_us": round(percentile(lat, 99), 2),
+                    "requests_per_s": round(timed / (w * 1e-6)),
+                    "payload_GBps": round(timed * 65536 / (w * 1e-6) / 1e9, 1),
+                    "p50_us": round(percentile(lat[n_storm:], 50), 2),
+                    "p99_us": round(percentile(lat[n_storm:], 99), 2),
+                    "host_ns_per_publish": round(split.publish_ns / max(split.published, 1), 1),
+                    "host_publishes_per_call": round(split.published / max(split.publish_calls, 1), 1),
+                    "host_share_of_wall_in_publish": round(split.publish_ns / max(split.wall_ns, 1.0), 3),
+                    "leader_entries_per_poll": round((stats1.leader_entries - stats0.leader_entries) / max(polls, 1), 2),
+                    "leader_polls_per_us": round(polls / max(split.wall_ns * 1e-3, 1e-9), 3),
+                    "leader_share_of_polls_fetching_64": round((stats1.leader_deep_polls - stats0.leader_deep_polls) / max(polls, 1), 3),
                 }
             )
+        best = max(sweep, key=lambda x: x["requests_per_s"])
         result["storm_64KiB"] = {
-            "requests": n_storm,
+            "requests": n_storm * storm_reps,
+            "requests_timed": n_storm * (storm_reps - 1),
             "latency": "publish of a request's slot -> host poller observes its completion word",
+            "best": {k: best[k] for k in ("requests_in_flight", "requests_per_s", "payload_GBps")},
             "sweep": sweep,
         }
         result["storm_64KiB_requests_per_s"] = next(x["requests_per_s"] for x in sweep if x["requests_in_flight"] == 16)

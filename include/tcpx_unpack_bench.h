@@ -51,12 +51,15 @@ typedef struct tcpxuStreamItem {
   uint32_t payload_bytes;          /* sum of the descriptors' lengths, 0 = unknown (see tcpxuEngineSubmitSized) */
 } tcpxuStreamItem;
 
-/* Slots the streaming driver can keep in flight: the unpack queues of eight receive comms. */
-#define TCPXU_STREAM_MAX_DEPTH (8 * TCPXU_QUEUE_DEPTH)
+/* Slots the streaming driver can keep in flight: the unpack queues of 128 receive comms (the storm of 2048
+ * concurrent small requests) -- with whole slots of TCPXU_SLOT_PAGES descriptors up to the queues of eight comms,
+ * beyond that for items of at most 64 descriptors only. */
+#define TCPXU_STREAM_MAX_DEPTH (128 * TCPXU_QUEUE_DEPTH)
+#define TCPXU_STREAM_FULL_SLOT_DEPTH (8 * TCPXU_QUEUE_DEPTH)
 
 /* Drives a started engine the way the plugin's proxy loop does, from one host thread: a mapped ring of `depth`
  * slots (1..TCPXU_STREAM_MAX_DEPTH; TCPXU_QUEUE_DEPTH is one comm's unpack queue, a multiple of it is that many
- * comms taking turns) of TCPXU_SLOT_PAGES descriptors each; for every item, in order: wait until the slot's
+ * comms taking turns) of TCPXU_SLOT_PAGES descriptors each (of 64 beyond TCPXU_STREAM_FULL_SLOT_DEPTH); for every item, in order: wait until the slot's
  * previous occupant has completed, copy the item's descriptors into the slot (the memcpy of
  * src/net_tcpx.cc:1128-1130), publish it (src/net_tcpx.cc:1354-1357), and poll completion words in FIFO order
  * (the tcpxTest / tcpxIrecvConsumed cadence).  Writes the wall time from the first publish to the last
@@ -65,6 +68,18 @@ typedef struct tcpxuStreamItem {
  * `stall_timeout_ms` milliseconds.  One stream at a time per process. */
 int tcpxuEngineStream(tcpxuEngine* engine, const tcpxuStreamItem* items, uint64_t n_items, uint32_t depth,
                       uint32_t stall_timeout_ms, double* wall_us, double* latency_us);
+
+/* Where the host thread's time went in the process's last stream (any of the calls below): nanoseconds inside the
+ * publish step (descriptors into the slot where not staged ahead, the batch of submissions, tcpxuEngineSubmitMany),
+ * the submissions and calls that made, the passes of the loop and the stream's wall time. */
+typedef struct tcpxuStreamSplit {
+  double publish_ns;
+  double wall_ns;
+  uint64_t published;
+  uint64_t publish_calls;
+  uint64_t passes;
+} tcpxuStreamSplit;
+int tcpxuStreamLastSplit(tcpxuStreamSplit* split);
 
 /* Same, with the first `warmup_items` items left out of *wall_us: the clock starts at the publish of item
  * `warmup_items` and stops at the last completion. */

@@ -111,7 +111,7 @@ int tcpxuUnpackBatch(int device, const void* bounce_base, void* dst_base, const 
 typedef struct tcpxuEngine tcpxuEngine;
 
 typedef struct tcpxuEngineConfig {
-  uint32_t ring_entries;    /* submission ring size, power of two >= 16, 0 = default (1024) */
+  uint32_t ring_entries;    /* submission ring size, power of two >= 16, 0 = default (4096) */
   uint32_t workgroups;      /* persistent grid size, 0 = two worker workgroups per compute unit + the leader */
   uint32_t descs_per_ticket;/* descriptors one workgroup takes at a time (1..64); 0 = chosen per submission from
                                the backlog of descriptors not yet unpacked: 8 when the engine is idle (lowest
@@ -147,6 +147,23 @@ int tcpxuEngineSubmit(tcpxuEngine* engine, const void* bounce_base, void* dst_ba
 int tcpxuEngineSubmitSized(tcpxuEngine* engine, const void* bounce_base, void* dst_base, const void* descs_dev,
                            uint32_t n_descs, uint64_t payload_bytes, void* done_flag_dev, uint64_t done_value);
 
+/* Several slots published under one lock with one store of the ring's tail: what a poller that finds several
+ * requests complete in one pass submits together (a storm of small requests is bound by the host's cost per
+ * publish).  All `n` submissions are checked first and none is queued if one is refused (TCPXU_INVALID_ARGUMENT).
+ * *accepted (may be NULL) receives how many went into the ring, in order from the first: all of them with
+ * TCPXU_SUCCESS, fewer (possibly none) with TCPXU_IN_PROGRESS when the ring is full -- the caller submits the rest
+ * later.  payload_bytes as in tcpxuEngineSubmitSized (0 = unknown; sizes of 4 GiB and more are passed as 2^32-1). */
+typedef struct tcpxuSubmission {
+  const void* bounce_base;
+  void* dst_base;
+  const void* descs_dev;
+  void* done_flag_dev;
+  uint64_t done_value;
+  uint32_t n_descs;
+  uint32_t payload_bytes;
+} tcpxuSubmission;
+int tcpxuEngineSubmitMany(tcpxuEngine* engine, const tcpxuSubmission* submissions, uint32_t n, uint32_t* accepted);
+
 /* Limits: n_descs may not exceed 65536 tickets' worth -- 65536 x descs_per_ticket, or 524288 (65536 x 8) with
  * descs_per_ticket = 0, and never 1048576: TCPXU_INVALID_ARGUMENT otherwise, decided on the host, nothing queued.
  * TCPXU_INTERNAL_ERROR from a submit means the kernel stopped answering while the entry was already queued: the
@@ -164,6 +181,18 @@ int tcpxuEngineTicketPlan(uint32_t workgroups, uint32_t descs_per_ticket, uint32
 
 /* Number of submissions the GPU has fully completed since creation (monotone; read from mapped memory). */
 int tcpxuEngineCompleted(tcpxuEngine* engine, uint64_t* completed);
+
+/* Counters since creation.  The leader's are written by the kernel when it leaves (stop or idle exit), so they
+ * are current after tcpxuEngineStop: polls of the submission ring, entries those polls consumed, and how many of
+ * the polls fetched 64 entries instead of 16 (the leader does that after a poll that found all sixteen there). */
+typedef struct tcpxuEngineStats {
+  uint64_t launches;
+  uint64_t submissions;
+  uint64_t leader_polls;
+  uint64_t leader_entries;
+  uint64_t leader_deep_polls;
+} tcpxuEngineStats;
+int tcpxuEngineGetStats(tcpxuEngine* engine, tcpxuEngineStats* stats);
 
 /* The configuration in effect (defaults resolved: actual grid size, ring size; ticket size 0 = by backlog). */
 int tcpxuEngineGetConfig(tcpxuEngine* engine, tcpxuEngineConfig* config);

@@ -83,6 +83,44 @@ class StreamItem(ctypes.Structure):
     ]
 
 
+class Submission(ctypes.Structure):
+    """tcpxuSubmission (include/tcpx_unpack_hip.h)."""
+
+    _fields_ = [
+        ("bounce_base", ctypes.c_void_p),
+        ("dst_base", ctypes.c_void_p),
+        ("descs_dev", ctypes.c_void_p),
+        ("done_flag_dev", ctypes.c_void_p),
+        ("done_value", ctypes.c_uint64),
+        ("n_descs", ctypes.c_uint32),
+        ("payload_bytes", ctypes.c_uint32),
+    ]
+
+
+class EngineStats(ctypes.Structure):
+    """tcpxuEngineStats (include/tcpx_unpack_hip.h)."""
+
+    _fields_ = [
+        ("launches", ctypes.c_uint64),
+        ("submissions", ctypes.c_uint64),
+        ("leader_polls", ctypes.c_uint64),
+        ("leader_entries", ctypes.c_uint64),
+        ("leader_deep_polls", ctypes.c_uint64),
+    ]
+
+
+class StreamSplit(ctypes.Structure):
+    """tcpxuStreamSplit (include/tcpx_unpack_bench.h)."""
+
+    _fields_ = [
+        ("publish_ns", ctypes.c_double),
+        ("wall_ns", ctypes.c_double),
+        ("published", ctypes.c_uint64),
+        ("publish_calls", ctypes.c_uint64),
+        ("passes", ctypes.c_uint64),
+    ]
+
+
 class MissingLibrary(RuntimeError):
     pass
 
@@ -170,6 +208,8 @@ _HIP_PROTOTYPES = {
         ],
     ),
     "tcpxuEngineCompleted": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint64)]),
+    "tcpxuEngineSubmitMany": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(Submission), ctypes.c_uint32, ctypes.POINTER(ctypes.c_uint32)]),
+    "tcpxuEngineGetStats": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(EngineStats)]),
     "tcpxuEngineRunning": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]),
     "tcpxuEngineGetConfig": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(EngineConfig)]),
     "tcpxuEngineDevice": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]),
@@ -191,6 +231,7 @@ _HIP_PROTOTYPES = {
 _BENCH_PROTOTYPES = {
     "tcpxuBenchLastError": (ctypes.c_char_p, []),
     "tcpxuCopyKernelLaunch": (ctypes.c_int, [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "tcpxuStreamLastSplit": (ctypes.c_int, [ctypes.POINTER(StreamSplit)]),
     "tcpxuEngineRunStamped": (
         ctypes.c_int,
         [

@@ -195,14 +195,22 @@ int copy_geometry(int device, void* dst, const void* src, size_t bytes, CopyLaun
 // is answered with a publish at once and the copy of up to 32 KiB of descriptors is not part of a slot's
 // turn-around.  This is where the plugin has them as well: it builds a request's descriptors while its fragments
 // arrive (src/sock/tcpx.h:178-199 into the task's scatter list), long before tcpxTest publishes the count.
+//
+// Up to TCPXU_STREAM_FULL_SLOT_DEPTH slots in flight each slot holds a whole unpack-queue slot (2048 descriptors);
+// beyond that, up to TCPXU_STREAM_MAX_DEPTH, every item must be small (at most kSmallSlotDescs descriptors: the
+// storm of 64 KiB requests) and the slots are that size.
 constexpr size_t kFlagStride = 64;
 constexpr size_t kSlotBytes = sizeof(tcpxuLoadMeta) * TCPXU_SLOT_PAGES;
+constexpr uint32_t kSmallSlotDescs = 64;
+constexpr size_t kSmallSlotBytes = sizeof(tcpxuLoadMeta) * kSmallSlotDescs;
 constexpr uint32_t kPhysSlots = 2 * TCPXU_STREAM_MAX_DEPTH;
 constexpr size_t kFlagsBytes = kFlagStride * kPhysSlots;
+constexpr size_t kSlotsBytes = std::max(kSlotBytes * 2 * TCPXU_STREAM_FULL_SLOT_DEPTH, kSmallSlotBytes* kPhysSlots);
 // Descriptors of a small item that are also copied into host-visible device memory, and the room per slot.
 constexpr uint32_t kStageDescs = 16;
 constexpr size_t kStageBytes = kStageDescs * sizeof(tcpxuLoadMeta);
 constexpr uint32_t kStageMaxDepth = 16;
+constexpr uint32_t kPublishBatch = 64;  // submissions handed to the engine under one lock
 
 struct Driver {
   void* host = nullptr;
@@ -213,15 +221,16 @@ struct Driver {
 };
 Driver g_driver[64];
 std::mutex g_driver_mu;  // one stream at a time
+tcpxuStreamSplit g_last_split = {};
 
 int driver_for(int device, Driver** out) {
   if (device < 0 || device >= 64) return TCPXU_INVALID_ARGUMENT;
   Driver* d = &g_driver[device];
-  if (!d->host) BENCH_TRY(tcpxuMappedAlloc(device, kFlagsBytes + kSlotBytes * kPhysSlots, &d->host, &d->dev));
+  if (!d->host) BENCH_TRY(tcpxuMappedAlloc(device, kFlagsBytes + kSlotsBytes, &d->host, &d->dev));
   if (!d->stage_tried) {
     // Optional: without it every item's descriptors are read from the mapped slot.
     d->stage_tried = true;
-    if (tcpxuVisibleAlloc(device, kStageBytes * kPhysSlots, &d->stage_host, &d->stage_dev) != TCPXU_SUCCESS)
+    if (tcpxuVisibleAlloc(device, kStageBytes * 2 * kStageMaxDepth, &d->stage_host, &d->stage_dev) != TCPXU_SUCCESS)
       d->stage_host = d->stage_dev = nullptr;
   }
   *out = d;
@@ -229,17 +238,25 @@ int driver_for(int device, Driver** out) {
 }
 
 // The streaming loop.  pub_us[i] / done_us[i]: when item i was published / seen completed, in microseconds since
-// the first publish.
+// the first publish.  One pass of the loop reaps what has completed, publishes up to `depth` in flight -- the
+// items of a pass go to the engine together (tcpxuEngineSubmitMany), as a poller that finds several requests
+// complete submits them -- and stages descriptors ahead.  The clock is read per pass, not per item (a read costs
+// 20 ns, a third of what a storm of small requests leaves the host per request): an item's publish stamp is taken
+// just before its batch is submitted and its completion stamp just after the reap that found it, so a latency is
+// never understated.
 int stream_items(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_items, uint32_t depth,
                  uint32_t stall_timeout_ms, double* pub_us, double* done_us) {
   if (!e || !items || depth == 0 || depth > TCPXU_STREAM_MAX_DEPTH) {
     set_error("stream needs an engine, items and 1..%d slots in flight", TCPXU_STREAM_MAX_DEPTH);
     return TCPXU_INVALID_ARGUMENT;
   }
+  const bool small_slots = depth > TCPXU_STREAM_FULL_SLOT_DEPTH;
+  const uint32_t slot_descs = small_slots ? kSmallSlotDescs : static_cast<uint32_t>(TCPXU_SLOT_PAGES);
+  const size_t slot_bytes = small_slots ? kSmallSlotBytes : kSlotBytes;
   for (uint64_t i = 0; i < n_items; ++i) {
-    if (items[i].n_descs > TCPXU_SLOT_PAGES) {
-      set_error("stream item %llu has %u descriptors, a slot holds %d", static_cast<unsigned long long>(i),
-                items[i].n_descs, TCPXU_SLOT_PAGES);
+    if (items[i].n_descs > slot_descs) {
+      set_error("stream item %llu has %u descriptors, a slot holds %u with %u in flight",
+                static_cast<unsigned long long>(i), items[i].n_descs, slot_descs, depth);
       return TCPXU_INVALID_ARGUMENT;
     }
   }
@@ -260,13 +277,14 @@ int stream_items(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_items,
   std::vector<const void*> descs_dev(phys, nullptr);
   int rc = TCPXU_SUCCESS;
   uint64_t next_stage = 0, next_submit = 0, next_done = 0;
+  tcpxuStreamSplit split = {};
   // Writes item i's descriptors where the GPU will read them.  The twin slot i % phys is free once item i - phys
   // has completed.
   auto stage = [&](uint64_t i) {
     const uint32_t slot = static_cast<uint32_t>(i % phys);
     const tcpxuStreamItem& it = items[i];
-    if (it.n_descs) memcpy(hb + kFlagsBytes + kSlotBytes * slot, it.descs_host, sizeof(tcpxuLoadMeta) * it.n_descs);
-    descs_dev[slot] = db + kFlagsBytes + kSlotBytes * slot;
+    if (it.n_descs) memcpy(hb + kFlagsBytes + slot_bytes * slot, it.descs_host, sizeof(tcpxuLoadMeta) * it.n_descs);
+    descs_dev[slot] = db + kFlagsBytes + slot_bytes * slot;
     if (small_to_device && it.n_descs != 0 && it.n_descs <= kStageDescs) {
       // A small request with few ahead of it: its descriptors also go into the GPU's own memory, ahead of the
       // submission.  (With many in flight the request waits in queues anyway, and the write through the BAR with
@@ -276,27 +294,49 @@ int stream_items(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_items,
       descs_dev[slot] = static_cast<uint8_t*>(d->stage_dev) + kStageBytes * slot;
     }
   };
+  tcpxuSubmission batch[kPublishBatch];
   const auto t0 = clock::now();
   auto last_progress = t0;
+  auto now = t0;
   while (next_done < n_items) {
     bool progress = false;
-    // Reap completions in FIFO order.
+    // Reap completions in FIFO order.  The completion words are lines that the GPU has just written, i.e. misses:
+    // the ones further on are asked for early.
+    const uint64_t done_before = next_done;
     while (next_done < next_submit) {
       const uint32_t slot = static_cast<uint32_t>(next_done % phys);
+      __builtin_prefetch(hb + kFlagStride * ((slot + 4) % phys));
       auto* flag = reinterpret_cast<std::atomic<uint64_t>*>(hb + kFlagStride * slot);
       if (flag->load(std::memory_order_acquire) != next_done + 1) break;
-      done_us[next_done] = us_since(t0, clock::now());
       ++next_done;
+    }
+    if (next_done != done_before) {
+      now = clock::now();
+      const double at = us_since(t0, now);
+      for (uint64_t i = done_before; i < next_done; ++i) done_us[i] = at;
       progress = true;
     }
     // Publish while fewer than `depth` are in flight.
     while (next_submit < n_items && next_submit - next_done < depth) {
-      if (next_stage == next_submit) stage(next_stage++);
-      const uint32_t slot = static_cast<uint32_t>(next_submit % phys);
-      const tcpxuStreamItem& it = items[next_submit];
-      pub_us[next_submit] = next_submit == 0 ? 0.0 : us_since(t0, clock::now());
-      rc = tcpxuEngineSubmitSized(e, it.bounce_base, it.dst_base, descs_dev[slot], it.n_descs, it.payload_bytes,
-                                  db + kFlagStride * slot, next_submit + 1);
+      const uint64_t want = std::min<uint64_t>(std::min<uint64_t>(n_items, next_done + depth) - next_submit, kPublishBatch);
+      const auto before = next_submit == 0 ? t0 : clock::now();
+      for (uint64_t k = 0; k < want; ++k) {
+        const uint64_t i = next_submit + k;
+        if (next_stage == i) stage(next_stage++);
+        const uint32_t slot = static_cast<uint32_t>(i % phys);
+        const tcpxuStreamItem& it = items[i];
+        batch[k] = tcpxuSubmission{it.bounce_base, it.dst_base, descs_dev[slot], db + kFlagStride * slot, i + 1, it.n_descs, it.payload_bytes};
+      }
+      uint32_t accepted = 0;
+      rc = tcpxuEngineSubmitMany(e, batch, static_cast<uint32_t>(want), &accepted);
+      now = clock::now();
+      const double at = us_since(t0, before);
+      for (uint64_t k = 0; k < accepted; ++k) pub_us[next_submit + k] = at;
+      next_submit += accepted;
+      split.publish_ns += 1e3 * us_since(before, now);
+      split.published += accepted;
+      split.publish_calls += 1;
+      if (accepted != 0) progress = true;
       if (rc == TCPXU_IN_PROGRESS) {
         rc = TCPXU_SUCCESS;
         break;  // engine ring full: reap first
@@ -305,26 +345,30 @@ int stream_items(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_items,
         set_error("submit of item %llu failed: %s", static_cast<unsigned long long>(next_submit), tcpxuLastError());
         break;
       }
-      ++next_submit;
-      progress = true;
     }
     if (rc != TCPXU_SUCCESS) break;
-    // One item's descriptors ahead per pass, so that completions are still seen promptly.
-    if (next_stage < n_items && next_stage < next_done + phys) {
+    // Descriptors ahead: one item per pass with few in flight, so that completions are still seen promptly; with
+    // many, as many as the last reap made room for.
+    for (uint32_t k = 0, most = depth <= 16 ? 1 : 16; k < most && next_stage < n_items && next_stage < next_done + phys; ++k) {
       stage(next_stage++);
       progress = true;
     }
-    const auto now = clock::now();
+    split.passes += 1;
     if (progress) {
       last_progress = now;
-    } else if (now - last_progress > std::chrono::milliseconds(stall_timeout_ms)) {
-      set_error("stream stalled: %llu of %llu items completed, %llu published",
-                static_cast<unsigned long long>(next_done), static_cast<unsigned long long>(n_items),
-                static_cast<unsigned long long>(next_submit));
-      rc = TCPXU_INTERNAL_ERROR;
-      break;
+    } else if ((split.passes & 1023) == 0) {
+      now = clock::now();
+      if (now - last_progress > std::chrono::milliseconds(stall_timeout_ms)) {
+        set_error("stream stalled: %llu of %llu items completed, %llu published",
+                  static_cast<unsigned long long>(next_done), static_cast<unsigned long long>(n_items),
+                  static_cast<unsigned long long>(next_submit));
+        rc = TCPXU_INTERNAL_ERROR;
+        break;
+      }
     }
   }
+  split.wall_ns = 1e3 * us_since(t0, clock::now());
+  g_last_split = split;
   return rc;
 }
 
@@ -414,6 +458,13 @@ int tcpxuCopyKernelLaunch(int device, void* dst, const void* src, size_t bytes, 
   CopyLaunch c;
   BENCH_TRY(copy_geometry(device, dst, src, bytes, &c));
   return launch_copy(&c, static_cast<hipStream_t>(stream));
+}
+
+int tcpxuStreamLastSplit(tcpxuStreamSplit* split) {
+  if (!split) return TCPXU_INVALID_ARGUMENT;
+  std::lock_guard<std::mutex> lock(g_driver_mu);
+  *split = g_last_split;
+  return TCPXU_SUCCESS;
 }
 
 int tcpxuEngineStreamWarm(tcpxuEngine* e, const tcpxuStreamItem* items, uint64_t n_items, uint64_t warmup_items,

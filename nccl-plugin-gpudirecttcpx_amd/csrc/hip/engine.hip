@@ -130,7 +130,11 @@ __host__ __device__ constexpr uint32_t max_descs_for(uint32_t fixed_per_ticket) 
   return fit < kMaxDescsPerSubmission ? static_cast<uint32_t>(fit) : kMaxDescsPerSubmission;
 }
 constexpr uint32_t kStopReplicas = 64;
-constexpr uint32_t kPollEntries = 16;  // submission entries fetched per leader poll (16 B per lane)
+constexpr uint32_t kPollEntries = 16;  // submission entries fetched per load instruction of a leader poll (16 B per lane)
+// A poll that finds all sixteen entries there and turns them into tickets at a stroke is followed by a deep poll:
+// four loads in flight together, 64 entries for the one PCIe round trip (about 1.5 us) that sixteen cost -- which
+// is what capped a storm of one-ticket requests near 9 M/s.
+constexpr uint32_t kDeepGroups = 3;    // groups of kPollEntries beyond the first in a deep poll
 constexpr uint32_t kAuxTicketsDone = 32, kAuxHostStop = 33, kAuxJobsCompleted = 34;  // lanes of the auxiliary load
 constexpr uint32_t kNeverIdleOut = 0xFFFFFFFFu;
 constexpr uint32_t kDefaultIdlePolls = 400;  // empty polls (about 1.2 us each) before the kernel leaves by itself
@@ -173,6 +177,11 @@ struct HostCtl {  // mapped host memory
   alignas(64) uint64_t completed;  // GPU -> host: submissions fully unpacked (mirrored when idle and at exit)
   alignas(64) uint64_t exited;     // GPU -> host: 0 running, 1 stopped on request, 2 left after being idle
   alignas(64) uint64_t exiting;    // GPU -> host: the leader is about to leave for idleness (see leader_loop)
+  // GPU -> host, written by the leader when it leaves: its polls of the ring, the entries they consumed and the
+  // polls that fetched 64 entries instead of 16, since the engine was created.
+  alignas(64) uint64_t leader_polls;
+  uint64_t leader_entries;
+  uint64_t leader_deep_polls;
   alignas(64) Record ring[1];      // ring_entries follow
 };
 
@@ -188,6 +197,7 @@ struct DevState {  // device memory
   alignas(64) uint64_t jobs_completed;  // submissions completed since creation
   alignas(64) uint64_t sub_head;        // leader-private: next submission index
   uint64_t tickets_out;                 // leader-private: tickets written so far
+  uint64_t leader_polls, leader_entries, leader_deep_polls;  // leader-private: running totals (see HostCtl)
   alignas(64) uint32_t exited_wgs;      // reset at every start, as are the stop words
   uint32_t exit_reason;
   alignas(256) StopWord stop[kStopReplicas];
@@ -240,7 +250,6 @@ __device__ __forceinline__ uint32_t lane_value(uint32_t v, uint32_t src_lane) {
 
 __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uint32_t* job_target,
                             uint32_t ring_mask, uint32_t fixed_per_ticket, uint32_t spin_limit) {
-  const uint32_t lane = threadIdx.x;
   // The leader's positions are the same in every lane: said outright, so that they stay in scalar registers (in
   // vector registers the compiler waits for the leader's own stores at the top of every pass).
   auto same_in_all_lanes = [](uint64_t v) {
@@ -254,6 +263,10 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
   const uint32_t workers = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(gridDim.x - 1)));
   uint64_t idle = 0;
   uint32_t reason = 0;
+  uint32_t polls = 0, entries = 0, deep_polls = 0;  // of this launch; added to the running totals at the end
+  // The next poll fetches 64 entries.  (A ring of fewer entries than that never has them.)
+  bool deep = false;
+  const bool ring_allows_deep = ring_mask + 1u >= (kDeepGroups + 1) * kPollEntries;
   // Fixed per-lane roles in the auxiliary load (second load of every poll), so that both loads of a poll are
   // issued back to back by all lanes and waited for once:
   //   lanes 0-15  jobs_done of the job slots of entries s..s+15    lanes 16-31  job_target of the same slots
@@ -264,6 +277,12 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
   const uint32_t* const jobs_completed_lo = reinterpret_cast<const uint32_t*>(&st->jobs_completed);
 
   for (;;) {
+    // What depends on the lane is worked out afresh in every pass (the empty statement hides from the compiler that
+    // the lane is the same each time): a dozen per-lane addresses kept in registers for the life of the loop are
+    // what would push the kernel beyond the 80 vector registers that let two workgroups share a compute unit, and a
+    // pass waits a microsecond for the host's memory anyway.
+    uint32_t lane = threadIdx.x;
+    asm volatile("" : "+v"(lane));
     // One round trip fetches entries s .. s+15: lane 4k+j reads sector j (three payload words and the stamp) of
     // entry s+k.
     const uint32_t k_of_lane = lane >> 2;
@@ -274,6 +293,26 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
     else if (lane == kAuxTicketsDone) aux_addr = tickets_done_lo;
     else if (lane == kAuxJobsCompleted) aux_addr = jobs_completed_lo;
     const uint32_t aux = sys_load(aux_addr);
+    // A deep poll: entries s+16 .. s+63 and their job slots' counters ride along in the same round trip.
+    u32x4 sect_more[kDeepGroups];
+    uint32_t aux_more[kDeepGroups];
+#pragma unroll
+    for (uint32_t g = 0; g < kDeepGroups; ++g) {
+      sect_more[g] = u32x4{0u, 0u, 0u, 0u};
+      aux_more[g] = 0;
+    }
+    if (deep) {
+#pragma unroll
+      for (uint32_t g = 0; g < kDeepGroups; ++g) {
+        const uint64_t s_g = s + (g + 1) * kPollEntries;
+        sect_more[g] = load_vec_sys(reinterpret_cast<const uint8_t*>(&ctl->ring[(s_g + k_of_lane) & ring_mask]) + 16 * (lane & 3));
+        if (lane < 2 * kPollEntries)
+          aux_more[g] = sys_load(lane < kPollEntries ? &jobs_done[(s_g + lane) & ring_mask]
+                                                     : &job_target[(s_g + lane - kPollEntries) & ring_mask]);
+      }
+      ++deep_polls;
+    }
+    ++polls;
 
     const uint32_t expect = static_cast<uint32_t>(s + k_of_lane + 1);
     const uint64_t ok_mask = __ballot(sect.w == expect);
@@ -302,46 +341,88 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
     // tickets: nothing here would apply to them, and what is worked out per lane first would only add to their
     // latency.)
     uint32_t consumed = 0;
+    bool deep_next = false;
     const uint32_t n_first = lane_value(sect.y, 3);
+    // What the four lanes of an entry know about it, for the sixteen entries of one group at once.
+    struct EntryView {
+      uint32_t n, bytes, per_ticket, target_prev, in_flight, slot;
+      bool sane, slot_free;
+    };
+    auto view_entries = [&](const u32x4& sc, uint32_t ax, uint64_t s0, uint64_t okm) {
+      EntryView v;
+      v.n = bcast(sc.y, lane | 3u);      // payload word 10 sits in .y of sector 3
+      v.bytes = bcast(sc.z, lane | 3u);  // payload word 11 sits in .z of sector 3
+      const bool all_sectors = ((okm >> (4 * k_of_lane)) & 0xFull) == 0xFull;
+      const uint32_t done_now = bcast(ax, k_of_lane);
+      v.target_prev = bcast(ax, kPollEntries + k_of_lane);
+      v.in_flight = static_cast<uint32_t>(s0 + k_of_lane) - jobs_completed + 1u;
+      v.per_ticket = fixed_per_ticket != 0 ? fixed_per_ticket : ticket_size_for_submission(v.in_flight, v.n, v.bytes, workers);
+      if (fixed_per_ticket == 0 && leader_behind && v.per_ticket < kFullTicket) v.per_ticket = kFullTicket;  // see below
+      v.sane = all_sectors && v.n - 1u < kMaxDescsPerSubmission;  // 1 .. 2^20 descriptors
+      v.slot_free = done_now == v.target_prev;  // every ticket ever issued for the job slot has been counted
+      v.slot = static_cast<uint32_t>(s0 + k_of_lane) & ring_mask;
+      return v;
+    };
+    // Every entry of a group fits one ticket (a storm of small requests): the leading run of them becomes tickets in
+    // one store instruction.  Returns the length of the run; `room` is what the ticket ring still takes.
+    auto write_single_tickets = [&](const EntryView& v, const u32x4& sc, uint32_t room) {
+      const uint64_t not_now = ~__ballot(v.sane && v.slot_free);
+      uint32_t run = not_now == 0 ? kPollEntries : static_cast<uint32_t>(__builtin_ctzll(not_now)) >> 2;
+      run = std::min(run, room);
+      if (run != 0) {
+        if (k_of_lane < run) {
+          const uint64_t t = tickets_out + k_of_lane;
+          const uint32_t stamp = static_cast<uint32_t>(t + 1);
+          const uint32_t target = v.target_prev + 1u;
+          u32x4 out{sc.x, sc.y, sc.z, stamp};
+          if ((lane & 3u) == 3) {
+            out.y = v.n | (v.slot << 8) | kOnlyTicket;
+            out.z = target;
+            sys_store(&job_target[v.slot], target);
+          }
+          store_vec_sys(reinterpret_cast<uint8_t*>(&st->tickets[t & (kTicketRing - 1)]) + 16 * (lane & 3u), out);
+        }
+        tickets_out += run;
+      }
+      return run;
+    };
     if ((ok_mask & 0xFull) == 0xFull &&  // entry s is there
         (n_first <= kMaxDescsPerTicket || (ready >= 2 && n_first <= kLaneTickets * kFullTicket))) {
-      const uint32_t n = bcast(sect.y, lane | 3u);      // payload word 10 sits in .y of sector 3
-      const uint32_t bytes = bcast(sect.z, lane | 3u);  // payload word 11 sits in .z of sector 3
-      const bool all_sectors = ((ok_mask >> (4 * k_of_lane)) & 0xFull) == 0xFull;
-      const uint32_t done_now = bcast(aux, k_of_lane);
-      const uint32_t target_prev = bcast(aux, kPollEntries + k_of_lane);
-      const uint32_t in_flight = static_cast<uint32_t>(s + k_of_lane) - jobs_completed + 1u;
-      uint32_t per_ticket =
-          fixed_per_ticket != 0 ? fixed_per_ticket : ticket_size_for_submission(in_flight, n, bytes, workers);
-      if (fixed_per_ticket == 0 && leader_behind && per_ticket < kFullTicket) per_ticket = kFullTicket;  // see below
-      const bool sane = all_sectors && n - 1u < kMaxDescsPerSubmission;  // 1 .. 2^20 descriptors
-      const bool slot_free = done_now == target_prev;  // every ticket ever issued for the job slot has been counted
+      const EntryView ev = view_entries(sect, aux, s, ok_mask);
+      const uint32_t n = ev.n, bytes = ev.bytes, per_ticket = ev.per_ticket, target_prev = ev.target_prev;
+      const uint32_t in_flight = ev.in_flight, slot = ev.slot;
+      const bool sane = ev.sane, slot_free = ev.slot_free;
       // The ticket ring has room while fewer than its size are outstanding (32-bit wrapping arithmetic).
       const uint32_t room = kTicketRing - (static_cast<uint32_t>(tickets_out) - tickets_done);
       const uint32_t sector = lane & 3u;
-      const uint32_t slot = static_cast<uint32_t>(s + k_of_lane) & ring_mask;
       if (__ballot(sane && n > per_ticket) == 0) {
-        // Every entry that is there fits one ticket (a storm of small requests): the leading run of them becomes
-        // tickets in one store instruction.
-        const uint64_t not_now = ~__ballot(sane && slot_free);
-        uint32_t run = not_now == 0 ? kPollEntries : static_cast<uint32_t>(__builtin_ctzll(not_now)) >> 2;
-        run = std::min(run, room);
-        if (run != 0) {
-          if (k_of_lane < run) {
-            const uint64_t t = tickets_out + k_of_lane;
-            const uint32_t stamp = static_cast<uint32_t>(t + 1);
-            const uint32_t target = target_prev + 1u;
-            u32x4 v{sect.x, sect.y, sect.z, stamp};
-            if (sector == 3) {
-              v.y = n | (slot << 8) | kOnlyTicket;
-              v.z = target;
-              sys_store(&job_target[slot], target);
+        consumed = write_single_tickets(ev, sect, room);
+        if (deep && consumed == kPollEntries) {
+          // The groups that rode along, in order, each as long as the one before it went through whole.  One loop
+          // body that the groups pass through in turn (the registers rotate), so that the three are not worked out
+          // side by side in three times the registers: the kernel must stay within 80 for two workgroups per
+          // compute unit.
+          uint32_t left = room - consumed;
+          u32x4 sc0 = sect_more[0], sc1 = sect_more[1], sc2 = sect_more[2];
+          uint32_t ax0 = aux_more[0], ax1 = aux_more[1], ax2 = aux_more[2];
+          static_assert(kDeepGroups == 3, "the rotation below");
+#pragma unroll 1
+          for (uint32_t g = 0; g < kDeepGroups; ++g) {
+            const uint64_t s_g = s + consumed;
+            const uint64_t okm = __ballot(sc0.w == static_cast<uint32_t>(s_g + k_of_lane + 1));
+            uint32_t run = 0;
+            if ((okm & 0xFull) == 0xFull) {
+              const EntryView more = view_entries(sc0, ax0, s_g, okm);
+              if (__ballot(more.sane && more.n > more.per_ticket) == 0) run = write_single_tickets(more, sc0, left);
             }
-            store_vec_sys(reinterpret_cast<uint8_t*>(&st->tickets[t & (kTicketRing - 1)]) + 16 * sector, v);
+            consumed += run;
+            left -= run;
+            if (run != kPollEntries) break;
+            sc0 = sc1, sc1 = sc2;
+            ax0 = ax1, ax1 = ax2;
           }
-          tickets_out += run;
-          consumed = run;
         }
+        deep_next = ring_allows_deep && consumed >= kPollEntries;
       } else if (ready >= 2 && n_first <= kLaneTickets * lane_value(per_ticket, 0)) {
         // Several entries, some of more than one ticket, the first of them not too many.  (The empty statement keeps
         // the compiler from working this block's division and lane exchanges out ahead of the branch, where every
@@ -474,8 +555,11 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
       }
       ++consumed;
     }
+    deep = deep_next;
     if (consumed != 0) {
+      consumed = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(consumed)));
       s += consumed;
+      entries += consumed;
       idle = 0;
       if (lane == 0) sys_store(&ctl->head, s);
       continue;
@@ -523,11 +607,20 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
   }
 
   // Every ticket written must be visible before any stop word is.
+  const uint32_t lane = threadIdx.x;
   drain_memory_ops();
   if (lane == 0) {
     sys_store(&st->sub_head, s);
     sys_store(&st->tickets_out, tickets_out);
     sys_store(&st->exit_reason, reason);
+    const uint64_t totals[3] = {sys_load(&st->leader_polls) + polls, sys_load(&st->leader_entries) + entries,
+                                sys_load(&st->leader_deep_polls) + deep_polls};
+    sys_store(&st->leader_polls, totals[0]);
+    sys_store(&st->leader_entries, totals[1]);
+    sys_store(&st->leader_deep_polls, totals[2]);
+    sys_store(&ctl->leader_polls, totals[0]);
+    sys_store(&ctl->leader_entries, totals[1]);
+    sys_store(&ctl->leader_deep_polls, totals[2]);
   }
   drain_memory_ops();
   sys_store(&st->stop[lane].value, 1u);
@@ -861,7 +954,7 @@ __device__ void worker_loop(State* st, uint32_t* jobs_done, uint32_t flags, uint
   }
 }
 
-__global__ __launch_bounds__(kEngineThreads) void unpack_engine_kernel(HostCtl* ctl, DevState* st, uint32_t* jobs_done,
+__global__ __launch_bounds__(kEngineThreads) __attribute__((amdgpu_waves_per_eu(6))) void unpack_engine_kernel(HostCtl* ctl, DevState* st, uint32_t* jobs_done,
                                                                    uint32_t* job_target, uint32_t ring_mask,
                                                                    uint32_t per_ticket, uint32_t spin_limit,
                                                                    uint32_t flags) {
@@ -954,6 +1047,7 @@ struct tcpxuEngine {
   bool launched = false;  // between a launch and the Stop that reaps it (the kernel may have left by itself)
   bool failed = false;    // the kernel stopped answering (see tcpxuEngineSubmitSized); nothing more is accepted
   uint64_t launches = 0;
+  uint64_t submissions = 0;
   std::mutex mu;
 };
 
@@ -989,7 +1083,7 @@ int tcpxuEngineCreate(int device, const tcpxuEngineConfig* config, tcpxuEngine**
   *engine = nullptr;
   tcpxuEngineConfig cfg{};
   if (config) cfg = *config;
-  if (cfg.ring_entries == 0) cfg.ring_entries = 1024;
+  if (cfg.ring_entries == 0) cfg.ring_entries = 4096;
   if ((cfg.ring_entries & (cfg.ring_entries - 1)) != 0 || cfg.ring_entries > (1u << 16) || cfg.ring_entries < 16) {
     set_error("ring_entries %u must be a power of two in [16, 65536]", cfg.ring_entries);
     return TCPXU_INVALID_ARGUMENT;
@@ -1186,47 +1280,84 @@ int tcpxuEngineSubmit(tcpxuEngine* e, const void* bounce_base, void* dst_base, c
 
 int tcpxuEngineSubmitSized(tcpxuEngine* e, const void* bounce_base, void* dst_base, const void* descs_dev,
                            uint32_t n_descs, uint64_t payload_bytes, void* done_flag_dev, uint64_t done_value) {
-  if (!e || !done_flag_dev || done_value == 0 || reinterpret_cast<uintptr_t>(done_flag_dev) % 8 != 0) {
+  const tcpxuSubmission one = {bounce_base, dst_base, descs_dev, done_flag_dev, done_value, n_descs,
+                               payload_bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : static_cast<uint32_t>(payload_bytes)};
+  uint32_t accepted = 0;
+  return tcpxuEngineSubmitMany(e, &one, 1, &accepted);
+}
+
+// What a submission must look like; decided on the host, before anything is queued.
+static int check_submission(const tcpxuEngine* e, const tcpxuSubmission& s) {
+  if (!s.done_flag_dev || s.done_value == 0 || reinterpret_cast<uintptr_t>(s.done_flag_dev) % 8 != 0) {
     set_error("submit needs an 8-byte aligned completion word and a nonzero completion value");
     return TCPXU_INVALID_ARGUMENT;
   }
-  if (n_descs > 0 && (!bounce_base || !dst_base || !descs_dev || reinterpret_cast<uintptr_t>(descs_dev) % 16 != 0)) {
+  if (s.n_descs > 0 && (!s.bounce_base || !s.dst_base || !s.descs_dev || reinterpret_cast<uintptr_t>(s.descs_dev) % 16 != 0)) {
     set_error("submit needs bounce, destination and a 16-byte aligned descriptor address");
     return TCPXU_INVALID_ARGUMENT;
   }
-  // Refused here, on the host: a submission whose tickets can never all fit the ticket ring would sit at the head of
-  // the submission ring for ever, and the leader neither stops nor idles out with an entry waiting.
-  if (n_descs > max_descs_for(e->per_ticket)) {
+  // A submission whose tickets can never all fit the ticket ring would sit at the head of the submission ring for
+  // ever, and the leader neither stops nor idles out with an entry waiting.
+  if (s.n_descs > max_descs_for(e->per_ticket)) {
     set_error("%u descriptors in one submission exceed the limit of %u (tickets of %u at least, %u tickets in flight at most)",
-              n_descs, max_descs_for(e->per_ticket), e->per_ticket ? e->per_ticket : kSmallestAdaptiveTicket, kTicketRing);
+              s.n_descs, max_descs_for(e->per_ticket), e->per_ticket ? e->per_ticket : kSmallestAdaptiveTicket, kTicketRing);
     return TCPXU_INVALID_ARGUMENT;
   }
+  return TCPXU_SUCCESS;
+}
+
+int tcpxuEngineSubmitMany(tcpxuEngine* e, const tcpxuSubmission* subs, uint32_t n, uint32_t* accepted) {
+  if (accepted) *accepted = 0;
+  if (!e || (!subs && n != 0)) {
+    set_error("submit needs an engine and submissions");
+    return TCPXU_INVALID_ARGUMENT;
+  }
+  for (uint32_t i = 0; i < n; ++i) TCPXU_TRY(check_submission(e, subs[i]));  // all or nothing: none is queued if one is refused
+  if (n == 0) return TCPXU_SUCCESS;
   std::lock_guard<std::mutex> lock(e->mu);
   if (e->failed) {
     set_error("the engine stopped answering earlier and accepts nothing more");
     return TCPXU_INTERNAL_ERROR;
   }
   const uint64_t head = reinterpret_cast<std::atomic<uint64_t>*>(&e->ctl->head)->load(std::memory_order_acquire);
-  if (e->tail - head >= e->ring_entries) return kTcpxuInProgress;
-  uint32_t p[kPayloadWords] = {};
-  const uint64_t v[5] = {reinterpret_cast<uint64_t>(bounce_base), reinterpret_cast<uint64_t>(dst_base),
-                         reinterpret_cast<uint64_t>(descs_dev), reinterpret_cast<uint64_t>(done_flag_dev),
-                         done_value};
-  for (int i = 0; i < 5; ++i) {
-    p[2 * i] = static_cast<uint32_t>(v[i]);
-    p[2 * i + 1] = static_cast<uint32_t>(v[i] >> 32);
+  const uint64_t room = e->ring_entries - (e->tail - head);
+  const uint32_t take = static_cast<uint32_t>(std::min<uint64_t>(room, n));
+  if (take == 0) return kTcpxuInProgress;
+  for (uint32_t k = 0; k < take; ++k) {
+    const tcpxuSubmission& sub = subs[k];
+    const uint64_t v[5] = {reinterpret_cast<uint64_t>(sub.bounce_base), reinterpret_cast<uint64_t>(sub.dst_base),
+                           reinterpret_cast<uint64_t>(sub.descs_dev), reinterpret_cast<uint64_t>(sub.done_flag_dev),
+                           sub.done_value};
+    // The entry's sixteen words in the order they lie (three payload words and the stamp per sector), written as
+    // four 16-byte stores: a record is valid for the leader once all four stamps are there, in whatever order the
+    // sectors arrive, so nothing has to be ordered within it.
+    const uint32_t stamp = static_cast<uint32_t>(e->tail + 1);
+    alignas(64) uint32_t w[16];
+    uint32_t p[kPayloadWords];
+    for (int i = 0; i < 5; ++i) {
+      p[2 * i] = static_cast<uint32_t>(v[i]);
+      p[2 * i + 1] = static_cast<uint32_t>(v[i] >> 32);
+    }
+    p[10] = sub.n_descs;
+    p[11] = sub.payload_bytes;
+    for (int sct = 0; sct < 4; ++sct) {
+      w[4 * sct] = p[3 * sct];
+      w[4 * sct + 1] = p[3 * sct + 1];
+      w[4 * sct + 2] = p[3 * sct + 2];
+      w[4 * sct + 3] = stamp;
+    }
+    Record* ent = &e->ctl->ring[e->tail & (e->ring_entries - 1)];
+    // What the descriptors say must be in memory before the entry that points to them can be seen.
+    std::atomic_thread_fence(std::memory_order_release);
+    typedef uint32_t host_u32x4 __attribute__((ext_vector_type(4)));
+    for (int sct = 0; sct < 4; ++sct)
+      *reinterpret_cast<volatile host_u32x4*>(&ent->w[4 * sct]) = *reinterpret_cast<const host_u32x4*>(&w[4 * sct]);
+    e->tail += 1;
   }
-  p[10] = n_descs;
-  p[11] = payload_bytes > 0xFFFFFFFFull ? 0xFFFFFFFFu : static_cast<uint32_t>(payload_bytes);
-  Record* ent = &e->ctl->ring[e->tail & (e->ring_entries - 1)];
-  volatile uint32_t* w = ent->w;
-  for (int i = 0; i < kPayloadWords; ++i) w[payload_slot(i)] = p[i];
+  e->submissions += take;
   std::atomic_thread_fence(std::memory_order_release);
-  const uint32_t stamp = static_cast<uint32_t>(e->tail + 1);
-  for (int sct = 0; sct < 4; ++sct) w[sct * 4 + 3] = stamp;
-  std::atomic_thread_fence(std::memory_order_release);
-  e->tail += 1;
   reinterpret_cast<std::atomic<uint64_t>*>(&e->ctl->tail)->store(e->tail, std::memory_order_release);
+  if (accepted) *accepted = take;
   // The kernel may have left for idleness, or be leaving right now (see leader_loop): publish first, then look.
   if (e->launched) {
     std::atomic_thread_fence(std::memory_order_seq_cst);
@@ -1234,7 +1365,7 @@ int tcpxuEngineSubmitSized(tcpxuEngine* e, const void* bounce_base, void* dst_ba
       const auto t0 = std::chrono::steady_clock::now();
       while (host_load(&e->ctl->exiting) != 0 && host_load(&e->ctl->exited) == 0) {
         if (std::chrono::steady_clock::now() - t0 > std::chrono::seconds(5)) {
-          // The entry is in the ring and stays there: this is not "not submitted, try again".  The engine is
+          // The entries are in the ring and stay there: this is not "not submitted, try again".  The engine is
           // marked failed so that the caller cannot queue the same work twice by retrying.
           e->failed = true;
           set_error("engine kernel announced that it is leaving and never did; the submission stays queued and the "
@@ -1245,6 +1376,17 @@ int tcpxuEngineSubmitSized(tcpxuEngine* e, const void* bounce_base, void* dst_ba
     }
     if (host_load(&e->ctl->exited) == 2) TCPXU_TRY(launch_locked(e));  // it left by itself: bring it back
   }
+  return take == n ? TCPXU_SUCCESS : kTcpxuInProgress;
+}
+
+int tcpxuEngineGetStats(tcpxuEngine* e, tcpxuEngineStats* stats) {
+  if (!e || !stats) return TCPXU_INVALID_ARGUMENT;
+  std::lock_guard<std::mutex> lock(e->mu);
+  stats->launches = e->launches;
+  stats->submissions = e->submissions;
+  stats->leader_polls = host_load(&e->ctl->leader_polls);
+  stats->leader_entries = host_load(&e->ctl->leader_entries);
+  stats->leader_deep_polls = host_load(&e->ctl->leader_deep_polls);
   return TCPXU_SUCCESS;
 }
 

@@ -73,8 +73,14 @@ def test_bench_extras_report_latency_and_the_storm_sweep():
     lat = r["latency_us"]["request_64KiB_16_descs"]
     assert 0 < lat["p50"] <= lat["p99"] and r["p50_request_us"] == lat["p50"]
     sweep = r["storm_64KiB"]["sweep"]
-    assert [x["descriptors_in_flight"] for x in sweep] == [64, 128, 256, 512, 1024, 2048] and r["storm_64KiB"]["requests"] == 2048
+    assert [x["requests_in_flight"] for x in sweep] == [4, 8, 16, 32, 64, 128, 256, 512, 1024, 2048]  # up to "2048 concurrent"
+    assert r["storm_64KiB"]["requests"] == 16 * 2048 and r["storm_64KiB"]["requests_timed"] == 15 * 2048
     assert all(x["requests_per_s"] > 0 and 0 < x["p50_us"] <= x["p99_us"] for x in sweep)
+    # where the time went: the host's cost per publish and what the leader's polls found
+    assert all(x["host_ns_per_publish"] > 0 and 0 < x["host_share_of_wall_in_publish"] <= 1 for x in sweep)
+    assert all(0 < x["leader_entries_per_poll"] <= 64 and x["leader_polls_per_us"] > 0 for x in sweep)
+    assert r["storm_64KiB"]["best"]["requests_per_s"] == max(x["requests_per_s"] for x in sweep)
+    assert 1 <= r["plugin_path"]["max_slots_at_gpu"] <= 16
     assert r["single_comm"]["value"] > 0 and r["plugin_path"]["payload_GBps"] > 0 and r["plain_copy_kernel"]["rw_GBps"] > 0
     assert sorted(r["other_configs"]) == ["config_1", "config_4", "config_5"]
     assert all(v["payload_GBps"] > 0 for v in r["other_configs"].values())

@@ -295,10 +295,102 @@ def test_engine_stream_depths(pkg, hip, oracle, depth, benchlib):
     e.destroy()
     got = dst_d.cpu().numpy()
     assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
-    # more than TCPXU_STREAM_MAX_DEPTH slots is refused before anything is launched
+    # beyond 128 slots in flight a slot holds 64 descriptors, and more than TCPXU_STREAM_MAX_DEPTH slots there are not:
+    # both refused before anything is launched
     e = Engine(pkg, hip)
     assert benchlib.tcpxuEngineRunTimed(e.h, items, 4, 0, 129, 1000, ctypes.byref(wall), ctypes.byref(kern), None) == pkg.INVALID_ARGUMENT
+    assert benchlib.tcpxuEngineRunTimed(e.h, items, 4, 0, 2049, 1000, ctypes.byref(wall), ctypes.byref(kern), None) == pkg.INVALID_ARGUMENT
     e.destroy()
+
+
+@pytest.mark.parametrize("depth", [256, 2048])
+def test_engine_storm_of_small_requests_many_in_flight(pkg, hip, oracle, depth, benchlib):
+    """The small-message storm with hundreds to 2048 requests in flight (the unpack queues of 128 comms): the
+    leader then fetches 64 submission entries per poll and turns runs of sixteen into tickets at a stroke, the host
+    publishes in batches.  Every request twice, byte-exact; every submission consumed by exactly one poll."""
+    import torch
+
+    wl = pkg.Workload(3, seed=0x5708A + depth, shrink=1)  # 1024 requests of 16 x 4 KiB, 256 MiB pool
+    info = wl.info
+    pool = np.empty(info.pool_bytes, dtype=np.uint8)
+    wl.fill_window(0, pool)
+    expect = oracle_expected(oracle, pool, wl.descs, int(info.dst_bytes))
+    pool_d = torch.from_numpy(pool).to("cuda:0")
+    dst_d = torch.full((expect.nbytes,), SENTINEL, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    descs = np.array(wl.descs, copy=True)
+    reqs = wl.requests
+    n = len(reqs)
+    items = (pkg.StreamItem * (2 * n))()
+    for i in range(2 * n):
+        r = reqs[i % n]
+        first, cnt = int(r["first_desc"]), int(r["n_descs"])
+        items[i].bounce_base = pool_d.data_ptr()
+        items[i].dst_base = dst_d.data_ptr() + GUARD  # descriptor offsets count from the start of the message
+        items[i].descs_host = descs.ctypes.data + 16 * first
+        items[i].n_descs = cnt
+        items[i].payload_bytes = int(r["bytes"])
+    e = Engine(pkg, hip)
+    print("engine storm case: depth=%d items=%d" % (depth, 2 * n), flush=True)
+    wall, kern = ctypes.c_double(), ctypes.c_double()
+    lat = (ctypes.c_double * (2 * n))()
+    pkg.check(benchlib.tcpxuEngineRunTimed(e.h, items, 2 * n, 0, depth, 20000, ctypes.byref(wall), ctypes.byref(kern), lat), "tcpxuEngineRunTimed")
+    stats, split = pkg.EngineStats(), pkg.StreamSplit()
+    pkg.check(hip.tcpxuEngineGetStats(e.h, ctypes.byref(stats)), "tcpxuEngineGetStats")
+    pkg.check(benchlib.tcpxuStreamLastSplit(ctypes.byref(split)), "tcpxuStreamLastSplit")
+    print("engine storm case: %.2f M requests/s, %d polls of which %d fetched 64 entries, %.0f ns of host time per publish"
+          % (2 * n / wall.value, stats.leader_polls, stats.leader_deep_polls, split.publish_ns / split.published), flush=True)  # fmt: skip
+    assert e.completed() == 2 * n and min(lat) > 0
+    assert stats.submissions == stats.leader_entries == 2 * n and stats.launches == 1
+    assert 0 < stats.leader_polls and stats.leader_deep_polls <= stats.leader_polls
+    assert split.published == 2 * n and split.publish_calls <= split.published and split.publish_ns < split.wall_ns
+    e.destroy()
+    got = dst_d.cpu().numpy()
+    assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
+
+
+def test_engine_submit_many(pkg, hip, oracle):
+    """tcpxuEngineSubmitMany: all submissions checked before any is queued; what the ring takes goes in under one
+    publish, in order, and the count comes back with "in progress" when that is not all."""
+    pool = np.random.default_rng(41).integers(0, 256, size=1 << 20, dtype=np.uint8)
+    rows = [((i * 4096 + 7 * i) % ((1 << 20) - 4096), 1 + (i * 997) % 4096, i * 4096) for i in range(160)]
+    descs = make_descs(rows)
+    expect = oracle_expected(oracle, pool, descs, 160 * 4096)
+    g = GpuBuffers(pool, descs, 160 * 4096)
+    m = Mapped(pkg, hip, descs, 40)
+    e = Engine(pkg, hip, ring_entries=16)
+    subs = (pkg.Submission * 40)()
+    for i in range(40):  # 40 submissions of 4 descriptors each
+        subs[i] = pkg.Submission(g.pool.data_ptr(), g.dst_base, m.desc_dev(4 * i), m.flag_dev(i), i + 1, 4, 0)
+    accepted = ctypes.c_uint32(99)
+    # one bad submission (no completion word) among good ones: nothing is queued
+    good = subs[3].done_flag_dev
+    subs[3].done_flag_dev = None
+    assert hip.tcpxuEngineSubmitMany(e.h, subs, 40, ctypes.byref(accepted)) == pkg.INVALID_ARGUMENT and accepted.value == 0
+    subs[3].done_flag_dev = good
+    assert hip.tcpxuEngineSubmitMany(e.h, subs, 0, ctypes.byref(accepted)) == pkg.SUCCESS and accepted.value == 0
+    # the engine is not started: a ring of 16 takes the first 16 and says so
+    assert hip.tcpxuEngineSubmitMany(e.h, subs, 40, ctypes.byref(accepted)) == pkg.IN_PROGRESS and accepted.value == 16
+    assert hip.tcpxuEngineSubmitMany(e.h, ctypes.byref(subs[16]), 24, ctypes.byref(accepted)) == pkg.IN_PROGRESS and accepted.value == 0
+    e.start()
+    at = 16
+    deadline = time.time() + 20
+    while at < 40:
+        rc = hip.tcpxuEngineSubmitMany(e.h, ctypes.byref(subs[at]), 40 - at, ctypes.byref(accepted))
+        assert rc in (pkg.SUCCESS, pkg.IN_PROGRESS), pkg.hip_layer().tcpxuLastError()
+        at += accepted.value
+        assert (rc == pkg.SUCCESS) == (at == 40)
+        assert time.time() < deadline, "the submission ring stayed full"
+    for i in range(40):
+        m.wait(i, i + 1)
+    e.stop()
+    stats = pkg.EngineStats()
+    pkg.check(hip.tcpxuEngineGetStats(e.h, ctypes.byref(stats)), "tcpxuEngineGetStats")
+    assert stats.submissions == stats.leader_entries == 40 and e.completed() == 40
+    got = g.result()
+    e.destroy()
+    m.free()
+    assert first_difference(got, expect) is None, repr(first_difference(got, expect))
 
 
 @pytest.mark.parametrize("hint", ["true", "none", "tiny", "huge"])
