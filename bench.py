@@ -411,7 +411,7 @@ def main():
     eff = pkg.EngineConfig()
     pkg.check(hip.tcpxuEngineGetConfig(engine, ctypes.byref(eff)), "tcpxuEngineGetConfig")
 
-    def run(items, depth, warmup_items=0, want_latency=False, timed_items=None):
+    def run(items, depth, warmup_items=0, want_latency=False, timed_items=None, engine=engine):
         """One launch of the engine over `items`.  With `timed_items`, the wall time is that of the timed items
         from completion to completion (the items after them only keep the queues full); otherwise from the publish
         of item `warmup_items` to the last completion."""
@@ -582,6 +582,48 @@ def main():
             "request_4MiB_1078_descs": {"p50": round(percentile(lat4m, 50), 2), "p99": round(percentile(lat4m, 99), 2)},
         }
         result["p50_request_us"] = result["latency_us"]["request_64KiB_16_descs"]["p50"]
+        # Where a lone request's time goes: the same two runs on a second engine that stamps the GPU's constant-rate
+        # clock at four points of every submission (the figures above come from the engine that does not).  The GPU's
+        # clock and the host's are not tied to each other, so the two crossings of PCIe -- the publish until the
+        # leader's poll has it, the completion word until the host's poll has it -- come out as one term: the request's
+        # whole time less what lies between the first and the last stamp.
+        stamped = ctypes.c_void_p()
+        pkg.check(hip.tcpxuEngineCreate(dev, ctypes.byref(cfg), ctypes.byref(stamped)), "tcpxuEngineCreate")
+        ticks_per_us = ctypes.c_double()
+        pkg.check(hip.tcpxuEngineEnableStamps(stamped, ctypes.byref(ticks_per_us)), "tcpxuEngineEnableStamps")
+
+        def budget(items, first):
+            n = len(items)
+            _, _, lat = run(items, 1, want_latency=True, engine=stamped)
+            raw = np.zeros(4 * n, dtype=np.uint64)
+            pkg.check(hip.tcpxuEngineReadStamps(stamped, first, n, raw.ctypes.data_as(ctypes.POINTER(ctypes.c_uint64))), "tcpxuEngineReadStamps")
+            t = raw.reshape(n, 4).astype(np.float64) / ticks_per_us.value
+            ok = (raw.reshape(n, 4) != np.uint64(0xFFFFFFFFFFFFFFFF)).all(axis=1)
+            t, total = t[ok], lat[ok]
+            on_gpu = t[:, 3] - t[:, 0]
+            med = lambda v: round(float(np.median(v)), 2)  # noqa: E731
+            return {
+                "p50_with_stamps": med(total),
+                "publish_to_leader_plus_completion_word_to_host": med(total - on_gpu),
+                "leader_saw_it_to_first_ticket_fetched": med(t[:, 1] - t[:, 0]),
+                "ticket_fetched_to_descriptors_staged": med(t[:, 2] - t[:, 1]),
+                "descriptors_staged_to_last_store_acknowledged": med(t[:, 3] - t[:, 2]),
+                "requests": int(ok.sum()),
+            }
+
+        b64k = budget(storm_items, 0)
+        b4m = budget(lat4m_items, n_storm)
+        empty = (pkg.StreamItem * 500)()  # no descriptors: the leader itself writes the completion word
+        for i in range(500):
+            empty[i].bounce_base, empty[i].dst_base, empty[i].descs_host, empty[i].n_descs = pool_d.data_ptr(), dst_base, sd.ctypes.data, 0
+        _, _, lat0 = run(empty, 1, want_latency=True, engine=stamped)
+        pkg.check(hip.tcpxuEngineDestroy(stamped), "tcpxuEngineDestroy")
+        result["latency_us"]["budget"] = {
+            "definition": "medians, microseconds, one request in flight; stamps of the GPU's %g MHz clock taken by the kernel" % ticks_per_us.value,
+            "request_64KiB_16_descs": b64k,
+            "request_4MiB_1078_descs": b4m,
+            "empty_submission_round_trip_p50": round(percentile(lat0, 50), 2),
+        }
         # The small-message storm: the 2048 requests of 64 KiB (16 fragments of 4 KiB each) sixteen times over, W of
         # them in flight, W x 16 = 64 .. 32768 descriptors with the engine at a time; W = 2048 is the workload's
         # "2048 concurrent requests" (the unpack queues of 128 comms).  The first 2048 are left out of the rate.

@@ -194,6 +194,17 @@ typedef struct tcpxuEngineStats {
 } tcpxuEngineStats;
 int tcpxuEngineGetStats(tcpxuEngine* engine, tcpxuEngineStats* stats);
 
+/* Where a submission's time goes inside the GPU, for measurement (no counterpart in the reference).  After
+ * tcpxuEngineEnableStamps (engine stopped; *ticks_per_us, may be NULL, receives the rate of the GPU's constant
+ * clock) the kernel keeps four readings of that clock per submission: [0] the leader saw its entry, [1] a
+ * workgroup had fetched the first of its tickets, [2] that workgroup had the ticket's descriptors staged, [3] the
+ * workgroup that completed it had its last store acknowledged.  tcpxuEngineReadStamps (engine stopped) copies the
+ * readings of submissions first_submission .. +n (counted from the engine's creation; n at most ring_entries, and
+ * only the last ring_entries submissions are kept) into out[4 * n] and clears them.  A reading of all ones means
+ * "never taken". */
+int tcpxuEngineEnableStamps(tcpxuEngine* engine, double* ticks_per_us);
+int tcpxuEngineReadStamps(tcpxuEngine* engine, uint64_t first_submission, uint32_t n, uint64_t* out);
+
 /* The configuration in effect (defaults resolved: actual grid size, ring size; ticket size 0 = by backlog). */
 int tcpxuEngineGetConfig(tcpxuEngine* engine, tcpxuEngineConfig* config);
 

@@ -209,6 +209,8 @@ _HIP_PROTOTYPES = {
     ),
     "tcpxuEngineCompleted": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint64)]),
     "tcpxuEngineSubmitMany": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(Submission), ctypes.c_uint32, ctypes.POINTER(ctypes.c_uint32)]),
+    "tcpxuEngineEnableStamps": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_double)]),
+    "tcpxuEngineReadStamps": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint32, ctypes.POINTER(ctypes.c_uint64)]),
     "tcpxuEngineGetStats": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(EngineStats)]),
     "tcpxuEngineRunning": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]),
     "tcpxuEngineGetConfig": (ctypes.c_int, [ctypes.c_void_p, ctypes.POINTER(EngineConfig)]),

@@ -248,8 +248,15 @@ __device__ __forceinline__ uint32_t lane_value(uint32_t v, uint32_t src_lane) {
   return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), static_cast<int>(src_lane)));
 }
 
+// Stamps (optional, tcpxuEngineEnableStamps): four 64-bit readings of the GPU's constant-rate clock per job slot, in
+// device memory that the host has filled with ones -- [0] the leader saw the submission, [1] the first of its
+// tickets was fetched by a workgroup, [2] the first workgroup had its descriptors staged (both kept as minima),
+// [3] the workgroup that completed the submission had its last store acknowledged.
+constexpr uint32_t kStampsPerJob = 4;
+__device__ __forceinline__ uint64_t clock_now() { return wall_clock64(); }
+
 __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uint32_t* job_target,
-                            uint32_t ring_mask, uint32_t fixed_per_ticket, uint32_t spin_limit) {
+                            uint32_t ring_mask, uint32_t fixed_per_ticket, uint32_t spin_limit, uint64_t* stamps) {
   // The leader's positions are the same in every lane: said outright, so that they stay in scalar registers (in
   // vector registers the compiler waits for the leader's own stores at the top of every pass).
   auto same_in_all_lanes = [](uint64_t v) {
@@ -379,6 +386,7 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
             out.y = v.n | (v.slot << 8) | kOnlyTicket;
             out.z = target;
             sys_store(&job_target[v.slot], target);
+            if (stamps) sys_store(&stamps[kStampsPerJob * v.slot], clock_now());
           }
           store_vec_sys(reinterpret_cast<uint8_t*>(&st->tickets[t & (kTicketRing - 1)]) + 16 * (lane & 3u), out);
         }
@@ -470,7 +478,10 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
               store_vec_sys(reinterpret_cast<uint8_t*>(&st->tickets[t & (kTicketRing - 1)]) + 16 * sector, v);
             }
           }
-          if (takes_part && sector == 3) sys_store(&job_target[slot], target);
+          if (takes_part && sector == 3) {
+            sys_store(&job_target[slot], target);
+            if (stamps) sys_store(&stamps[kStampsPerJob * slot], clock_now());
+          }
           tickets_out += static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(total)));
           consumed = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(run)));
         }
@@ -511,7 +522,10 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
         if (done_now != target_prev) break;
         if (static_cast<uint32_t>(tickets_out) + nt - tickets_done > kTicketRing) break;
         const uint32_t target = target_prev + nt;
-        if (lane == 0) sys_store(&job_target[slot], target);
+        if (lane == 0) {
+          sys_store(&job_target[slot], target);
+          if (stamps) sys_store(&stamps[kStampsPerJob * slot], clock_now());
+        }
         // Four neighbouring lanes write the four sectors of one ticket, so that one store instruction of the
         // wavefront fills 16 consecutive tickets (1 KiB of whole lines).  A ticket's sector differs from the entry's
         // in two places only, so every lane fetches the entry's sector of its own kind from the lane that holds it
@@ -659,6 +673,13 @@ struct Stage {
   RoundRec rec[kMaxDescsPerTicket];
 };
 
+// The stages live in LDS, and every access says so: through a plain pointer the compiler loses track of that and
+// reads the records with flat instructions (a 64-bit address in vector registers each, and slower).
+#define TCPXU_LDS __attribute__((address_space(3)))
+typedef TCPXU_LDS Stage LdsStage;
+typedef TCPXU_LDS uint32_t lds_u32;
+typedef TCPXU_LDS u32x4 lds_u32x4;
+
 __device__ __forceinline__ uint32_t lane_shift(uint32_t v, uint32_t from_lane) {
   return static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(static_cast<int>((from_lane & 63u) << 2), static_cast<int>(v)));
 }
@@ -666,8 +687,8 @@ __device__ __forceinline__ uint32_t lane_shift(uint32_t v, uint32_t from_lane) {
 // Fetcher: look once at the slot of ticket number `ticket` (one 64-byte read, with this workgroup's stop word in
 // the same round trip).  Returns 1 and stages the ticket if it is there.  Wave-uniform.
 template <typename State>
-__device__ uint32_t try_fetch_ticket(State* st, const uint32_t* stop_word, uint64_t ticket, Stage* stage,
-                                     uint32_t lane, bool* stop_up) {
+__device__ uint32_t try_fetch_ticket(State* st, const uint32_t* stop_word, uint64_t ticket, LdsStage* stage,
+                                     uint32_t lane, bool* stop_up, uint64_t* stamps) {
   const Record* rec = &st->tickets[ticket & (State::kTickets - 1)];
   const uint32_t expect = static_cast<uint32_t>(ticket + 1);
   uint32_t word = 0;
@@ -676,6 +697,7 @@ __device__ uint32_t try_fetch_ticket(State* st, const uint32_t* stop_word, uint6
   *stop_up = bcast(word, 16) != 0;
   const bool stamp_ok = (lane < 16 && (lane & 3) == 3) ? (word == expect) : true;
   if (!__all(stamp_ok)) return 0;
+  const uint64_t fetched_at = stamps ? clock_now() : 0;
   // Lane broadcasts need the whole wavefront: gather first, then let 12 lanes store.
   const uint32_t pl = lane < kPayloadWords ? lane : 0u;
   const uint32_t gathered = bcast(word, (pl / 3) * 4 + (pl % 3));
@@ -752,7 +774,18 @@ __device__ uint32_t try_fetch_ticket(State* st, const uint32_t* stop_word, uint6
     r.nvec = plan.nvec;
     r.bits = plan.head | (plan.tail << 8) | (share_next ? 1u << 16 : 0u) | (kind << 24);
     r.pad = 0;
-    stage->rec[lane] = r;
+    lds_u32x4* out = reinterpret_cast<lds_u32x4*>(&stage->rec[lane]);
+    out[0] = u32x4{r.src_lo, r.src_hi, r.dst_lo, r.dst_hi};
+    out[1] = u32x4{r.next_lo, r.next_hi, r.start_off, r.end_off};
+    out[2] = u32x4{r.len, r.nvec, r.bits, r.pad};
+  }
+  if (stamps) {
+    const uint32_t job = (ticket_bits >> 8) & 0xFFFFu;
+    const uint64_t staged_at = clock_now();
+    if (lane == 0) {
+      __hip_atomic_fetch_min(&stamps[kStampsPerJob * job + 1], fetched_at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_fetch_min(&stamps[kStampsPerJob * job + 2], staged_at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
   }
   return 1;
 }
@@ -760,7 +793,7 @@ __device__ uint32_t try_fetch_ticket(State* st, const uint32_t* stop_word, uint6
 // Counts a finished ticket (all of its payload is in memory); the last ticket of a submission publishes the
 // completion word.
 template <typename State>
-__device__ void retire_ticket(State* st, uint32_t* jobs_done, const Stage* stage, uint32_t lane) {
+__device__ void retire_ticket(State* st, uint32_t* jobs_done, const LdsStage* stage, uint32_t lane, uint64_t* stamps) {
   if (lane == 0) {
     const uint32_t job = (stage->payload[10] >> 8) & 0xFFFFu;
     const uint32_t target = stage->payload[11];
@@ -769,6 +802,7 @@ __device__ void retire_ticket(State* st, uint32_t* jobs_done, const Stage* stage
     if ((stage->payload[10] & kOnlyTicket) != 0) {
       // The submission's only ticket completes it: tell the caller first, count afterwards (nobody waits for the
       // counts' round trips; the leader reads them when it wants the job slot again).
+      if (stamps) sys_store(&stamps[kStampsPerJob * job + 3], clock_now());
       sys_store(reinterpret_cast<uint64_t*>(done_flag), done_value);
       __hip_atomic_fetch_add(&jobs_done[job], 1u, __ATOMIC_RELAXED, SYS);
       __hip_atomic_fetch_add(&st->tickets_done, 1ull, __ATOMIC_RELAXED, SYS);
@@ -779,6 +813,7 @@ __device__ void retire_ticket(State* st, uint32_t* jobs_done, const Stage* stage
     __hip_atomic_fetch_add(&st->tickets_done, 1ull, __ATOMIC_RELAXED, SYS);
     if (count == target) {
       // Every other ticket's payload was in memory before it was counted, and so is this one's.
+      if (stamps) sys_store(&stamps[kStampsPerJob * job + 3], clock_now());
       sys_store(reinterpret_cast<uint64_t*>(done_flag), done_value);
       __hip_atomic_fetch_add(&st->jobs_completed, 1ull, __ATOMIC_RELAXED, SYS);
     }
@@ -789,7 +824,7 @@ __device__ void retire_ticket(State* st, uint32_t* jobs_done, const Stage* stage
 // ticket, rounded up), one round (at most 4 KiB) in flight at a time.  A wavefront that writes one contiguous
 // stretch of the destination after another measured about 1 % faster end to end than fragments dealt out in turn
 // (wave, wave + kCopyWaves, ...).
-__device__ void copy_ticket(const Stage* stage, uint32_t wave, uint32_t lane, uint32_t* waves_on_last) {
+__device__ void copy_ticket(const LdsStage* stage, uint32_t wave, uint32_t lane, lds_u32* waves_on_last) {
   auto uniform = [](uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(v)); };
   wave = uniform(wave);
   const uint32_t n = uniform(stage->payload[10]) & 0xFFu;
@@ -817,7 +852,7 @@ __device__ void copy_ticket(const Stage* stage, uint32_t wave, uint32_t lane, ui
       return true;
     }
     while (j < end) {
-      const u32x4* words = reinterpret_cast<const u32x4*>(&stage->rec[j]);
+      const lds_u32x4* words = reinterpret_cast<const lds_u32x4*>(&stage->rec[j]);
       const u32x4 w0 = words[0], w1 = words[1], w2 = words[2];
       ++j;
       if (j >= end) on_last_fragment();
@@ -862,7 +897,7 @@ __device__ void copy_ticket(const Stage* stage, uint32_t wave, uint32_t lane, ui
 // which the workgroup gives up (0 = never, the engine's workers wait for the leader as long as it lives).
 template <typename State>
 __device__ void worker_loop(State* st, uint32_t* jobs_done, uint32_t flags, uint64_t ticket_limit,
-                            uint32_t look_limit) {
+                            uint32_t look_limit, uint64_t* stamps) {
   __shared__ Stage stages[2];
   __shared__ uint32_t s_waves_done;  // copy wavefronts that have finished (and drained) a ticket, running total
   __shared__ uint32_t s_waves_on_last;  // copy wavefronts that have turned to their last fragment of a ticket, ditto
@@ -894,7 +929,7 @@ __device__ void worker_loop(State* st, uint32_t* jobs_done, uint32_t flags, uint
     const uint32_t* const claim_gate = (flags & 2u) != 0 ? &s_waves_on_last : &s_waves_done;
     const uint32_t backoff_cap = (flags >> 8) & 0xFFu;
     for (;;) {
-      Stage* next = &stages[staged & 1];
+      LdsStage* next = (LdsStage*)&stages[staged & 1];
       if (!eager) {
         // Wait for the copy of ticket staged-1 to finish (LDS only: no memory traffic while waiting).
         while (__hip_atomic_load(claim_gate, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != staged * kCopyWaves)
@@ -907,7 +942,7 @@ __device__ void worker_loop(State* st, uint32_t* jobs_done, uint32_t flags, uint
       uint32_t backoff = 1, looks = 0;
       for (;;) {
         bool stop_up = false;
-        if (ticket < ticket_limit && try_fetch_ticket(st, stop_word, ticket, next, lane, &stop_up)) {
+        if (ticket < ticket_limit && try_fetch_ticket(st, stop_word, ticket, next, lane, &stop_up, stamps)) {
           eager = first_look && allow_eager;
           break;
         }
@@ -941,15 +976,15 @@ __device__ void worker_loop(State* st, uint32_t* jobs_done, uint32_t flags, uint
     // ---- copy wavefronts ----
     for (uint32_t i = 0;; ++i) {
       __syncthreads();  // stage i&1 is ready
-      const Stage* stage = &stages[i & 1];
+      LdsStage* stage = (LdsStage*)&stages[i & 1];
       if (stage->go == 0) break;
-      copy_ticket(stage, wave, lane, &s_waves_on_last);
+      copy_ticket(stage, wave, lane, (lds_u32*)&s_waves_on_last);
       drain_memory_ops();  // this wavefront's write-through stores are acknowledged
       uint32_t arrived = 0;
       if (lane == 0)
         arrived = __hip_atomic_fetch_add(&s_waves_done, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) + 1u;
       // The wavefront that finishes last counts the ticket: every wavefront's payload is in memory by then.
-      if (bcast(arrived, 0) == (i + 1) * kCopyWaves) retire_ticket(st, jobs_done, stage, lane);
+      if (bcast(arrived, 0) == (i + 1) * kCopyWaves) retire_ticket(st, jobs_done, stage, lane, stamps);
     }
   }
 }
@@ -957,11 +992,11 @@ __device__ void worker_loop(State* st, uint32_t* jobs_done, uint32_t flags, uint
 __global__ __launch_bounds__(kEngineThreads) __attribute__((amdgpu_waves_per_eu(6))) void unpack_engine_kernel(HostCtl* ctl, DevState* st, uint32_t* jobs_done,
                                                                    uint32_t* job_target, uint32_t ring_mask,
                                                                    uint32_t per_ticket, uint32_t spin_limit,
-                                                                   uint32_t flags) {
+                                                                   uint32_t flags, uint64_t* stamps) {
   if (blockIdx.x == 0) {
-    if (threadIdx.x < kWaveLanes) leader_loop(ctl, st, jobs_done, job_target, ring_mask, per_ticket, spin_limit);
+    if (threadIdx.x < kWaveLanes) leader_loop(ctl, st, jobs_done, job_target, ring_mask, per_ticket, spin_limit, stamps);
   } else {
-    worker_loop(st, jobs_done, flags, ~0ull, 0u);
+    worker_loop(st, jobs_done, flags, ~0ull, 0u, stamps);
   }
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -1021,7 +1056,7 @@ __global__ __launch_bounds__(kOneShotTickets) void oneshot_prepare_kernel(OneSho
 // look finds each; the look limit only keeps a misuse (two calls overlapping on one GPU) from spinning for ever.
 __global__ __launch_bounds__(kEngineThreads) void unpack_oneshot_kernel(OneShotState* st, uint32_t flags,
                                                                     uint32_t n_tickets) {
-  worker_loop(st, st->jobs_done, flags, n_tickets, 1u << 16);
+  worker_loop(st, st->jobs_done, flags, n_tickets, 1u << 16, nullptr);
 }
 
 }  // namespace
@@ -1048,6 +1083,7 @@ struct tcpxuEngine {
   bool failed = false;    // the kernel stopped answering (see tcpxuEngineSubmitSized); nothing more is accepted
   uint64_t launches = 0;
   uint64_t submissions = 0;
+  uint64_t* stamps = nullptr;  // device memory, kStampsPerJob per ring entry, or null (tcpxuEngineEnableStamps)
   std::mutex mu;
 };
 
@@ -1202,7 +1238,7 @@ static int launch_locked(tcpxuEngine* e) {
   std::atomic_thread_fence(std::memory_order_seq_cst);
   TCPXU_HIP(hipEventRecord(e->ev_start, e->stream));
   hipLaunchKernelGGL(unpack_engine_kernel, dim3(e->workgroups), dim3(kEngineThreads), 0, e->stream, e->ctl_dev, e->st,
-                     e->jobs_done, e->job_target, e->ring_entries - 1, e->per_ticket, e->spin_limit, e->flags);
+                     e->jobs_done, e->job_target, e->ring_entries - 1, e->per_ticket, e->spin_limit, e->flags, e->stamps);
   TCPXU_HIP(hipGetLastError());
   TCPXU_HIP(hipEventRecord(e->ev_stop, e->stream));
   e->launched = true;
@@ -1268,6 +1304,7 @@ int tcpxuEngineDestroy(tcpxuEngine* e) {
   if (e->ev_stop) (void)hipEventDestroy(e->ev_stop);
   if (e->stream) (void)hipStreamDestroy(e->stream);
   if (e->st) (void)hipFree(e->st);
+  if (e->stamps) (void)hipFree(e->stamps);
   if (e->ctl) (void)hipHostFree(e->ctl);
   delete e;
   return TCPXU_SUCCESS;
@@ -1377,6 +1414,48 @@ int tcpxuEngineSubmitMany(tcpxuEngine* e, const tcpxuSubmission* subs, uint32_t 
     if (host_load(&e->ctl->exited) == 2) TCPXU_TRY(launch_locked(e));  // it left by itself: bring it back
   }
   return take == n ? TCPXU_SUCCESS : kTcpxuInProgress;
+}
+
+int tcpxuEngineEnableStamps(tcpxuEngine* e, double* ticks_per_us) {
+  if (!e) return TCPXU_INVALID_ARGUMENT;
+  std::lock_guard<std::mutex> lock(e->mu);
+  if (e->launched) {
+    set_error("stamps are switched on while the engine is stopped");
+    return TCPXU_INVALID_USAGE;
+  }
+  DeviceScope scope(e->device);
+  TCPXU_TRY(scope.rc());
+  const size_t bytes = sizeof(uint64_t) * kStampsPerJob * e->ring_entries;
+  if (!e->stamps) TCPXU_HIP(hipMalloc(reinterpret_cast<void**>(&e->stamps), bytes));
+  TCPXU_HIP(hipMemset(e->stamps, 0xFF, bytes));
+  if (ticks_per_us) {
+    int khz = 0;
+    TCPXU_HIP(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, e->device));
+    *ticks_per_us = khz / 1000.0;
+  }
+  return TCPXU_SUCCESS;
+}
+
+int tcpxuEngineReadStamps(tcpxuEngine* e, uint64_t first_submission, uint32_t n, uint64_t* out) {
+  if (!e || !out || n > e->ring_entries) {
+    set_error("stamps: at most ring_entries submissions at a time");
+    return TCPXU_INVALID_ARGUMENT;
+  }
+  std::lock_guard<std::mutex> lock(e->mu);
+  if (!e->stamps || e->launched) {
+    set_error("stamps are read while the engine is stopped, after tcpxuEngineEnableStamps");
+    return TCPXU_INVALID_USAGE;
+  }
+  DeviceScope scope(e->device);
+  TCPXU_TRY(scope.rc());
+  std::vector<uint64_t> all(static_cast<size_t>(kStampsPerJob) * e->ring_entries);
+  TCPXU_HIP(hipMemcpy(all.data(), e->stamps, all.size() * sizeof(uint64_t), hipMemcpyDeviceToHost));
+  for (uint32_t i = 0; i < n; ++i) {
+    const size_t slot = (first_submission + i) & (e->ring_entries - 1);
+    for (uint32_t k = 0; k < kStampsPerJob; ++k) out[kStampsPerJob * i + k] = all[kStampsPerJob * slot + k];
+  }
+  TCPXU_HIP(hipMemset(e->stamps, 0xFF, all.size() * sizeof(uint64_t)));  // the minima start from ones again
+  return TCPXU_SUCCESS;
 }
 
 int tcpxuEngineGetStats(tcpxuEngine* e, tcpxuEngineStats* stats) {

@@ -906,3 +906,48 @@ def test_engine_lines_shared_across_the_ends_of_tickets(pkg, hip, oracle, per_ti
     e.destroy()
     m.free()
     assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
+
+
+def test_engine_stamps_order_the_stages_of_a_submission(pkg, hip, oracle):
+    """With stamps switched on the kernel records when the leader saw a submission, when its first ticket was
+    fetched, when that ticket's descriptors were staged and when its last store was acknowledged: four readings of
+    one clock, in that order, for single-ticket, multi-ticket and empty-descriptor submissions alike; the bytes are
+    the oracle's as ever."""
+    wl = pkg.Workload(2, seed=0x57A3, shrink=2)  # 2 MiB in two requests of about 270 descriptors
+    info = wl.info
+    pool = np.empty(info.pool_bytes, dtype=np.uint8)
+    wl.fill_window(0, pool)
+    expect = oracle_expected(oracle, pool, wl.descs, info.dst_bytes)
+    g = GpuBuffers(pool, wl.descs, info.dst_bytes)
+    m = Mapped(pkg, hip, np.ascontiguousarray(wl.descs), 8)
+    e = Engine(pkg, hip)
+    rate = ctypes.c_double()
+    pkg.check(hip.tcpxuEngineEnableStamps(e.h, ctypes.byref(rate)), "tcpxuEngineEnableStamps")
+    assert 1.0 <= rate.value <= 10000.0
+    out = (ctypes.c_uint64 * 32)()
+    e.start()
+    assert hip.tcpxuEngineReadStamps(e.h, 0, 1, out) == pkg.INVALID_USAGE  # only while stopped
+    subs = []
+    for i, r in enumerate(wl.requests):  # whole requests: many tickets each
+        subs.append((int(r["first_desc"]), int(r["n_descs"])))
+    first, n = subs[0]
+    subs += [(first, 5), (first + 5, 3)]  # and two that fit one ticket
+    for i, (f, cnt) in enumerate(subs):
+        e.submit(g.pool.data_ptr(), g.dst_base, m.desc_dev(f), cnt, m.flag_dev(i), i + 1)
+        m.wait(i, i + 1)
+    e.stop()
+    pkg.check(hip.tcpxuEngineReadStamps(e.h, 0, len(subs), out), "tcpxuEngineReadStamps")
+    never = 0xFFFFFFFFFFFFFFFF
+    for i in range(len(subs)):
+        t = [out[4 * i + k] for k in range(4)]
+        assert never not in t, (i, t)
+        assert t[0] <= t[1] <= t[2] <= t[3], (i, t)
+        assert (t[3] - t[0]) / rate.value < 1e6, "a small submission takes microseconds, not a second"
+        if i:
+            assert t[0] >= out[4 * (i - 1) + 3], "one at a time: a submission is seen after the one before it completed"
+    pkg.check(hip.tcpxuEngineReadStamps(e.h, 0, len(subs), out), "tcpxuEngineReadStamps")
+    assert all(out[k] == never for k in range(4 * len(subs))), "reading clears the stamps"
+    got = g.result()
+    e.destroy()
+    m.free()
+    assert first_difference(got, expect) is None, repr(first_difference(got, expect))
