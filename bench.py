@@ -491,6 +491,9 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "steps_run": steps_per_launch,  # what the launch carried: fill_steps + windows x steps + the tail
+        "fill_steps": fill_steps,
+        "windows": windows,
         "ms_per_step": round(wall_us / 1000.0 / args.steps, 6),
         "higher_is_better": True,
         "scaling": "weak",
@@ -516,7 +519,7 @@ def main():
             "device": name.value.decode(),
             "compute_units": cus.value,
             "engine_workgroups": eff.workgroups,
-            "descs_per_ticket": eff.descs_per_ticket if eff.descs_per_ticket else "8..16 by backlog (a submission of at most 32 stays whole; up to 64 for short fragments)",
+            "descs_per_ticket": eff.descs_per_ticket if eff.descs_per_ticket else "8, 12, 14 or 16 by backlog (a submission of at most 32 stays whole; 32, 48 or 64 for short fragments)",
         },
         "roofline": {
             "bound": "hbm",
@@ -535,6 +538,9 @@ def main():
         },
         "window_ms": {
             "median": round(wall_us / 1000.0, 6),
+            "mean": round(float(np.mean(window_us)) / 1000.0, 6),
+            # every timed step over all the timed time: nothing dropped, slow windows included
+            "value_over_all_windows_GBps": round(payload * windows / (float(np.sum(window_us)) * 1e-6) / 1e9, 2),
             "p10": round(percentile(window_us, 10) / 1000.0, 6),
             "p90": round(percentile(window_us, 90) / 1000.0, 6),
             "windows": windows,

@@ -115,9 +115,10 @@ typedef struct tcpxuEngineConfig {
   uint32_t workgroups;      /* persistent grid size, 0 = two worker workgroups per compute unit + the leader */
   uint32_t descs_per_ticket;/* descriptors one workgroup takes at a time (1..64); 0 = chosen per submission from
                                the backlog of descriptors not yet unpacked: 8 when the engine is idle (lowest
-                               latency), 12, then 16 when every workgroup has work queued (highest throughput), and
-                               with a payload hint that tells of short fragments 32, 48 or 64;
-                               a submission of at most 32 descriptors stays whole once 8 or more are in flight */
+                               latency), 12, then 14 while the backlog is there but shallow (below 100 descriptors
+                               per workgroup), 16 when it is deep (highest throughput), and with a payload hint that
+                               tells of short fragments 32, 48 or 64; a submission of at most 32 descriptors stays
+                               whole once 8 or more are in flight (tcpxuEngineTicketPlan gives the same answers) */
   uint32_t spin_limit;      /* the kernel leaves by itself after this many consecutive empty polls of the ring
                                (about 1.2 us each) and is launched again by the next submission, so that a
                                device-wide synchronize never waits on an idle engine; 0 = default (400, about
@@ -227,7 +228,12 @@ int tcpxuEngineRunning(tcpxuEngine* engine, int* running);
  * ticket cursor and done counters live in a fixed array of device memory inside the library (17 KiB, held by
  * every GPU the library runs on until the process ends), which every call on a GPU shares and which each call
  * clears with its own first kernel.  Calls that overlap on one GPU (two streams, two threads) race on that
- * array: issue them on one stream, or order them otherwise. */
+ * array: issue them on one stream, or order them otherwise.  (A workgroup that finds its ticket overwritten by
+ * such a race gives up after 65536 looks and stores the complement of `done_value` to the completion word, so that
+ * a poller is not left waiting; the slot's bytes are then not all there.)
+ * Under HIP graph capture: make one ordinary call on the device first -- it looks up the array's address and loads
+ * the kernels' code, which do not belong under capture -- then capture; a replay launches the same two kernels
+ * with the same arguments. */
 int tcpxuUnpackSlotNoAlloc(int device, const void* bounce_base, void* dst_base, const void* descs_dev,
                            uint32_t n_descs, void* done_flag_dev, uint64_t done_value, void* stream);
 

@@ -40,6 +40,7 @@
 #include <mutex>
 #include <new>
 #include <thread>
+#include <type_traits>
 #include <vector>
 
 #include "hip_common.h"
@@ -88,7 +89,8 @@ __host__ __device__ __forceinline__ uint32_t tickets_for(uint32_t n, uint32_t pe
 // at 8 in flight, 17.5 -> 9.3 us at 32, where the leader's loop had become the queue.)
 //
 // `bytes` is the submission's payload if the caller said (0 = unknown: whole pages).  The largest step, 16, stands
-// for whole pages: a submission of shorter fragments gets more descriptors per ticket, in multiples of 16 so that
+// for whole pages (14 while the backlog is shallow, see below: seven copy wavefronts then get two fragments each and
+// one gets none); a submission of shorter fragments gets more descriptors per ticket, in multiples of 16 so that
 // the copy wavefronts' shares come out even, up to 64 (full_ticket_size).  Written as comparisons: the leader runs
 // this for every submission and a division costs it forty instructions.
 constexpr uint32_t kManyInFlight = 8, kSmallSubmission = 32;
@@ -217,6 +219,9 @@ struct OneShotState {
   alignas(64) uint64_t jobs_completed;
   alignas(64) uint32_t jobs_done[16];  // [0]: tickets of the slot counted so far
   alignas(64) uint64_t unused_flag;    // completion word of a caller that passed none
+  // The call's completion word and value, for a workgroup that gives up (see worker_loop's look limit): it cannot
+  // have them from a ticket, because a ticket is what it did not find.
+  uint64_t flag_addr, flag_value;
   alignas(256) StopWord stop[kStops];
   alignas(64) Record tickets[kOneShotTickets];
 };
@@ -947,6 +952,13 @@ __device__ void worker_loop(State* st, uint32_t* jobs_done, uint32_t flags, uint
           break;
         }
         if (ticket >= ticket_limit || (look_limit != 0 && ++looks >= look_limit)) {
+          if constexpr (std::is_same<State, OneShotState>::value) {
+            // A ticket that exists and never shows up: two calls overlapped on one GPU and overwrote each other's
+            // tickets.  The slot cannot be completed; whoever polls its completion word is told so with the
+            // complement of the value it waits for, rather than left waiting.
+            if (ticket < ticket_limit && lane == 0)
+              sys_store(reinterpret_cast<uint64_t*>(sys_load(&st->flag_addr)), ~sys_load(&st->flag_value));
+          }
           give_up = true;
           if (lane == 0) next->go = 0;
           break;
@@ -1033,6 +1045,8 @@ __global__ __launch_bounds__(kOneShotTickets) void oneshot_prepare_kernel(OneSho
     sys_store(&st->jobs_completed, static_cast<uint64_t>(0));
     sys_store(&st->jobs_done[0], 0u);
     sys_store(&st->stop[0].value, 0u);
+    sys_store(&st->flag_addr, done_flag);
+    sys_store(&st->flag_value, done_value);
     if (n_descs == 0) sys_store(reinterpret_cast<uint64_t*>(done_flag), done_value);
   }
   const uint32_t nt = (n_descs + kOneShotTicketSize - 1) / kOneShotTicketSize;

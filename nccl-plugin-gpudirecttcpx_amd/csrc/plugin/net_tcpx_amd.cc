@@ -133,8 +133,8 @@ void parse_device_type() {
 // NCCL_GPUDIRECTTCPX_RX_BINDINGS: the CPUs a receive comm's socket thread may run on, per network device, in the
 // reference's syntax "name:lo-hi,lo-hi;name:lo-hi" (parseCoreRanges, src/common.cc:65-130; the names are the ones
 // getProperties reports).  A device that is not named keeps the CPUs the process may use (the reference's default is
-// the NIC's NUMA node, src/net_tcpx.cc:592-611; a synthetic device has none).  A malformed entry is reported and
-// skipped, as there.  Called once the device names exist.
+// the NIC's NUMA node, src/net_tcpx.cc:592-611; a synthetic device has none).  A malformed range is reported and
+// skipped and the device's other ranges stand, as there (src/common.cc:104-108).  Called once the device names exist.
 void parse_rx_bindings() {
   for (int d = 0; d < kMaxDevices; ++d) {
     CPU_ZERO(&g.rx_cpus[d]);
@@ -163,9 +163,8 @@ void parse_rx_bindings() {
     }
     cpu_set_t set;
     CPU_ZERO(&set);
-    bool ok = true;
     size_t r = colon + 1;
-    while (ok && r <= phrase.size()) {
+    while (r <= phrase.size()) {
       size_t comma = phrase.find(',', r);
       if (comma == std::string::npos) comma = phrase.size();
       const std::string range = phrase.substr(r, comma - r);
@@ -174,12 +173,11 @@ void parse_rx_bindings() {
       char tail = 0;
       if (sscanf(range.c_str(), "%d-%d%c", &lo, &hi, &tail) != 2 || lo < 0 || hi < lo || hi >= CPU_SETSIZE) {
         WARN("invalid range %s", range.c_str());
-        ok = false;
-        break;
+        continue;  // this range only
       }
       for (int c = lo; c <= hi; ++c) CPU_SET(c, &set);
     }
-    if (!ok || CPU_COUNT(&set) == 0) continue;
+    if (CPU_COUNT(&set) == 0) continue;  // nothing valid was named: the device stays unbound
     g.rx_cpus[dev] = set;
     g.rx_bound[dev] = true;
   }
@@ -869,8 +867,12 @@ ncclResult_t tcpxAccept_v5(void* listenComm, void** recvComm, ncclNetDeviceHandl
     return ncclInternalError;
   }
   Comm* c = nullptr;
-  TCPXCHECK(new_comm(l->dev, true, &c));
-  ncclResult_t rc = g.device_type == kDeviceHost ? ensure_engine(ds) : ncclSuccess;
+  ncclResult_t rc = new_comm(l->dev, true, &c);
+  if (rc != ncclSuccess) {
+    l->backlog.fetch_add(1, std::memory_order_release);  // the connection stays in the backlog
+    return rc;
+  }
+  rc = g.device_type == kDeviceHost ? ensure_engine(ds) : ncclSuccess;
   if (rc == ncclSuccess) rc = unpack_queue_new(l->dev, true, &c->queue);  // tcpxGetDeviceHandle, src/net_tcpx.cc:1452-1471
   if (rc != ncclSuccess) {
     delete c;

@@ -652,6 +652,10 @@ def test_socket_thread_binding():
         assert cpus("tcpx-amd-synth0:%d-%d,%d-%d" % (lo, lo, hi, hi)) == [2]
     assert cpus("eth9:0-1") == [len(allowed)]  # another device's
     assert cpus("tcpx-amd-synth0:%d" % one) == [len(allowed)]  # no upper end: invalid, as in the reference
+    # an invalid range is skipped on its own and the device's other ranges stand (src/common.cc:104-108); so does a
+    # trailing comma
+    assert cpus("tcpx-amd-synth0:%d,%d-%d" % (one, one, one)) == [1]
+    assert cpus("tcpx-amd-synth0:%d-%d,bogus," % (one, one)) == [1]
     assert cpus("tcpx-amd-synth0:%d-%d" % (one, one), helper="0") == [0]  # no socket thread
 
 

@@ -83,6 +83,51 @@ def test_two_calls_in_a_row_match_the_engine(pkg, hip, oracle, config, seed, shr
     mapped.free()
 
 
+def test_two_calls_captured_into_a_hip_graph_and_replayed(pkg, hip, oracle):
+    """What the entry point is for: after one ordinary call (which looks up the scratch memory's address and loads the
+    kernels' code, neither of which belongs under capture), two calls in a row -- a large slot, then a smaller one --
+    are captured into a HIP graph on a caller's stream and replayed; every replay, with the pool refilled, the
+    destination reset and the completion words cleared by ordinary eager work in between, must give the oracle's
+    bytes for the pool of that replay."""
+    import torch
+
+    wl, pool = slots_of(pkg, 2, 0xA110F, shrink=0)
+    info = wl.info
+    reqs = [(int(r["first_desc"]), int(r["n_descs"])) for r in wl.requests]
+    big = max(reqs, key=lambda r: r[1])
+    other = next(r for r in reqs if r != big)
+    slots = [big, (other[0], max(1, other[1] // 3))]
+    descs = np.ascontiguousarray(wl.descs)
+    used = np.concatenate([descs[f : f + n] for f, n in slots])
+    buf = GpuBuffers(pool, descs, info.dst_bytes, info.dst_misalign)
+    mapped = Mapped(pkg, hip, descs, len(slots))
+    stream = torch.cuda.Stream()
+    # the warm call, not captured
+    pkg.check(hip.tcpxuUnpackSlotNoAlloc(0, buf.pool.data_ptr(), buf.dst_base, mapped.desc_dev(slots[1][0]), slots[1][1], mapped.flag_dev(1), 7, stream.cuda_stream), "tcpxuUnpackSlotNoAlloc")
+    torch.cuda.synchronize()
+    assert int(mapped.flags[1]) == 7
+    graph = torch.cuda.CUDAGraph()
+    print("no-alloc graph case: slots of %d and %d descriptors captured" % (slots[0][1], slots[1][1]), flush=True)
+    with torch.cuda.graph(graph, stream=stream):
+        s = torch.cuda.current_stream().cuda_stream
+        for i, (first, n) in enumerate(slots):
+            pkg.check(hip.tcpxuUnpackSlotNoAlloc(0, buf.pool.data_ptr(), buf.dst_base, mapped.desc_dev(first), n, mapped.flag_dev(i), 1000 + i, ctypes.c_void_p(s)), "tcpxuUnpackSlotNoAlloc")
+    for replay in range(3):
+        if replay:
+            pool = np.roll(pool, 4099 * replay) ^ np.uint8(replay)
+            buf.pool.copy_(torch.from_numpy(pool))
+        buf.reset()
+        for i in range(len(slots)):
+            mapped.flags[i] = 0
+        graph.replay()
+        torch.cuda.synchronize()
+        expect = oracle_expected(oracle, pool, used, info.dst_bytes, info.dst_misalign)
+        got = buf.result()
+        assert [int(mapped.flags[i]) for i in range(len(slots))] == [1000, 1001], "replay %d" % replay
+        assert first_difference(got, expect) is None, "replay %d, first (index, got, want, count): %r" % (replay, first_difference(got, expect))
+    mapped.free()
+
+
 def test_no_completion_word_and_the_default_stream(pkg, hip, oracle):
     """Without a completion word stream order is the only signal; the scratch memory then takes the store."""
     wl, pool = slots_of(pkg, 1, 0xA110E, shrink=2)
