@@ -349,12 +349,13 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
     // each (it fetches an entry's words from their lanes into scalars first: about half a microsecond) capped a
     // stream of 1 MiB requests at 2 M/s and a storm of 64 KiB requests at 1.6 M/s.  Taken when the run has some
     // width: a lone entry of many tickets is written faster by the loop below, sixteen tickets to the instruction.
-    // (Not for a lone entry of more descriptors than a ticket holds, nor for a first entry of more than 32 full
-    // tickets: nothing here would apply to them, and what is worked out per lane first would only add to their
-    // latency.)
+    // (Not for a lone entry of more descriptors than a ticket holds, nor for a first entry of more than 32 tickets of
+    // the size its payload asks for -- 512 whole pages, up to 2048 short fragments: nothing here would apply to
+    // them, and what is worked out per lane first would only add to their latency.)
     uint32_t consumed = 0;
     bool deep_next = false;
     const uint32_t n_first = lane_value(sect.y, 3);
+    const uint32_t lane_tickets_hold = kLaneTickets * (fixed_per_ticket != 0 ? fixed_per_ticket : full_ticket_size(lane_value(sect.z, 3), n_first));
     // What the four lanes of an entry know about it, for the sixteen entries of one group at once.
     struct EntryView {
       uint32_t n, bytes, per_ticket, target_prev, in_flight, slot;
@@ -400,7 +401,7 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
       return run;
     };
     if ((ok_mask & 0xFull) == 0xFull &&  // entry s is there
-        (n_first <= kMaxDescsPerTicket || (ready >= 2 && n_first <= kLaneTickets * kFullTicket))) {
+        (n_first <= kMaxDescsPerTicket || (ready >= 2 && n_first <= lane_tickets_hold))) {
       const EntryView ev = view_entries(sect, aux, s, ok_mask);
       const uint32_t n = ev.n, bytes = ev.bytes, per_ticket = ev.per_ticket, target_prev = ev.target_prev;
       const uint32_t in_flight = ev.in_flight, slot = ev.slot;
@@ -829,7 +830,7 @@ __device__ void retire_ticket(State* st, uint32_t* jobs_done, const LdsStage* st
 // ticket, rounded up), one round (at most 4 KiB) in flight at a time.  A wavefront that writes one contiguous
 // stretch of the destination after another measured about 1 % faster end to end than fragments dealt out in turn
 // (wave, wave + kCopyWaves, ...).
-__device__ void copy_ticket(const LdsStage* stage, uint32_t wave, uint32_t lane, lds_u32* waves_on_last) {
+__device__ __forceinline__ void copy_ticket(const LdsStage* stage, uint32_t wave, uint32_t lane, lds_u32* waves_on_last) {
   auto uniform = [](uint32_t v) { return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(v)); };
   wave = uniform(wave);
   const uint32_t n = uniform(stage->payload[10]) & 0xFFu;

@@ -873,6 +873,48 @@ def test_engine_many_mid_size_submissions_waiting_at_once(pkg, hip, oracle, per_
     assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
 
 
+@pytest.mark.parametrize("mean_len", [700, 1500, 2300])
+def test_engine_queued_submissions_of_short_fragments_with_the_payload_given(pkg, hip, oracle, mean_len):
+    """Forty submissions of 600 to 2048 short fragments each, every one with its byte count, all queued before the
+    kernel is launched: the payload asks for tickets of 64, 48 or 32 descriptors, so a submission is at most 32
+    tickets and the leader's lanes write the tickets of the whole run of entries they hold (up to 2048 descriptors
+    each, where without the byte count it is 512)."""
+    from test_unpack_gpu import seeded_pool
+
+    rng = np.random.default_rng(4000 + mean_len)
+    pool = seeded_pool(1 << 20, 4001)
+    sizes = [int(x) for x in rng.choice([600, 1024, 1500, 2047, 2048], size=40)]
+    rows, dst = [], 3
+    for n in sizes:
+        for _ in range(n):
+            ln = int(rng.integers(max(1, mean_len - 600), mean_len + 600))
+            rows.append((int(rng.integers(0, 255)) * 4096 + int(rng.integers(0, 4096 - ln + 1)), ln, dst))
+            dst += ln
+    descs = make_descs(rows)
+    expect = oracle_expected(oracle, pool, descs, dst + 64, 0)
+    g = GpuBuffers(pool, descs, dst + 64, 0)
+    m = Mapped(pkg, hip, np.ascontiguousarray(descs), len(sizes))
+    e = Engine(pkg, hip)
+    print("engine queued short-fragment case: %d submissions, %d descriptors, mean length %d" % (len(sizes), len(descs), mean_len), flush=True)
+    first = 0
+    for i, n in enumerate(sizes):
+        nbytes = int(descs["len"][first : first + n].sum())
+        rc = hip.tcpxuEngineSubmitSized(e.h, g.pool.data_ptr(), g.dst_base, m.desc_dev(first), n, nbytes, m.flag_dev(i), i + 1)
+        pkg.check(rc, "tcpxuEngineSubmitSized")
+        first += n
+    e.start()
+    try:
+        for i in range(len(sizes)):
+            m.wait(i, i + 1)
+    finally:
+        e.stop()
+    assert e.completed() == len(sizes)
+    got = g.result()
+    e.destroy()
+    m.free()
+    assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
+
+
 @pytest.mark.parametrize("per_ticket", [0, 5, 14, 16])
 def test_engine_lines_shared_across_the_ends_of_tickets(pkg, hip, oracle, per_ticket):
     """With eight or more submissions in flight the tickets of a submission share destination lines across their
