@@ -52,7 +52,7 @@ import __graft_entry__ as graft
 # the hardware counters FETCH_SIZE and WRITE_SIZE of one launch of `bench.py --one-launch --steps 20 --warmup 5`
 # (two rocprofv3 --pmc runs), each scaled by what the same counter reads for the plain copy kernel of known size
 # (`--calibrate-copy 256`); the summary with the counter values is profiles/unpack_engine_kernel_8MiB_chunk_pmc_traffic.txt.
-TRAFFIC_PER_ALGORITHMIC_BYTE = 1.0080
+TRAFFIC_PER_ALGORITHMIC_BYTE = 1.0079
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # Steps in the untimed launch that precedes the measured one, and the least steps the windows of the measured launch
 # add up to (60 ms each way): the rate the engine sustains shows only after some milliseconds of load.
@@ -717,15 +717,33 @@ def main():
         ev1.synchronize()
         runtime_copy_gbps = 2 * n_copy * 20 / (ev0.elapsed_time(ev1) * 1e-3) / 1e9
         del lo, hi
+        # A bare gather of short fragments: 1 GiB of them (four times the Infinity Cache each way) from random pages of
+        # a 4 GiB pool to a contiguous destination -- the grain of the adversarial workload (2 KiB a fragment on average)
+        # without any of the unpack kernel's work on it.
+        del scratch
+        gather_pool = torch.empty(4 * n_copy, dtype=torch.uint8, device="cuda:0")
+        gather_pool.zero_()
+        gather_dst = torch.empty(n_copy, dtype=torch.uint8, device="cuda:0")
+        gather = {}
+        for kib in (1, 2, 4):
+            n_frag = n_copy // (kib << 10)
+            pages_d = torch.randint(0, (4 * n_copy) // 4096, (n_frag,), dtype=torch.int32, device="cuda:0")
+            torch.cuda.synchronize()
+            pkg.check(benchlib.tcpxuGatherKernelTimed(dev, gather_dst.data_ptr(), gather_pool.data_ptr(), pages_d.data_ptr(), n_frag, kib << 10, 2, 10, ctypes.byref(us)), "gather timed")
+            gather["gather_%dKiB_fragments_rw_GBps" % kib] = round(2 * n_copy / us.value / 1e3, 1)
+            del pages_d
+        del gather_pool, gather_dst
         result["hbm_yardsticks"] = {
             "read_only_GBps": round(read_gbps, 1),
             "write_only_GBps": round(write_gbps, 1),
             "runtime_device_to_device_copy_rw_GBps": round(runtime_copy_gbps, 1),
             "copy_bound_rw_GBps": round(2.0 / (1.0 / read_gbps + 1.0 / write_gbps), 1),
+            **gather,
             "note": "plain kernels over 2 GiB with the unpack kernel's load and store instructions; copy_bound is what a "
-            "plain copy made of these two halves comes to (1/read + 1/write per byte), against the roofline's 8000 GB/s",
+            "plain copy made of these two halves comes to (1/read + 1/write per byte), against the roofline's 8000 GB/s; "
+            "gather_*: 1 GiB made of the first 1, 2 or 4 KiB of random pages of a 4 GiB pool to a contiguous destination, "
+            "one wavefront per fragment, sixteen per compute unit",
         }
-        del scratch
 
         result["other_configs"] = other_configs(pkg, torch, run)
         result["launch_per_batch_1GiB"] = batch_kernel_line(pkg, benchlib, torch, dev)

@@ -36,6 +36,13 @@ int tcpxuUnpackBatchTimed(int device, const void* bounce_base, void* dst_base, c
 int tcpxuCopyKernelTimed(int device, void* dst, const void* src, size_t bytes, int warmup, int iters,
                          double* mean_us);
 
+/* A bare gather, timed the same way: the first fragment_bytes (1024, 2048, 3072 or 4096) of page pages_dev[i] (a
+ * list of n_fragments 4 KiB page numbers in device memory) of `src` to dst + i * fragment_bytes, one wavefront per
+ * fragment with the unpack kernel's loads and stores and nothing else.  The yardstick for workloads of short
+ * fragments: what the memory system gives to a gather of that grain. */
+int tcpxuGatherKernelTimed(int device, void* dst, const void* src, const uint32_t* pages_dev, uint32_t n_fragments,
+                           uint32_t fragment_bytes, int warmup, int iters, double* mean_us);
+
 /* Launches the copy kernel once on `stream` (a hipStream_t) and returns: something else for the GPU to do while
  * the engine runs. */
 int tcpxuCopyKernelLaunch(int device, void* dst, const void* src, size_t bytes, void* stream);

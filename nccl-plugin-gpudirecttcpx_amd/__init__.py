@@ -260,6 +260,20 @@ _BENCH_PROTOTYPES = {
             ctypes.POINTER(ctypes.c_double),
         ],
     ),
+    "tcpxuGatherKernelTimed": (
+        ctypes.c_int,
+        [
+            ctypes.c_int,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.c_void_p,
+            ctypes.c_uint32,
+            ctypes.c_uint32,
+            ctypes.c_int,
+            ctypes.c_int,
+            ctypes.POINTER(ctypes.c_double),
+        ],
+    ),
     "tcpxuCopyKernelTimed": (
         ctypes.c_int,
         [

@@ -20,6 +20,7 @@ namespace tcpxu_bench {
 namespace {
 
 using tcpxu::kVecPerLane;
+using tcpxu::kWaveLanes;
 using tcpxu::kWgThreads;
 using tcpxu::load_vec_sys;
 using tcpxu::store_vec_stream;
@@ -99,6 +100,28 @@ __global__ __launch_bounds__(kWgThreads) void fill_kernel(uint8_t* __restrict__ 
   }
 }
 
+// A bare gather of short fragments: the first `K` KiB of the 4 KiB page pages[i] of `src` go to dst + i * K KiB, one
+// wavefront per fragment, one fragment in flight per wavefront, the unpack kernel's load and store instructions and
+// its sixteen copy wavefronts per compute unit -- and nothing else: no descriptors, no alignment work, no shared
+// lines.  What the memory system gives to a gather of fragments of that length.
+template <int K>
+__global__ __launch_bounds__(2 * kWgThreads) void gather_kernel(uint8_t* __restrict__ dst, const uint8_t* __restrict__ src,
+                                                                const uint32_t* __restrict__ pages, uint32_t n) {
+  constexpr uint32_t kWaves = 2 * kWgThreads / kWaveLanes;
+  const uint32_t lane = threadIdx.x & (kWaveLanes - 1);
+  const uint32_t wave = blockIdx.x * kWaves + threadIdx.x / kWaveLanes, n_waves = gridDim.x * kWaves;
+  for (uint32_t i = wave; i < n; i += n_waves) {
+    const uint8_t* from = src + (static_cast<uint64_t>(pages[i]) << 12);
+    uint8_t* to = dst + static_cast<uint64_t>(i) * (K * 1024);
+    u32x4 r[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) r[k] = load_vec_sys(from + ((k * kWaveLanes + lane) << 4));
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int k = 0; k < K; ++k) store_vec_stream(to + ((k * kWaveLanes + lane) << 4), r[k]);
+  }
+}
+
 // Mean of per-launch durations: every launch sits between its own pair of events on the launch stream, so
 // gaps between launches are not counted.
 int time_launches(hipStream_t stream, int warmup, int iters, double* mean_us, int (*launch)(void*, hipStream_t),
@@ -165,6 +188,28 @@ int launch_copy(const CopyLaunch* c, hipStream_t s) {
   }
   if (hipGetLastError() != hipSuccess) {
     set_error("copy kernel launch failed");
+    return TCPXU_DEVICE_ERROR;
+  }
+  return TCPXU_SUCCESS;
+}
+
+struct GatherLaunch {
+  uint8_t* dst;
+  const uint8_t* src;
+  const uint32_t* pages;
+  uint32_t n, kib, grid;
+};
+
+int launch_gather(const GatherLaunch* g, hipStream_t s) {
+  const dim3 grid(g->grid), block(2 * kWgThreads);
+  switch (g->kib) {
+    case 1: hipLaunchKernelGGL(gather_kernel<1>, grid, block, 0, s, g->dst, g->src, g->pages, g->n); break;
+    case 2: hipLaunchKernelGGL(gather_kernel<2>, grid, block, 0, s, g->dst, g->src, g->pages, g->n); break;
+    case 3: hipLaunchKernelGGL(gather_kernel<3>, grid, block, 0, s, g->dst, g->src, g->pages, g->n); break;
+    default: hipLaunchKernelGGL(gather_kernel<4>, grid, block, 0, s, g->dst, g->src, g->pages, g->n); break;
+  }
+  if (hipGetLastError() != hipSuccess) {
+    set_error("gather kernel launch failed");
     return TCPXU_DEVICE_ERROR;
   }
   return TCPXU_SUCCESS;
@@ -447,6 +492,29 @@ int tcpxuCopyKernelTimed(int device, void* dst, const void* src, size_t bytes, i
       &c);
   (void)hipStreamDestroy(stream);
   (void)hipFree(c.sink);
+  return rc;
+}
+
+int tcpxuGatherKernelTimed(int device, void* dst, const void* src, const uint32_t* pages_dev, uint32_t n_fragments,
+                           uint32_t fragment_bytes, int warmup, int iters, double* mean_us) {
+  if (!mean_us || iters <= 0 || warmup < 0 || !dst || !src || !pages_dev || n_fragments == 0 || fragment_bytes == 0 ||
+      fragment_bytes > TCPXU_PAGE_SIZE || fragment_bytes % 1024 != 0 || reinterpret_cast<uintptr_t>(dst) % 16 != 0 ||
+      reinterpret_cast<uintptr_t>(src) % 16 != 0) {
+    set_error("gather kernel needs 16-byte aligned buffers, a page list and fragments of 1, 2, 3 or 4 KiB");
+    return TCPXU_INVALID_ARGUMENT;
+  }
+  int cus = 0;
+  BENCH_TRY(tcpxuDeviceInfo(device, nullptr, 0, &cus));  // also makes the device current
+  GatherLaunch g{static_cast<uint8_t*>(dst), static_cast<const uint8_t*>(src), pages_dev, n_fragments, fragment_bytes / 1024,
+                 static_cast<uint32_t>(std::max(cus, 1)) * 2};
+  hipStream_t stream;
+  if (hipStreamCreate(&stream) != hipSuccess) {
+    set_error("hipStreamCreate failed");
+    return TCPXU_DEVICE_ERROR;
+  }
+  int rc = time_launches(
+      stream, warmup, iters, mean_us, [](void* p, hipStream_t s) { return launch_gather(static_cast<GatherLaunch*>(p), s); }, &g);
+  (void)hipStreamDestroy(stream);
   return rc;
 }
 
