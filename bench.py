@@ -226,6 +226,44 @@ def other_configs(pkg, torch, run, only=None):
     return out
 
 
+def fragment_length_sweep(pkg, torch, run):
+    """Fragments of one length through the engine, 64 slots in flight: 65536 fragments a pass, each the first `length`
+    bytes of a 4 KiB page of a 256 MiB pool (4 copies in turn), laid end to end from a line boundary, in requests of
+    2048 descriptors with their byte counts.  Sources and destinations sit on line boundaries, so nothing is shifted
+    and no destination line is shared: what remains is the grain, to be read beside hbm_yardsticks' bare gathers."""
+    out = {}
+    n_frag, per_req, copies, passes = 65536, 2048, 4, 40
+    pool_bytes = n_frag * 4096
+    pool_d = torch.empty(copies * pool_bytes, dtype=torch.uint8, device="cuda:0").random_(0, 256)
+    dst_d = torch.empty((1 << 30) + 8192, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    for length in (1024, 2048, 4096):
+        descs = np.zeros(n_frag, dtype=np.dtype([("src_off", "<u4"), ("len", "<u4"), ("dst_off", "<u8")]))
+        descs["src_off"] = np.arange(n_frag, dtype=np.int64) * 4096
+        descs["len"] = length
+        descs["dst_off"] = np.arange(n_frag, dtype=np.int64) * length
+        total = n_frag * length
+        n_dst = (1 << 30) // total
+        n_req = n_frag // per_req
+        items = (pkg.StreamItem * (passes * n_req))()
+        i = 0
+        for ps in range(passes):
+            for r in range(n_req):
+                items[i].bounce_base = pool_d.data_ptr() + (ps % copies) * pool_bytes
+                items[i].dst_base = dst_d.data_ptr() + 256 + (ps % n_dst) * total
+                items[i].descs_host = descs.ctypes.data + 16 * r * per_req
+                items[i].n_descs = per_req
+                items[i].payload_bytes = per_req * length
+                i += 1
+        wall_us, _, _ = run(items, 64, warmup_items=n_req)
+        out["fragments_of_%d" % length] = {
+            "payload_GBps": round(float(total) * (passes - 1) / (wall_us * 1e-6) / 1e9, 1),
+            "rw_frac_of_hbm_peak": round(2.0 * total * (passes - 1) / (wall_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+        }
+    del pool_d, dst_d
+    return out
+
+
 def storm_launch(pkg, hip, benchlib, torch, engine, in_flight, reps=64):
     """One launch of the engine over the storm of 64 KiB requests (2048 requests of 16 whole pages from a 512 MiB
     pool, `reps` times over, into a ring of 1 GiB of destinations), `in_flight` of them in flight."""
@@ -746,6 +784,7 @@ def main():
         }
 
         result["other_configs"] = other_configs(pkg, torch, run)
+        result["fragment_length_sweep"] = fragment_length_sweep(pkg, torch, run)
         result["launch_per_batch_1GiB"] = batch_kernel_line(pkg, benchlib, torch, dev)
 
     pkg.check(hip.tcpxuEngineDestroy(engine), "tcpxuEngineDestroy")

@@ -87,6 +87,10 @@ def test_bench_extras_report_latency_and_the_storm_sweep():
     assert r["launch_per_batch_1GiB"]["kernel"] == "unpack_batch_kernel" and r["launch_per_batch_1GiB"]["rw_GBps"] > 0
     yard = r["hbm_yardsticks"]
     assert yard["read_only_GBps"] > 0 and yard["write_only_GBps"] > 0 and yard["copy_bound_rw_GBps"] > 0
+    # the grain of short fragments: bare gathers, and the engine on fragments of one length
+    assert all(yard["gather_%dKiB_fragments_rw_GBps" % k] > 0 for k in (1, 2, 4))
+    assert sorted(r["fragment_length_sweep"]) == ["fragments_of_1024", "fragments_of_2048", "fragments_of_4096"]
+    assert all(0 < v["rw_frac_of_hbm_peak"] < 1 for v in r["fragment_length_sweep"].values())
 
 
 def test_one_config_mode_launches_the_engine_once_over_another_workload():
