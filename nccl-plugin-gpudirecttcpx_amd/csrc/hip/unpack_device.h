@@ -179,16 +179,15 @@ __device__ __forceinline__ uint32_t load_dword_sys(const uint8_t* p) {
 __device__ __forceinline__ void round_load(const CopyRound& c, CopyRegs& x, uint32_t lane) {
   const uint32_t skew = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(c.src_vec)) & 3u;
   const uint8_t* base4 = c.src_vec - skew;
-  x.edge_byte = 0;
-  x.tail_dword = 0;
-  x.line_a = u32x4{0, 0, 0, 0};
-  x.line_b = u32x4{0, 0, 0, 0};
+  // No register of the round is cleared first: a lane that loads nothing stores nothing (the same conditions guard
+  // the stores), and what the shifts read from such a lane never reaches a stored byte.  The empty statement only
+  // tells the compiler that the registers have a value (clearing them was a tenth of a short round's instructions).
+  asm volatile("" : "=v"(x.r[0]), "=v"(x.r[1]), "=v"(x.r[2]), "=v"(x.r[3]), "=v"(x.line_a), "=v"(x.line_b), "=v"(x.tail_dword), "=v"(x.edge_byte));
   if (c.has_edge) {
     if (c.edge_off != kNoEdge) x.edge_byte = load_byte_sys(c.src_frag + c.edge_off);
   }
 #pragma unroll
   for (int k = 0; k < kVecPerLane; ++k) {
-    x.r[k] = u32x4{0, 0, 0, 0};
     const uint32_t v = static_cast<uint32_t>(k) * kWaveLanes + lane;
     if (v < c.nvec) x.r[k] = load_vec_sys(base4 + (v << 4));
   }
