@@ -132,7 +132,7 @@ struct CopyRound {
 constexpr int kDppWaveShiftLeft1 = 0x130;  // lane i receives lane i+1's value; lane 63 keeps the first operand
 struct CopyRegs {
   u32x4 r[kVecPerLane];
-  u32x4 line_a, line_b;
+  u32x4 line;  // lanes 0..7: the shared line's vectors as loaded; lane 8: the first 16 bytes of the next fragment
   uint32_t tail_dword;
   uint32_t edge_byte;
 };
@@ -144,8 +144,8 @@ constexpr uint32_t kLineVecs = kLineBytes / 16;  // lanes that take part in the 
 //   vectors before the boundary are 16 bytes of A, vectors after it 16 bytes of B, each loaded where it lies
 //   (any alignment) and stored as loaded;
 //   the one vector the boundary cuts (none if rem is a multiple of 16) is the last `cut` bytes of A followed by
-//   the first 16 - cut bytes of B: its lane loads A's last 16 bytes and B's first 16 and takes bytes
-//   [16 - cut, 32 - cut) of the two, a shift by a wave-uniform amount.
+//   the first 16 - cut bytes of B: its lane loads A's last 16 bytes, lane 8 of the same instruction loads B's first
+//   16 for it, and it takes bytes [16 - cut, 32 - cut) of the two, a shift by a wave-uniform amount.
 // shares_line has seen to it that every one of these loads stays inside its fragment.
 // (An earlier form gave every lane two loads and a shift of its own, by a per-lane amount: some sixty vector
 // instructions a line instead of some twenty, a sixth of the time of a round of a 2 KiB fragment.)
@@ -182,7 +182,7 @@ __device__ __forceinline__ void round_load(const CopyRound& c, CopyRegs& x, uint
   // No register of the round is cleared first: a lane that loads nothing stores nothing (the same conditions guard
   // the stores), and what the shifts read from such a lane never reaches a stored byte.  The empty statement only
   // tells the compiler that the registers have a value (clearing them was a tenth of a short round's instructions).
-  asm volatile("" : "=v"(x.r[0]), "=v"(x.r[1]), "=v"(x.r[2]), "=v"(x.r[3]), "=v"(x.line_a), "=v"(x.line_b), "=v"(x.tail_dword), "=v"(x.edge_byte));
+  asm volatile("" : "=v"(x.r[0]), "=v"(x.r[1]), "=v"(x.r[2]), "=v"(x.r[3]), "=v"(x.line), "=v"(x.tail_dword), "=v"(x.edge_byte));
   if (c.has_edge) {
     if (c.edge_off != kNoEdge) x.edge_byte = load_byte_sys(c.src_frag + c.edge_off);
   }
@@ -196,14 +196,14 @@ __device__ __forceinline__ void round_load(const CopyRound& c, CopyRegs& x, uint
   }
   if (c.share_next) {
     const LinePlan p = line_plan(c);
-    if (lane < kLineVecs) {
+    // One load instruction: the line's eight vectors in lanes 0..7 and, where the boundary cuts a vector, the next
+    // fragment's first 16 bytes in lane 8 (a load of its own for that one lane was a fifth of a ragged round's loads).
+    if (lane < kLineVecs + (p.cut != 0 ? 1u : 0u)) {
       const uint32_t off = lane << 4;
       const uint8_t* from = lane < p.cut_lane ? c.src_frag + c.line_off + off : c.src_next + (off - p.rem);
       if (p.cut != 0 && lane == p.cut_lane) from = c.src_frag + c.frag_len - 16u;
-      x.line_a = load_vec_sys(from);
-    }
-    if (p.cut != 0) {
-      if (lane == p.cut_lane) x.line_b = load_vec_sys(c.src_next);
+      if (lane == kLineVecs) from = c.src_next;
+      x.line = load_vec_sys(from);
     }
   }
 }
@@ -214,7 +214,7 @@ __device__ __forceinline__ void round_load(const CopyRound& c, CopyRegs& x, uint
 // use of them can be scheduled before it.
 __device__ __forceinline__ void round_wait(CopyRegs& x) {
   asm volatile("s_waitcnt vmcnt(0)"
-               : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.r[2]), "+v"(x.r[3]), "+v"(x.line_a), "+v"(x.line_b),
+               : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.r[2]), "+v"(x.r[3]), "+v"(x.line),
                  "+v"(x.tail_dword), "+v"(x.edge_byte)
                :
                : "memory");
@@ -247,9 +247,14 @@ __device__ __forceinline__ void round_store_loaded(const CopyRound& c, CopyRegs&
   }
   if (c.share_next) {
     const LinePlan p = line_plan(c);
-    u32x4 line = x.line_a;
+    u32x4 line = x.line;
     if (p.cut != 0) {
-      const u32x4 cut_vector = extract16(x.line_a, x.line_b, 16u - p.cut);
+      // (lane 8's vector, the same for every lane: scalar registers)
+      u32x4 next16;
+#pragma unroll
+      for (int d = 0; d < 4; ++d)
+        next16[d] = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(x.line[d]), static_cast<int>(kLineVecs)));
+      const u32x4 cut_vector = extract16(x.line, next16, 16u - p.cut);
       if (lane == p.cut_lane) line = cut_vector;
     }
     if (lane < kLineVecs) store_vec_stream(c.dst_frag + c.line_off + (lane << 4), line);
