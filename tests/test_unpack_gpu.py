@@ -193,6 +193,25 @@ def test_yardstick_kernels_copy_read_fill(pkg, hip, benchlib):
     assert benchlib.tcpxuCopyKernelTimed(0, dst.data_ptr(), src.data_ptr(), n + 8, 1, 3, ctypes.byref(us)) == pkg.INVALID_ARGUMENT
 
 
+@pytest.mark.parametrize("kib", [1, 2, 3, 4])
+def test_yardstick_gather_kernel_moves_the_fragments_it_says(pkg, hip, benchlib, kib):
+    """The bare gather behind the benchmark's short-fragment yardsticks: fragment i of the destination is the first
+    kib KiB of page pages[i] of the pool, for every i, and nothing beyond the last fragment is written."""
+    import torch
+
+    n_pages, n_frag, frag = 4096, 3001, kib << 10
+    pool = torch.randint(0, 256, (n_pages * 4096,), dtype=torch.uint8, device="cuda:0")
+    pages = torch.randint(0, n_pages, (n_frag,), dtype=torch.int32, device="cuda:0")
+    dst = torch.full((n_frag * frag + 64,), SENTINEL, dtype=torch.uint8, device="cuda:0")
+    us = ctypes.c_double()
+    print("gather yardstick case: %d fragments of %d bytes" % (n_frag, frag), flush=True)
+    pkg.check(benchlib.tcpxuGatherKernelTimed(0, dst.data_ptr(), pool.data_ptr(), pages.data_ptr(), n_frag, frag, 1, 2, ctypes.byref(us)), "gather")
+    want = pool.view(n_pages, 4096)[pages.long(), :frag].reshape(-1)
+    assert us.value > 0 and torch.equal(dst[: n_frag * frag], want) and bool((dst[n_frag * frag :] == SENTINEL).all())
+    assert benchlib.tcpxuGatherKernelTimed(0, dst.data_ptr(), pool.data_ptr(), pages.data_ptr(), n_frag, frag + 512, 1, 2, ctypes.byref(us)) == pkg.INVALID_ARGUMENT
+    assert benchlib.tcpxuGatherKernelTimed(0, dst.data_ptr(), pool.data_ptr(), None, n_frag, frag, 1, 2, ctypes.byref(us)) == pkg.INVALID_ARGUMENT
+
+
 def test_batch_launches_replayed_from_a_hip_graph(pkg, hip, oracle):
     """A launch-bound loop of small batches (32 requests of 16 fragments, one tcpxuUnpackBatch each) captured once
     into a HIP graph on a caller's stream and replayed: every replay, with the pool refilled and the destination
