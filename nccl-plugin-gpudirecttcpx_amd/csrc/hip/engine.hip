@@ -137,6 +137,8 @@ constexpr uint32_t kPollEntries = 16;  // submission entries fetched per load in
 // four loads in flight together, 64 entries for the one PCIe round trip (about 1.5 us) that sixteen cost -- which
 // is what capped a storm of one-ticket requests near 9 M/s.
 constexpr uint32_t kDeepGroups = 3;    // groups of kPollEntries beyond the first in a deep poll
+constexpr uint32_t kStormBacklog = 256;  // entries published beyond a poll's 64 from which the leader takes them in a rolling loop
+constexpr uint32_t kAuxProbe = 35;  // lane of an auxiliary load that reads the stamp of an entry ahead
 constexpr uint32_t kAuxTicketsDone = 32, kAuxHostStop = 33, kAuxJobsCompleted = 34;  // lanes of the auxiliary load
 constexpr uint32_t kNeverIdleOut = 0xFFFFFFFFu;
 constexpr uint32_t kDefaultIdlePolls = 400;  // empty polls (about 1.2 us each) before the kernel leaves by itself
@@ -260,6 +262,179 @@ __device__ __forceinline__ uint32_t lane_value(uint32_t v, uint32_t src_lane) {
 constexpr uint32_t kStampsPerJob = 4;
 __device__ __forceinline__ uint64_t clock_now() { return wall_clock64(); }
 
+// What the four lanes of an entry know about it, for the sixteen entries of one group at once.
+struct EntryView {
+  uint32_t n, bytes, per_ticket, target_prev, in_flight, slot;
+  bool sane, slot_free;
+};
+
+// Every entry of a group fits one ticket (a storm of small requests): the leading run of them becomes tickets in
+// one store instruction.  Returns the length of the run; `room` is what the ticket ring still takes.
+__device__ __forceinline__ uint32_t write_single_tickets_of_group(DevState* st, uint32_t* job_target, uint64_t* stamps,
+                                                                  uint64_t& tickets_out, uint32_t lane, const EntryView& v,
+                                                                  const u32x4& sc, uint32_t room) {
+  const uint32_t k_of_lane = lane >> 2;
+  const uint64_t not_now = ~__ballot(v.sane && v.slot_free);
+  uint32_t run = not_now == 0 ? kPollEntries : static_cast<uint32_t>(__builtin_ctzll(not_now)) >> 2;
+  run = std::min(run, room);
+  if (run != 0) {
+    if (k_of_lane < run) {
+      const uint64_t t = tickets_out + k_of_lane;
+      const uint32_t stamp = static_cast<uint32_t>(t + 1);
+      const uint32_t target = v.target_prev + 1u;
+      u32x4 out{sc.x, sc.y, sc.z, stamp};
+      if ((lane & 3u) == 3) {
+        out.y = v.n | (v.slot << 8) | kOnlyTicket;
+        out.z = target;
+        sys_store(&job_target[v.slot], target);
+        if (stamps) sys_store(&stamps[kStampsPerJob * v.slot], clock_now());
+      }
+      store_vec_sys(reinterpret_cast<uint8_t*>(&st->tickets[t & (kTicketRing - 1)]) + 16 * (lane & 3u), out);
+    }
+    tickets_out += run;
+  }
+  return run;
+}
+
+__device__ __forceinline__ uint64_t same_in_all_lanes64(uint64_t v) {
+  return (static_cast<uint64_t>(static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(v >> 32)))) << 32) |
+         static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(v)));
+}
+template <typename T>
+__device__ __forceinline__ T* same_in_all_lanes_ptr(T* p) {
+  return reinterpret_cast<T*>(same_in_all_lanes64(reinterpret_cast<uint64_t>(p)));
+}
+
+// A storm: a deep poll turned all its 64 entries into tickets and the host has published kStormBacklog entries beyond
+// them.  Takes entries from s on for as long as they are published and are one ticket each; returns where it got to.
+//
+// Four groups of sixteen entries are in flight at a time, and the registers of a group that has gone through take the
+// group 64 entries on at once (every group's loads bring the stamp of the last entry of the group that would be asked
+// for next: entries are published in order, so if that one is there the whole group is).  The leader's time per group
+// is then a quarter of the round trip to the host's ring or what it takes to turn a group into tickets, whichever is
+// longer -- not their sum as in a poll (1024 requests of 64 KiB in flight: 21 -> 36 M requests/s).  Every group has
+// registers of its own (moving one that is still in flight to another register would wait for it), hence four copies
+// of one step instead of a loop over an array.  When the host's tail is reached nothing more is asked for and the
+// groups in flight go through: the loop ends with nothing in flight.
+//
+// The compiler would wait for everything in flight at the top of such a loop.  So the loop's loads are written as
+// instructions, which it does not track, and each step waits for its own group by count: the memory instructions of
+// a wavefront complete in the order issued, and between a group's loads and its turn three other groups have had
+// theirs, each with two stores (the tickets, their job slots' targets) and, while the loop feeds, two loads: twelve
+// instructions at the least, so "at most twelve outstanding" means that the group's own loads have landed.  (More
+// are issued when stamps are on, and the head word once a round: counting too few only waits for a little more than
+// is needed.)  Once the loop has stopped feeding, a group waits for everything.  The group's registers pass through
+// a statement after the wait so that nothing reads them before it.
+//
+// A function of its own, not inlined, and called from the top of the leader's loop where little is live: with this
+// loop inside the leader's, what the compiler did with the registers around it made every poll that never sees a
+// storm 0.2 us slower.  The running count of finished tickets is read once: too few counted as done only ends the
+// storm early (after at most kTicketRing entries, which is also how long the host's stop word can go unread).
+struct StormEnd {
+  uint64_t s, tickets_out;
+  uint32_t entries, rounds;  // entries taken off the ring, in so many rounds of up to 64
+};
+__device__ __attribute__((noinline)) StormEnd leader_storm(HostCtl* ctl_in, DevState* st_in, uint32_t* jobs_done_in,
+                                                          uint64_t* stamps_in, uint32_t ring_mask_in,
+                                                          uint32_t fixed_per_ticket_in, uint64_t s_in, uint64_t tickets_out_in) {
+  // Arguments arrive in vector registers.  These are the same in every lane and go back to scalar registers.  (The job
+  // slots' targets follow their counts in memory: one pointer for both.)
+  HostCtl* ctl = same_in_all_lanes_ptr(ctl_in);
+  DevState* st = same_in_all_lanes_ptr(st_in);
+  uint32_t* jobs_done = same_in_all_lanes_ptr(jobs_done_in);
+  uint64_t* stamps = same_in_all_lanes_ptr(stamps_in);
+  const uint32_t ring_mask = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(ring_mask_in)));
+  uint32_t* job_target = jobs_done + ring_mask + 1u;
+  const uint32_t fixed_per_ticket = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(fixed_per_ticket_in)));
+  uint64_t s = same_in_all_lanes64(s_in);
+  uint64_t tickets_out = same_in_all_lanes64(tickets_out_in);
+  const uint32_t lane = threadIdx.x;
+  const uint32_t k_of_lane = lane >> 2;
+  uint32_t consumed = 0, entries = 0, rounds = 0;
+  constexpr uint32_t kGroups = kDeepGroups + 1;  // in flight
+  static_assert(kGroups == 4, "four copies of one step below, and the count of the wait");
+  auto fetch_group_untracked = [&](u32x4& sc, uint32_t& ax, uint64_t s_g) {
+    const uint8_t* entry = reinterpret_cast<const uint8_t*>(&ctl->ring[(s_g + k_of_lane) & ring_mask]) + 16 * (lane & 3);
+    const uint32_t* at = lane < kPollEntries       ? &jobs_done[(s_g + lane) & ring_mask]
+                         : lane < 2 * kPollEntries ? &job_target[(s_g + lane - kPollEntries) & ring_mask]
+                                                   : &ctl->ring[(s_g + (kGroups + 1) * kPollEntries - 1) & ring_mask].w[15];  // (lane 35's probe; the others repeat it)
+    asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(sc) : "v"(entry) : "memory");
+    asm volatile("global_load_dword %0, %1, off sc0 sc1" : "=v"(ax) : "v"(at) : "memory");
+  };
+  // 4 while the loop feeds (four groups in flight); once it has caught up with the host, the groups still in flight
+  // that have not gone through: 3, 2, 1, and at 0 the storm is over.
+  uint32_t feeding = kGroups;
+  u32x4 sc0, sc1, sc2, sc3;
+  uint32_t ax0, ax1, ax2, ax3, tickets_done;
+  fetch_group_untracked(sc0, ax0, s);
+  fetch_group_untracked(sc1, ax1, s + kPollEntries);
+  fetch_group_untracked(sc2, ax2, s + 2 * kPollEntries);
+  fetch_group_untracked(sc3, ax3, s + 3 * kPollEntries);
+  asm volatile("global_load_dword %0, %1, off sc0 sc1" : "=v"(tickets_done) : "v"(reinterpret_cast<const uint32_t*>(&st->tickets_done)) : "memory");
+  asm volatile("s_waitcnt vmcnt(0)" : "+v"(sc0), "+v"(sc1), "+v"(sc2), "+v"(sc3), "+v"(ax0), "+v"(ax1), "+v"(ax2), "+v"(ax3), "+v"(tickets_done) : : "memory");
+  tickets_done = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(tickets_done)));
+  // One group through; false when the storm is over: nothing more in flight, or the group was not there whole or not
+  // all of one ticket each (then whatever is in flight is dropped, and the leader's next poll asks again).
+  auto pass = [&](u32x4& sc, uint32_t& ax) {
+    // (While the loop feeds, the three steps before this one all fed: it stops feeding once and for all.  The first
+    // four groups have landed, whichever wait they get.)
+    if (feeding == kGroups) asm volatile("s_waitcnt vmcnt(12)" : : : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+    asm volatile("" : "+v"(sc), "+v"(ax) : : "memory");
+    const uint64_t s_g = s + consumed;
+    const uint64_t okm = __ballot(sc.w == static_cast<uint32_t>(s_g + k_of_lane + 1));
+    uint32_t run = 0;
+    if ((okm & 0xFull) == 0xFull) {
+      const uint32_t left = kTicketRing - (static_cast<uint32_t>(tickets_out) - tickets_done);
+      // With hundreds of submissions waiting, one of at most 32 descriptors is one ticket (see
+      // ticket_size_for_submission; a fixed ticket size says so itself): no sizing here, and a group with a larger
+      // one ends the storm and goes the ordinary way.
+      EntryView more;
+      more.n = bcast(sc.y, lane | 3u);
+      more.bytes = 0, more.per_ticket = 0, more.in_flight = 0;  // (not looked at by write_single_tickets_of_group)
+      more.target_prev = bcast(ax, kPollEntries + k_of_lane);
+      more.sane = ((okm >> (4 * k_of_lane)) & 0xFull) == 0xFull && more.n - 1u < kMaxDescsPerSubmission;
+      more.slot_free = bcast(ax, k_of_lane) == more.target_prev;
+      more.slot = static_cast<uint32_t>(s_g + k_of_lane) & ring_mask;
+      const uint32_t one_ticket = fixed_per_ticket != 0 ? fixed_per_ticket : kSmallSubmission;
+      if (__ballot(more.sane && more.n > one_ticket) == 0) run = write_single_tickets_of_group(st, job_target, stamps, tickets_out, lane, more, sc, left);
+    }
+    consumed += run;
+    if (run != kPollEntries) return false;
+    if (feeding == kGroups) {
+      const uint64_t next = s_g + kGroups * kPollEntries;
+      if (lane_value(ax, kAuxProbe) == static_cast<uint32_t>(next + kPollEntries)) fetch_group_untracked(sc, ax, next);
+      else feeding = kGroups - 1;
+    } else {
+      --feeding;
+    }
+    feeding = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(feeding)));
+    return feeding != 0;
+  };
+#pragma unroll 1
+  for (;;) {
+    if (!pass(sc0, ax0)) break;
+    if (!pass(sc1, ax1)) break;
+    if (!pass(sc2, ax2)) break;
+    if (!pass(sc3, ax3)) break;
+    // 64 entries on: the host learns of it, and the counts of this launch take them as one more poll of 64
+    s += consumed;
+    entries += consumed;
+    consumed = 0;
+    if (lane == 0) sys_store(&ctl->head, s);
+    ++rounds;
+  }
+  // Whatever is still in flight is waited for, so that the registers it lands in are free.
+  asm volatile("s_waitcnt vmcnt(0)" : "+v"(sc0), "+v"(sc1), "+v"(sc2), "+v"(sc3), "+v"(ax0), "+v"(ax1), "+v"(ax2), "+v"(ax3) : : "memory");
+  if (consumed != 0) {  // the round that the storm ended in
+    s += consumed;
+    entries += consumed;
+    if (lane == 0) sys_store(&ctl->head, s);
+    ++rounds;
+  }
+  return StormEnd{s, tickets_out, entries, rounds};
+}
+
 __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uint32_t* job_target,
                             uint32_t ring_mask, uint32_t fixed_per_ticket, uint32_t spin_limit, uint64_t* stamps) {
   // The leader's positions are the same in every lane: said outright, so that they stay in scalar registers (in
@@ -278,7 +453,9 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
   uint32_t polls = 0, entries = 0, deep_polls = 0;  // of this launch; added to the running totals at the end
   // The next poll fetches 64 entries.  (A ring of fewer entries than that never has them.)
   bool deep = false;
+  bool storm_next = false;
   const bool ring_allows_deep = ring_mask + 1u >= (kDeepGroups + 1) * kPollEntries;
+  const bool ring_allows_storm = ring_mask + 1u >= 2 * ((kDeepGroups + 1) * kPollEntries + kStormBacklog);
   // Fixed per-lane roles in the auxiliary load (second load of every poll), so that both loads of a poll are
   // issued back to back by all lanes and waited for once:
   //   lanes 0-15  jobs_done of the job slots of entries s..s+15    lanes 16-31  job_target of the same slots
@@ -289,6 +466,17 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
   const uint32_t* const jobs_completed_lo = reinterpret_cast<const uint32_t*>(&st->jobs_completed);
 
   for (;;) {
+    // (Its rounds of 64 count as deep polls in this launch's figures.)
+    if (storm_next) {
+      storm_next = false;
+      const StormEnd end = leader_storm(ctl, st, jobs_done, stamps, ring_mask, fixed_per_ticket, s, tickets_out);
+      s = same_in_all_lanes(end.s);
+      tickets_out = same_in_all_lanes(end.tickets_out);
+      entries += end.entries;
+      polls += end.rounds;
+      deep_polls += end.rounds;
+      deep = ring_allows_deep;
+    }
     // What depends on the lane is worked out afresh in every pass (the empty statement hides from the compiler that
     // the lane is the same each time): a dozen per-lane addresses kept in registers for the life of the loop are
     // what would push the kernel beyond the 80 vector registers that let two workgroups share a compute unit, and a
@@ -318,9 +506,11 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
       for (uint32_t g = 0; g < kDeepGroups; ++g) {
         const uint64_t s_g = s + (g + 1) * kPollEntries;
         sect_more[g] = load_vec_sys(reinterpret_cast<const uint8_t*>(&ctl->ring[(s_g + k_of_lane) & ring_mask]) + 16 * (lane & 3));
-        if (lane < 2 * kPollEntries)
-          aux_more[g] = sys_load(lane < kPollEntries ? &jobs_done[(s_g + lane) & ring_mask]
-                                                     : &job_target[(s_g + lane - kPollEntries) & ring_mask]);
+        // (The upper lanes of the last group's load read the stamp of the entry kStormBacklog beyond the poll's 64.)
+        if (lane < 2 * kPollEntries || g == kDeepGroups - 1)
+          aux_more[g] = sys_load(lane < kPollEntries       ? &jobs_done[(s_g + lane) & ring_mask]
+                                 : lane < 2 * kPollEntries ? &job_target[(s_g + lane - kPollEntries) & ring_mask]
+                                                           : &ctl->ring[(s_g + kPollEntries + kStormBacklog - 1) & ring_mask].w[15]);
       }
       ++deep_polls;
     }
@@ -356,11 +546,6 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
     bool deep_next = false;
     const uint32_t n_first = lane_value(sect.y, 3);
     const uint32_t lane_tickets_hold = kLaneTickets * (fixed_per_ticket != 0 ? fixed_per_ticket : full_ticket_size(lane_value(sect.z, 3), n_first));
-    // What the four lanes of an entry know about it, for the sixteen entries of one group at once.
-    struct EntryView {
-      uint32_t n, bytes, per_ticket, target_prev, in_flight, slot;
-      bool sane, slot_free;
-    };
     auto view_entries = [&](const u32x4& sc, uint32_t ax, uint64_t s0, uint64_t okm) {
       EntryView v;
       v.n = bcast(sc.y, lane | 3u);      // payload word 10 sits in .y of sector 3
@@ -376,29 +561,8 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
       v.slot = static_cast<uint32_t>(s0 + k_of_lane) & ring_mask;
       return v;
     };
-    // Every entry of a group fits one ticket (a storm of small requests): the leading run of them becomes tickets in
-    // one store instruction.  Returns the length of the run; `room` is what the ticket ring still takes.
     auto write_single_tickets = [&](const EntryView& v, const u32x4& sc, uint32_t room) {
-      const uint64_t not_now = ~__ballot(v.sane && v.slot_free);
-      uint32_t run = not_now == 0 ? kPollEntries : static_cast<uint32_t>(__builtin_ctzll(not_now)) >> 2;
-      run = std::min(run, room);
-      if (run != 0) {
-        if (k_of_lane < run) {
-          const uint64_t t = tickets_out + k_of_lane;
-          const uint32_t stamp = static_cast<uint32_t>(t + 1);
-          const uint32_t target = v.target_prev + 1u;
-          u32x4 out{sc.x, sc.y, sc.z, stamp};
-          if ((lane & 3u) == 3) {
-            out.y = v.n | (v.slot << 8) | kOnlyTicket;
-            out.z = target;
-            sys_store(&job_target[v.slot], target);
-            if (stamps) sys_store(&stamps[kStampsPerJob * v.slot], clock_now());
-          }
-          store_vec_sys(reinterpret_cast<uint8_t*>(&st->tickets[t & (kTicketRing - 1)]) + 16 * (lane & 3u), out);
-        }
-        tickets_out += run;
-      }
-      return run;
+      return write_single_tickets_of_group(st, job_target, stamps, tickets_out, lane, v, sc, room);
     };
     if ((ok_mask & 0xFull) == 0xFull &&  // entry s is there
         (n_first <= kMaxDescsPerTicket || (ready >= 2 && n_first <= lane_tickets_hold))) {
@@ -437,6 +601,12 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
           }
         }
         deep_next = ring_allows_deep && consumed >= kPollEntries;
+        // All 64 entries of a deep poll became tickets and the entry kStormBacklog beyond them is published (entries
+        // are published in order, so everything up to it is there): a storm, taken from the top of the next pass.  How
+        // far the host has got is read off the ring itself: the host's tail word is a line that the host writes with
+        // every publish, and a poll that reads it as well waits half a microsecond longer for it.
+        storm_next = ring_allows_storm && consumed == (kDeepGroups + 1) * kPollEntries &&
+                     lane_value(aux_more[kDeepGroups - 1], kAuxProbe) == static_cast<uint32_t>(s + (kDeepGroups + 1) * kPollEntries + kStormBacklog);
       } else if (ready >= 2 && n_first <= kLaneTickets * lane_value(per_ticket, 0)) {
         // Several entries, some of more than one ticket, the first of them not too many.  (The empty statement keeps
         // the compiler from working this block's division and lane exchanges out ahead of the branch, where every
@@ -1214,7 +1384,9 @@ int tcpxuEngineCreate(int device, const tcpxuEngineConfig* config, tcpxuEngine**
     e->job_target = e->jobs_done + cfg.ring_entries;
     // Test aid: where the engine's counts of submissions and tickets start.  Records are stamped with the low 32 bits
     // of their sequence number, and a busy engine passes 2^32 submissions within the hour; a test that starts just
-    // below sees the crossing in milliseconds.
+    // below sees the crossing in milliseconds.  (Start more than a lap of the ticket ring below: a slot of either ring
+    // that was never written reads as stamped for sequence number 2^32-1, which an engine that counts from zero
+    // reaches only after every slot has been written many times.)
     const char* vc = getenv("TCPXU_ENGINE_COUNT_FROM");
     if (vc && *vc) {
       const uint64_t from = strtoull(vc, nullptr, 0);

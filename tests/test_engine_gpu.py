@@ -499,15 +499,20 @@ def test_engine_bursts_around_the_idle_exit(pkg, hip, oracle):
     assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
 
 
-def storm_workload(pkg, oracle, seed, n_submissions=3000):
+STORM_SIZES = [0, 1, 2, 7, 8, 9, 15, 16, 17, 31, 32, 33, 40, 64, 65, 300]
+STORM_MIXED = [.05, .1, .05, .05, .1, .05, .05, .2, .05, .05, .1, .03, .03, .03, .03, .03]
+# Nearly all of one ticket, so that hundreds in a row are: one in 250 is empty, just over a ticket, or of two.
+STORM_MOSTLY_ONE_TICKET = [.001, .1, .05, .05, .1, .05, .05, .3, .05, .05, .196, .001, .001, .001, 0, 0]
+
+
+def storm_workload(pkg, oracle, seed, n_submissions=3000, p=STORM_MIXED):
     """Submissions of 0 to 300 ragged fragments in random order, each owning a stretch of one destination buffer:
     (pool on the device, sentinel-filled destination on the device, stream items, expected bytes, descriptor count)."""
     import torch
 
     rng = np.random.default_rng(seed)
     pool = np.random.default_rng(0xD00D).integers(0, 256, size=8 << 20, dtype=np.uint8)
-    sizes = rng.choice([0, 1, 2, 7, 8, 9, 15, 16, 17, 31, 32, 33, 40, 64, 65, 300], size=n_submissions,
-                       p=[.05, .1, .05, .05, .1, .05, .05, .2, .05, .05, .1, .03, .03, .03, .03, .03])
+    sizes = rng.choice(STORM_SIZES, size=n_submissions, p=p)
     rows, subs, dst_off = [], [], 0
     for n in sizes:
         first = len(rows)
@@ -555,6 +560,41 @@ def test_engine_storm_of_mixed_small_submissions(pkg, hip, oracle, depth, benchl
     e.destroy()
     got = dst_d.cpu().numpy()
     assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
+
+
+@pytest.mark.parametrize("count_from", [0, (1 << 32) - 70000])
+def test_engine_long_runs_of_one_ticket_submissions_broken_by_others(pkg, hip, oracle, benchlib, monkeypatch, count_from):
+    """1024 in flight (a slot of the stream then holds up to 64 descriptors), nearly all of one ticket: with hundreds
+    of entries published ahead of it the leader takes them in its rolling loop, four groups of sixteen in flight, and
+    every few hundred entries an empty submission, one just over a ticket or one of two tickets ends that loop and
+    goes the ordinary way.  Every byte must be the oracle's, every submission consumed exactly once -- also when the
+    32-bit stamps of tickets and entries wrap in the middle of it (an engine that starts 70000 below 2^32: more than a
+    lap of the ticket ring, because a ring slot that was never written reads as the stamp of sequence number 2^32-1)."""
+    assert abs(sum(STORM_MOSTLY_ONE_TICKET) - 1) < 1e-9
+    pool_d, dst_d, items, expect, descs = storm_workload(pkg, oracle, 0x5709 + (count_from & 0xFF), 8000, STORM_MOSTLY_ONE_TICKET)
+    if count_from:
+        monkeypatch.setenv("TCPXU_ENGINE_COUNT_FROM", str(count_from))
+    e = Engine(pkg, hip)
+    monkeypatch.delenv("TCPXU_ENGINE_COUNT_FROM", raising=False)
+    assert e.completed() == count_from
+    launches = 70000 // len(items) + 3 if count_from else 1
+    print("engine rolling-loop case: count_from=%d launches=%d submissions each=%d descriptors=%d" % (count_from, launches, len(items), len(descs)), flush=True)  # fmt: skip
+    wall, kern = ctypes.c_double(), ctypes.c_double()
+    lat = (ctypes.c_double * len(items))()
+    stats = pkg.EngineStats()
+    for launch in range(launches):
+        dst_d.fill_(SENTINEL)
+        pkg.check(benchlib.tcpxuEngineRunTimed(e.h, items, len(items), 0, 1024, 20000, ctypes.byref(wall), ctypes.byref(kern), lat), "tcpxuEngineRunTimed")
+        pkg.check(hip.tcpxuEngineGetStats(e.h, ctypes.byref(stats)), "tcpxuEngineGetStats")
+        print("engine rolling-loop case: launch %d, %.2f M submissions/s, %d entries in %d polls of which %d of 64 so far"
+              % (launch, len(items) / wall.value, stats.leader_entries, stats.leader_polls, stats.leader_deep_polls), flush=True)  # fmt: skip
+        assert e.completed() == count_from + (launch + 1) * len(items) and min(lat) > 0
+        assert stats.submissions == stats.leader_entries == (launch + 1) * len(items) and stats.launches >= launch + 1
+        assert stats.leader_deep_polls <= stats.leader_polls
+        got = dst_d.cpu().numpy()
+        assert first_difference(got, expect) is None, "launch %d, first (index, got, want, count): %r" % (launch, first_difference(got, expect))
+    assert not count_from or e.completed() > (1 << 32)
+    e.destroy()
 
 
 def test_engine_sequence_numbers_cross_2_to_the_32(pkg, hip, oracle, benchlib, monkeypatch):
