@@ -313,8 +313,8 @@ __device__ __forceinline__ T* same_in_all_lanes_ptr(T* p) {
 // for next: entries are published in order, so if that one is there the whole group is).  The leader's time per group
 // is then a quarter of the round trip to the host's ring or what it takes to turn a group into tickets, whichever is
 // longer -- not their sum as in a poll (1024 requests of 64 KiB in flight: 21 -> 36 M requests/s).  Every group has
-// registers of its own (moving one that is still in flight to another register would wait for it), hence four copies
-// of one step instead of a loop over an array.  When the host's tail is reached nothing more is asked for and the
+// registers of its own (moving one that is still in flight to another register would wait for it), hence one step
+// unrolled per group, with every index into the groups' arrays a constant.  When the host's tail is reached nothing more is asked for and the
 // groups in flight go through: the loop ends with nothing in flight.
 //
 // The compiler would wait for everything in flight at the top of such a loop.  So the loop's loads are written as
@@ -323,8 +323,10 @@ __device__ __forceinline__ T* same_in_all_lanes_ptr(T* p) {
 // theirs, each with two stores (the tickets, their job slots' targets) and, while the loop feeds, two loads: twelve
 // instructions at the least, so "at most twelve outstanding" means that the group's own loads have landed.  (More
 // are issued when stamps are on, and the head word once a round: counting too few only waits for a little more than
-// is needed.)  Once the loop has stopped feeding, a group waits for everything.  The group's registers pass through
-// a statement after the wait so that nothing reads them before it.
+// is needed; fewer would let a group be read before it has landed, so this function must not spill registers to
+// memory -- the compiler's resource report for the kernel says 0 bytes of scratch.)  Once the loop has stopped
+// feeding, a group waits for everything.  The group's registers pass through a statement after the wait so that
+// nothing reads them before it.
 //
 // A function of its own, not inlined, and called from the top of the leader's loop where little is live: with this
 // loop inside the leader's, what the compiler did with the registers around it made every poll that never sees a
@@ -351,8 +353,9 @@ __device__ __attribute__((noinline)) StormEnd leader_storm(HostCtl* ctl_in, DevS
   const uint32_t lane = threadIdx.x;
   const uint32_t k_of_lane = lane >> 2;
   uint32_t consumed = 0, entries = 0, rounds = 0;
-  constexpr uint32_t kGroups = kDeepGroups + 1;  // in flight
-  static_assert(kGroups == 4, "four copies of one step below, and the count of the wait");
+  // Groups in flight.  (Six: 1024 requests of 64 KiB in flight 35.6 -> 36.9 M/s, 512 in flight 32 -> 28 M/s: with four
+  // the round trip is hidden already and what a group costs to turn into tickets, 0.43 us, is what is left.)
+  constexpr uint32_t kGroups = 4;
   auto fetch_group_untracked = [&](u32x4& sc, uint32_t& ax, uint64_t s_g) {
     const uint8_t* entry = reinterpret_cast<const uint8_t*>(&ctl->ring[(s_g + k_of_lane) & ring_mask]) + 16 * (lane & 3);
     const uint32_t* at = lane < kPollEntries       ? &jobs_done[(s_g + lane) & ring_mask]
@@ -364,21 +367,21 @@ __device__ __attribute__((noinline)) StormEnd leader_storm(HostCtl* ctl_in, DevS
   // 4 while the loop feeds (four groups in flight); once it has caught up with the host, the groups still in flight
   // that have not gone through: 3, 2, 1, and at 0 the storm is over.
   uint32_t feeding = kGroups;
-  u32x4 sc0, sc1, sc2, sc3;
-  uint32_t ax0, ax1, ax2, ax3, tickets_done;
-  fetch_group_untracked(sc0, ax0, s);
-  fetch_group_untracked(sc1, ax1, s + kPollEntries);
-  fetch_group_untracked(sc2, ax2, s + 2 * kPollEntries);
-  fetch_group_untracked(sc3, ax3, s + 3 * kPollEntries);
+  u32x4 sc[kGroups];
+  uint32_t ax[kGroups], tickets_done;
+#pragma unroll
+  for (uint32_t g = 0; g < kGroups; ++g) fetch_group_untracked(sc[g], ax[g], s + g * kPollEntries);
   asm volatile("global_load_dword %0, %1, off sc0 sc1" : "=v"(tickets_done) : "v"(reinterpret_cast<const uint32_t*>(&st->tickets_done)) : "memory");
-  asm volatile("s_waitcnt vmcnt(0)" : "+v"(sc0), "+v"(sc1), "+v"(sc2), "+v"(sc3), "+v"(ax0), "+v"(ax1), "+v"(ax2), "+v"(ax3), "+v"(tickets_done) : : "memory");
+  asm volatile("s_waitcnt vmcnt(0)" : "+v"(tickets_done) : : "memory");
+#pragma unroll
+  for (uint32_t g = 0; g < kGroups; ++g) asm volatile("" : "+v"(sc[g]), "+v"(ax[g]) : : "memory");
   tickets_done = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(tickets_done)));
   // One group through; false when the storm is over: nothing more in flight, or the group was not there whole or not
   // all of one ticket each (then whatever is in flight is dropped, and the leader's next poll asks again).
   auto pass = [&](u32x4& sc, uint32_t& ax) {
     // (While the loop feeds, the three steps before this one all fed: it stops feeding once and for all.  The first
     // four groups have landed, whichever wait they get.)
-    if (feeding == kGroups) asm volatile("s_waitcnt vmcnt(12)" : : : "memory");
+    if (feeding == kGroups) asm volatile("s_waitcnt vmcnt(%0)" : : "n"((kGroups - 1) * 4) : "memory");
     else asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
     asm volatile("" : "+v"(sc), "+v"(ax) : : "memory");
     const uint64_t s_g = s + consumed;
@@ -411,13 +414,16 @@ __device__ __attribute__((noinline)) StormEnd leader_storm(HostCtl* ctl_in, DevS
     feeding = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(feeding)));
     return feeding != 0;
   };
+  auto round = [&]() {
+#pragma unroll
+    for (uint32_t g = 0; g < kGroups; ++g)
+      if (!pass(sc[g], ax[g])) return false;
+    return true;
+  };
 #pragma unroll 1
   for (;;) {
-    if (!pass(sc0, ax0)) break;
-    if (!pass(sc1, ax1)) break;
-    if (!pass(sc2, ax2)) break;
-    if (!pass(sc3, ax3)) break;
-    // 64 entries on: the host learns of it, and the counts of this launch take them as one more poll of 64
+    if (!round()) break;
+    // a round of entries on: the host learns of it, and the counts of this launch take them as one more poll
     s += consumed;
     entries += consumed;
     consumed = 0;
@@ -425,7 +431,9 @@ __device__ __attribute__((noinline)) StormEnd leader_storm(HostCtl* ctl_in, DevS
     ++rounds;
   }
   // Whatever is still in flight is waited for, so that the registers it lands in are free.
-  asm volatile("s_waitcnt vmcnt(0)" : "+v"(sc0), "+v"(sc1), "+v"(sc2), "+v"(sc3), "+v"(ax0), "+v"(ax1), "+v"(ax2), "+v"(ax3) : : "memory");
+  asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+#pragma unroll
+  for (uint32_t g = 0; g < kGroups; ++g) asm volatile("" : "+v"(sc[g]), "+v"(ax[g]) : : "memory");
   if (consumed != 0) {  // the round that the storm ended in
     s += consumed;
     entries += consumed;
