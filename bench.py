@@ -568,7 +568,7 @@ def main():
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "traffic": round(2.0 * launch_payload * TRAFFIC_PER_ALGORITHMIC_BYTE),
             "traffic_source": "FETCH_SIZE and WRITE_SIZE of this kernel on this workload (two rocprofv3 --pmc runs, scaled by "
-            "the same counters on the plain copy kernel: x1.99975 and x1.0) came to %.4f x the algorithmic bytes; "
+            "the same counters on the plain copy kernel: x1.99977 and x1.0) came to %.4f x the algorithmic bytes; "
             "that ratio times bytes_per_launch" % TRAFFIC_PER_ALGORITHMIC_BYTE,
             "bytes_per_launch": 2.0 * launch_payload,
             "steps_per_launch": steps_per_launch,
