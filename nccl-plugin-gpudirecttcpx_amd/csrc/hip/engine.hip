@@ -137,7 +137,7 @@ constexpr uint32_t kPollEntries = 16;  // submission entries fetched per load in
 // four loads in flight together, 64 entries for the one PCIe round trip (about 1.5 us) that sixteen cost -- which
 // is what capped a storm of one-ticket requests near 9 M/s.
 constexpr uint32_t kDeepGroups = 3;    // groups of kPollEntries beyond the first in a deep poll
-constexpr uint32_t kStormBacklog = 256;  // entries published beyond a poll's 64 from which the leader takes them in a rolling loop
+constexpr uint32_t kStormBacklog = 128;  // entries published beyond a poll's 64 from which the leader takes them in a rolling loop
 constexpr uint32_t kAuxProbe = 35;  // lane of an auxiliary load that reads the stamp of an entry ahead
 constexpr uint32_t kAuxTicketsDone = 32, kAuxHostStop = 33, kAuxJobsCompleted = 34;  // lanes of the auxiliary load
 constexpr uint32_t kNeverIdleOut = 0xFFFFFFFFu;
@@ -296,6 +296,13 @@ __device__ __forceinline__ uint32_t write_single_tickets_of_group(DevState* st, 
   return run;
 }
 
+// Every lane takes the value that lane q of its own group of four holds: one move, no trip through the LDS.
+template <int q>
+__device__ __forceinline__ uint32_t quad_value(uint32_t v) {
+  static_assert(q >= 0 && q < 4, "a lane of the quad");
+  return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), q * 0x55, 0xF, 0xF, false));
+}
+
 __device__ __forceinline__ uint64_t same_in_all_lanes64(uint64_t v) {
   return (static_cast<uint64_t>(static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(v >> 32)))) << 32) |
          static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(v)));
@@ -312,7 +319,7 @@ __device__ __forceinline__ T* same_in_all_lanes_ptr(T* p) {
 // group 64 entries on at once (every group's loads bring the stamp of the last entry of the group that would be asked
 // for next: entries are published in order, so if that one is there the whole group is).  The leader's time per group
 // is then a quarter of the round trip to the host's ring or what it takes to turn a group into tickets, whichever is
-// longer -- not their sum as in a poll (1024 requests of 64 KiB in flight: 21 -> 36 M requests/s).  Every group has
+// longer -- not their sum as in a poll (1024 requests of 64 KiB in flight: 21 -> 36-39 M requests/s).  Every group has
 // registers of its own (moving one that is still in flight to another register would wait for it), hence one step
 // unrolled per group, with every index into the groups' arrays a constant.  When the host's tail is reached nothing more is asked for and the
 // groups in flight go through: the loop ends with nothing in flight.
@@ -353,14 +360,18 @@ __device__ __attribute__((noinline)) StormEnd leader_storm(HostCtl* ctl_in, DevS
   const uint32_t lane = threadIdx.x;
   const uint32_t k_of_lane = lane >> 2;
   uint32_t consumed = 0, entries = 0, rounds = 0;
-  // Groups in flight.  (Six: 1024 requests of 64 KiB in flight 35.6 -> 36.9 M/s, 512 in flight 32 -> 28 M/s: with four
-  // the round trip is hidden already and what a group costs to turn into tickets, 0.43 us, is what is left.)
+  // Groups in flight.  (Five and six: 1024 requests of 64 KiB in flight 39.5 -> 40.7 and 41.2 M/s, 384 in flight 26.5 ->
+  // 26.0 and 25.2 M/s: with four the round trip is nearly hidden already and what a group costs to turn into tickets,
+  // 0.4 us, is what is left.)
   constexpr uint32_t kGroups = 4;
   auto fetch_group_untracked = [&](u32x4& sc, uint32_t& ax, uint64_t s_g) {
     const uint8_t* entry = reinterpret_cast<const uint8_t*>(&ctl->ring[(s_g + k_of_lane) & ring_mask]) + 16 * (lane & 3);
-    const uint32_t* at = lane < kPollEntries       ? &jobs_done[(s_g + lane) & ring_mask]
-                         : lane < 2 * kPollEntries ? &job_target[(s_g + lane - kPollEntries) & ring_mask]
-                                                   : &ctl->ring[(s_g + (kGroups + 1) * kPollEntries - 1) & ring_mask].w[15];  // (lane 35's probe; the others repeat it)
+    // The four lanes that hold an entry's sectors also fetch what is known of its job slot -- tickets counted as
+    // done, tickets ever issued -- so that both reach all four with a move inside the quad; the other two lanes read
+    // the stamp of the last entry of the group that would be asked for next (the probe).
+    const uint32_t* at = (lane & 3) == 0   ? &jobs_done[(s_g + k_of_lane) & ring_mask]
+                         : (lane & 3) == 1 ? &job_target[(s_g + k_of_lane) & ring_mask]
+                                           : &ctl->ring[(s_g + (kGroups + 1) * kPollEntries - 1) & ring_mask].w[15];
     asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(sc) : "v"(entry) : "memory");
     asm volatile("global_load_dword %0, %1, off sc0 sc1" : "=v"(ax) : "v"(at) : "memory");
   };
@@ -393,11 +404,11 @@ __device__ __attribute__((noinline)) StormEnd leader_storm(HostCtl* ctl_in, DevS
       // ticket_size_for_submission; a fixed ticket size says so itself): no sizing here, and a group with a larger
       // one ends the storm and goes the ordinary way.
       EntryView more;
-      more.n = bcast(sc.y, lane | 3u);
+      more.n = quad_value<3>(sc.y);  // payload word 10 sits in .y of sector 3
       more.bytes = 0, more.per_ticket = 0, more.in_flight = 0;  // (not looked at by write_single_tickets_of_group)
-      more.target_prev = bcast(ax, kPollEntries + k_of_lane);
+      more.target_prev = quad_value<1>(ax);
       more.sane = ((okm >> (4 * k_of_lane)) & 0xFull) == 0xFull && more.n - 1u < kMaxDescsPerSubmission;
-      more.slot_free = bcast(ax, k_of_lane) == more.target_prev;
+      more.slot_free = quad_value<0>(ax) == more.target_prev;
       more.slot = static_cast<uint32_t>(s_g + k_of_lane) & ring_mask;
       const uint32_t one_ticket = fixed_per_ticket != 0 ? fixed_per_ticket : kSmallSubmission;
       if (__ballot(more.sane && more.n > one_ticket) == 0) run = write_single_tickets_of_group(st, job_target, stamps, tickets_out, lane, more, sc, left);
@@ -406,7 +417,7 @@ __device__ __attribute__((noinline)) StormEnd leader_storm(HostCtl* ctl_in, DevS
     if (run != kPollEntries) return false;
     if (feeding == kGroups) {
       const uint64_t next = s_g + kGroups * kPollEntries;
-      if (lane_value(ax, kAuxProbe) == static_cast<uint32_t>(next + kPollEntries)) fetch_group_untracked(sc, ax, next);
+      if (lane_value(ax, 2) == static_cast<uint32_t>(next + kPollEntries)) fetch_group_untracked(sc, ax, next);
       else feeding = kGroups - 1;
     } else {
       --feeding;
