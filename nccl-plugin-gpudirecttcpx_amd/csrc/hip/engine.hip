@@ -380,13 +380,17 @@ __device__ __attribute__((noinline)) StormEnd leader_storm(HostCtl* ctl_in, DevS
   uint32_t feeding = kGroups;
   u32x4 sc[kGroups];
   uint32_t ax[kGroups], tickets_done;
+  // The first groups, from s on, and the running count of finished tickets: one round trip, waited for whole.
+  auto arm = [&]() {
+    feeding = kGroups;
 #pragma unroll
-  for (uint32_t g = 0; g < kGroups; ++g) fetch_group_untracked(sc[g], ax[g], s + g * kPollEntries);
-  asm volatile("global_load_dword %0, %1, off sc0 sc1" : "=v"(tickets_done) : "v"(reinterpret_cast<const uint32_t*>(&st->tickets_done)) : "memory");
-  asm volatile("s_waitcnt vmcnt(0)" : "+v"(tickets_done) : : "memory");
+    for (uint32_t g = 0; g < kGroups; ++g) fetch_group_untracked(sc[g], ax[g], s + g * kPollEntries);
+    asm volatile("global_load_dword %0, %1, off sc0 sc1" : "=v"(tickets_done) : "v"(reinterpret_cast<const uint32_t*>(&st->tickets_done)) : "memory");
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(tickets_done) : : "memory");
 #pragma unroll
-  for (uint32_t g = 0; g < kGroups; ++g) asm volatile("" : "+v"(sc[g]), "+v"(ax[g]) : : "memory");
-  tickets_done = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(tickets_done)));
+    for (uint32_t g = 0; g < kGroups; ++g) asm volatile("" : "+v"(sc[g]), "+v"(ax[g]) : : "memory");
+    tickets_done = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(tickets_done)));
+  };
   // One group through; false when the storm is over: nothing more in flight, or the group was not there whole or not
   // all of one ticket each (then whatever is in flight is dropped, and the leader's next poll asks again).
   auto pass = [&](u32x4& sc, uint32_t& ax) {
@@ -433,23 +437,34 @@ __device__ __attribute__((noinline)) StormEnd leader_storm(HostCtl* ctl_in, DevS
   };
 #pragma unroll 1
   for (;;) {
-    if (!round()) break;
-    // a round of entries on: the host learns of it, and the counts of this launch take them as one more poll
-    s += consumed;
-    entries += consumed;
-    consumed = 0;
-    if (lane == 0) sys_store(&ctl->head, s);
-    ++rounds;
-  }
-  // Whatever is still in flight is waited for, so that the registers it lands in are free.
-  asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+    arm();
+#pragma unroll 1
+    for (;;) {
+      if (!round()) break;
+      // a round of entries on: the host learns of it, and the counts of this launch take them as one more poll
+      s += consumed;
+      entries += consumed;
+      consumed = 0;
+      if (lane == 0) sys_store(&ctl->head, s);
+      ++rounds;
+    }
+    // Whatever is still in flight is waited for, so that the registers it lands in are free.
+    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
 #pragma unroll
-  for (uint32_t g = 0; g < kGroups; ++g) asm volatile("" : "+v"(sc[g]), "+v"(ax[g]) : : "memory");
-  if (consumed != 0) {  // the round that the storm ended in
-    s += consumed;
-    entries += consumed;
-    if (lane == 0) sys_store(&ctl->head, s);
-    ++rounds;
+    for (uint32_t g = 0; g < kGroups; ++g) asm volatile("" : "+v"(sc[g]), "+v"(ax[g]) : : "memory");
+    if (consumed != 0) {  // the round that the loop ended in
+      s += consumed;
+      entries += consumed;
+      consumed = 0;
+      if (lane == 0) sys_store(&ctl->head, s);
+      ++rounds;
+    }
+    // Caught up with the host, every group in flight gone through whole (64 entries at the least since the loop was
+    // armed): the host publishes as requests complete, so more is on its way -- ask again from here instead of
+    // leaving, waiting for the ordinary loop to find 64 entries and as many again beyond them, and coming back.
+    // Anything else -- a group not there whole, entries of more than one ticket, no room in the ticket ring --
+    // is for the ordinary loop.
+    if (feeding != 0) break;
   }
   return StormEnd{s, tickets_out, entries, rounds};
 }
@@ -1400,7 +1415,7 @@ int tcpxuEngineCreate(int device, const tcpxuEngineConfig* config, tcpxuEngine**
       break;
     }
     e->jobs_done = reinterpret_cast<uint32_t*>(reinterpret_cast<uint8_t*>(e->st) + sizeof(DevState));
-    e->job_target = e->jobs_done + cfg.ring_entries;
+    e->job_target = e->jobs_done + cfg.ring_entries;  // (leader_storm works the second out from the first)
     // Test aid: where the engine's counts of submissions and tickets start.  Records are stamped with the low 32 bits
     // of their sequence number, and a busy engine passes 2^32 submissions within the hour; a test that starts just
     // below sees the crossing in milliseconds.  (Start more than a lap of the ticket ring below: a slot of either ring
