@@ -204,7 +204,8 @@ int tcpxuEngineGetStats(tcpxuEngine* engine, tcpxuEngineStats* stats);
  * workgroup that completed it had its last store acknowledged.  tcpxuEngineReadStamps (engine stopped) copies the
  * readings of submissions first_submission .. +n (counted from the engine's creation; n at most ring_entries, and
  * only the last ring_entries submissions are kept) into out[4 * n] and clears them.  A reading of all ones means
- * "never taken". */
+ * "never taken".  Readings [1] and [2] are kept as minima and only reading clears them: read at least once every
+ * ring_entries submissions, or they may be those of the submission that had the same place in the ring before. */
 int tcpxuEngineEnableStamps(tcpxuEngine* engine, double* ticks_per_us);
 int tcpxuEngineReadStamps(tcpxuEngine* engine, uint64_t first_submission, uint32_t n, uint64_t* out);
 

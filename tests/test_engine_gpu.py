@@ -562,21 +562,27 @@ def test_engine_storm_of_mixed_small_submissions(pkg, hip, oracle, depth, benchl
     assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
 
 
-@pytest.mark.parametrize("count_from", [0, (1 << 32) - 70000])
-def test_engine_long_runs_of_one_ticket_submissions_broken_by_others(pkg, hip, oracle, benchlib, monkeypatch, count_from):
+@pytest.mark.parametrize("count_from,with_stamps", [(0, False), (0, True), ((1 << 32) - 70000, False)])
+def test_engine_long_runs_of_one_ticket_submissions_broken_by_others(pkg, hip, oracle, benchlib, monkeypatch, count_from, with_stamps):
     """1024 in flight (a slot of the stream then holds up to 64 descriptors), nearly all of one ticket: with hundreds
     of entries published ahead of it the leader takes them in its rolling loop, four groups of sixteen in flight, and
     every few hundred entries an empty submission, one just over a ticket or one of two tickets ends that loop and
     goes the ordinary way.  Every byte must be the oracle's, every submission consumed exactly once -- also when the
     32-bit stamps of tickets and entries wrap in the middle of it (an engine that starts 70000 below 2^32: more than a
-    lap of the ticket ring, because a ring slot that was never written reads as the stamp of sequence number 2^32-1)."""
+    lap of the ticket ring, because a ring slot that was never written reads as the stamp of sequence number 2^32-1),
+    and with the kernel's clock stamps switched on (the rolling loop then issues one more store per group, which the
+    count it waits by must survive; the four stamps of each of the last 2048 submissions must be there and in order)."""
     assert abs(sum(STORM_MOSTLY_ONE_TICKET) - 1) < 1e-9
-    pool_d, dst_d, items, expect, descs = storm_workload(pkg, oracle, 0x5709 + (count_from & 0xFF), 8000, STORM_MOSTLY_ONE_TICKET)
+    # (with stamps: fewer submissions than the ring has entries, so that no place in the ring is stamped twice)
+    pool_d, dst_d, items, expect, descs = storm_workload(pkg, oracle, 0x5709 + (count_from & 0xFF), 4000 if with_stamps else 8000, STORM_MOSTLY_ONE_TICKET)
     if count_from:
         monkeypatch.setenv("TCPXU_ENGINE_COUNT_FROM", str(count_from))
     e = Engine(pkg, hip)
     monkeypatch.delenv("TCPXU_ENGINE_COUNT_FROM", raising=False)
     assert e.completed() == count_from
+    rate = ctypes.c_double()
+    if with_stamps:
+        pkg.check(hip.tcpxuEngineEnableStamps(e.h, ctypes.byref(rate)), "tcpxuEngineEnableStamps")
     launches = 70000 // len(items) + 3 if count_from else 1
     print("engine rolling-loop case: count_from=%d launches=%d submissions each=%d descriptors=%d" % (count_from, launches, len(items), len(descs)), flush=True)  # fmt: skip
     wall, kern = ctypes.c_double(), ctypes.c_double()
@@ -594,6 +600,19 @@ def test_engine_long_runs_of_one_ticket_submissions_broken_by_others(pkg, hip, o
         got = dst_d.cpu().numpy()
         assert first_difference(got, expect) is None, "launch %d, first (index, got, want, count): %r" % (launch, first_difference(got, expect))
     assert not count_from or e.completed() > (1 << 32)
+    if with_stamps:
+        last = 2048
+        out = (ctypes.c_uint64 * (4 * last))()
+        pkg.check(hip.tcpxuEngineReadStamps(e.h, len(items) - last, last, out), "tcpxuEngineReadStamps")
+        for i in range(last):
+            t = [out[4 * i + k] for k in range(4)]
+            if items[len(items) - last + i].n_descs == 0:
+                continue  # completed by the leader itself: no workgroup ever stamps it
+            # [0] is the leader's reading and the others a workgroup's, on another compute unit whose clock may differ by
+            # a few ticks: a workgroup that was already looking for the ticket can have it within that.
+            slack = 0.5 * rate.value
+            assert 0xFFFFFFFFFFFFFFFF not in t and t[0] <= t[1] + slack and t[1] <= t[2] <= t[3], (len(items) - last + i, t)
+            assert (t[3] - t[0]) / rate.value < 1e6, "microseconds, not a second"
     e.destroy()
 
 
