@@ -315,25 +315,26 @@ __device__ __forceinline__ T* same_in_all_lanes_ptr(T* p) {
 // A storm: a deep poll turned all its 64 entries into tickets and the host has published kStormBacklog entries beyond
 // them.  Takes entries from s on for as long as they are published and are one ticket each; returns where it got to.
 //
-// Four groups of sixteen entries are in flight at a time, and the registers of a group that has gone through take the
-// group 64 entries on at once (every group's loads bring the stamp of the last entry of the group that would be asked
-// for next: entries are published in order, so if that one is there the whole group is).  The leader's time per group
-// is then a quarter of the round trip to the host's ring or what it takes to turn a group into tickets, whichever is
-// longer -- not their sum as in a poll (1024 requests of 64 KiB in flight: 21 -> 36-39 M requests/s).  Every group has
-// registers of its own (moving one that is still in flight to another register would wait for it), hence one step
-// unrolled per group, with every index into the groups' arrays a constant.  When the host's tail is reached nothing more is asked for and the
-// groups in flight go through: the loop ends with nothing in flight.
+// kGroups (five) groups of sixteen entries are in flight at a time, and the registers of a group that has gone through
+// take the group 16 x kGroups entries on at once (every group's loads bring the stamp of the last entry of the group
+// that would be asked for next: entries are published in order, so if that one is there the whole group is).  The
+// leader's time per group is then a fifth of the round trip to the host's ring or what it takes to turn a group into
+// tickets, whichever is longer -- not their sum as in a poll (1024 requests of 64 KiB in flight: 21 -> 44 M
+// requests/s, where the copy itself becomes the bound).  Every group has registers of its own (moving one that is
+// still in flight to another register would wait for it), hence one step unrolled per group, with every index into
+// the groups' arrays a constant.  When the host's tail is reached nothing more is asked for and the groups in flight
+// go through: the loop ends with nothing in flight.
 //
 // The compiler would wait for everything in flight at the top of such a loop.  So the loop's loads are written as
 // instructions, which it does not track, and each step waits for its own group by count: the memory instructions of
-// a wavefront complete in the order issued, and between a group's loads and its turn three other groups have had
-// theirs, each with two stores (the tickets, their job slots' targets) and, while the loop feeds, two loads: twelve
-// instructions at the least, so "at most twelve outstanding" means that the group's own loads have landed.  (More
-// are issued when stamps are on, and the head word once a round: counting too few only waits for a little more than
-// is needed; fewer would let a group be read before it has landed, so this function must not spill registers to
-// memory -- the compiler's resource report for the kernel says 0 bytes of scratch.)  Once the loop has stopped
-// feeding, a group waits for everything.  The group's registers pass through a statement after the wait so that
-// nothing reads them before it.
+// a wavefront complete in the order issued, and between a group's loads and its turn the other kGroups - 1 groups
+// have had theirs, each with two stores (the tickets, their job slots' targets) and, while the loop feeds, two loads:
+// 4 x (kGroups - 1) instructions at the least, so "at most that many outstanding" means that the group's own loads
+// have landed.  (More are issued when stamps are on, and the head word once a round: counting too few only waits for
+// a little more than is needed; fewer would let a group be read before it has landed, so this function must not
+// spill registers to memory -- the build checks the compiler's resource report for 0 bytes of scratch.)  Once the
+// loop has stopped feeding, a group waits for everything.  The group's registers pass through a statement after the
+// wait so that nothing reads them before it.
 //
 // A function of its own, not inlined, and called from the top of the leader's loop where little is live: with this
 // loop inside the leader's, what the compiler did with the registers around it made every poll that never sees a
@@ -341,7 +342,7 @@ __device__ __forceinline__ T* same_in_all_lanes_ptr(T* p) {
 // storm early (after at most kTicketRing entries, which is also how long the host's stop word can go unread).
 struct StormEnd {
   uint64_t s, tickets_out;
-  uint32_t entries, rounds;  // entries taken off the ring, in so many rounds of up to 64
+  uint32_t entries;  // taken off the ring
 };
 __device__ __attribute__((noinline)) StormEnd leader_storm(HostCtl* ctl_in, DevState* st_in, uint32_t* jobs_done_in,
                                                           uint64_t* stamps_in, uint32_t ring_mask_in,
@@ -359,24 +360,34 @@ __device__ __attribute__((noinline)) StormEnd leader_storm(HostCtl* ctl_in, DevS
   uint64_t tickets_out = same_in_all_lanes64(tickets_out_in);
   const uint32_t lane = threadIdx.x;
   const uint32_t k_of_lane = lane >> 2;
-  uint32_t consumed = 0, entries = 0, rounds = 0;
-  // Groups in flight.  (Five and six: 1024 requests of 64 KiB in flight 39.5 -> 40.7 and 41.2 M/s, 384 in flight 26.5 ->
-  // 26.0 and 25.2 M/s: with four the round trip is nearly hidden already and what a group costs to turn into tickets,
-  // 0.4 us, is what is left.)
-  constexpr uint32_t kGroups = 4;
+  uint32_t consumed = 0, entries = 0;
+  // Groups in flight: the round trip to the host's ring, 1.55 us, over what a group costs to turn into tickets, 0.36 us,
+  // and one more.  (1024 requests of 64 KiB in flight: 40.3 M/s with four, 44.6 with five -- where the copy itself is
+  // the bound -- and 45.5 with six, which spills registers; 384 in flight: 29.4, 27.2, 26.4.)
+  constexpr uint32_t kGroups = 5;
+  // The four lanes that hold an entry's sectors also fetch what is known of its job slot -- tickets counted as done
+  // (first lane), tickets ever issued (second) -- so that both reach all four with a move inside the quad; the other two
+  // lanes read the stamp of the last entry of the group that would be asked for next (the probe).  What of a lane's two
+  // addresses does not change from group to group is worked out once (and hidden from the compiler, which would work
+  // it out again with a branch per kind of lane in every step): address = base + (((s_g + add) & ring_mask) << shift).
+  const uint32_t kind = lane & 3;
+  uint64_t entry_base = reinterpret_cast<uint64_t>(&ctl->ring[0]) + 16 * kind;
+  uint64_t aux_base = kind == 0   ? reinterpret_cast<uint64_t>(jobs_done)
+                      : kind == 1 ? reinterpret_cast<uint64_t>(job_target)
+                                  : reinterpret_cast<uint64_t>(&ctl->ring[0].w[15]);
+  uint32_t aux_add = kind < 2 ? k_of_lane : (kGroups + 1) * kPollEntries - 1;
+  uint32_t aux_shift = kind < 2 ? 2 : 6;
+  static_assert(sizeof(Record) == 64 && sizeof(uint32_t) == 4, "the shifts above");
+  asm volatile("" : "+v"(entry_base), "+v"(aux_base), "+v"(aux_add), "+v"(aux_shift));
   auto fetch_group_untracked = [&](u32x4& sc, uint32_t& ax, uint64_t s_g) {
-    const uint8_t* entry = reinterpret_cast<const uint8_t*>(&ctl->ring[(s_g + k_of_lane) & ring_mask]) + 16 * (lane & 3);
-    // The four lanes that hold an entry's sectors also fetch what is known of its job slot -- tickets counted as
-    // done, tickets ever issued -- so that both reach all four with a move inside the quad; the other two lanes read
-    // the stamp of the last entry of the group that would be asked for next (the probe).
-    const uint32_t* at = (lane & 3) == 0   ? &jobs_done[(s_g + k_of_lane) & ring_mask]
-                         : (lane & 3) == 1 ? &job_target[(s_g + k_of_lane) & ring_mask]
-                                           : &ctl->ring[(s_g + (kGroups + 1) * kPollEntries - 1) & ring_mask].w[15];
+    const uint32_t at_s = static_cast<uint32_t>(s_g);  // (the mask keeps low bits only)
+    const uint64_t entry = entry_base + (static_cast<uint64_t>((at_s + k_of_lane) & ring_mask) << 6);
+    const uint64_t at = aux_base + (static_cast<uint64_t>((at_s + aux_add) & ring_mask) << aux_shift);
     asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(sc) : "v"(entry) : "memory");
     asm volatile("global_load_dword %0, %1, off sc0 sc1" : "=v"(ax) : "v"(at) : "memory");
   };
-  // 4 while the loop feeds (four groups in flight); once it has caught up with the host, the groups still in flight
-  // that have not gone through: 3, 2, 1, and at 0 the storm is over.
+  // kGroups while the loop feeds (that many groups in flight); once it has caught up with the host, the groups still
+  // in flight that have not gone through: kGroups - 1, ..., 1, and at 0 the storm is over.
   uint32_t feeding = kGroups;
   u32x4 sc[kGroups];
   uint32_t ax[kGroups], tickets_done;
@@ -394,8 +405,8 @@ __device__ __attribute__((noinline)) StormEnd leader_storm(HostCtl* ctl_in, DevS
   // One group through; false when the storm is over: nothing more in flight, or the group was not there whole or not
   // all of one ticket each (then whatever is in flight is dropped, and the leader's next poll asks again).
   auto pass = [&](u32x4& sc, uint32_t& ax) {
-    // (While the loop feeds, the three steps before this one all fed: it stops feeding once and for all.  The first
-    // four groups have landed, whichever wait they get.)
+    // (While the loop feeds, the kGroups - 1 steps before this one all fed: it stops feeding once and for all.  The
+    // first groups have landed, whichever wait they get.)
     if (feeding == kGroups) asm volatile("s_waitcnt vmcnt(%0)" : : "n"((kGroups - 1) * 4) : "memory");
     else asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
     asm volatile("" : "+v"(sc), "+v"(ax) : : "memory");
@@ -441,12 +452,11 @@ __device__ __attribute__((noinline)) StormEnd leader_storm(HostCtl* ctl_in, DevS
 #pragma unroll 1
     for (;;) {
       if (!round()) break;
-      // a round of entries on: the host learns of it, and the counts of this launch take them as one more poll
+      // a round of entries on: the host learns of it
       s += consumed;
       entries += consumed;
       consumed = 0;
       if (lane == 0) sys_store(&ctl->head, s);
-      ++rounds;
     }
     // Whatever is still in flight is waited for, so that the registers it lands in are free.
     asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
@@ -457,16 +467,15 @@ __device__ __attribute__((noinline)) StormEnd leader_storm(HostCtl* ctl_in, DevS
       entries += consumed;
       consumed = 0;
       if (lane == 0) sys_store(&ctl->head, s);
-      ++rounds;
     }
-    // Caught up with the host, every group in flight gone through whole (64 entries at the least since the loop was
-    // armed): the host publishes as requests complete, so more is on its way -- ask again from here instead of
+    // Caught up with the host, every group in flight gone through whole (16 x kGroups entries at the least since the
+    // loop was armed): the host publishes as requests complete, so more is on its way -- ask again from here instead of
     // leaving, waiting for the ordinary loop to find 64 entries and as many again beyond them, and coming back.
     // Anything else -- a group not there whole, entries of more than one ticket, no room in the ticket ring --
     // is for the ordinary loop.
     if (feeding != 0) break;
   }
-  return StormEnd{s, tickets_out, entries, rounds};
+  return StormEnd{s, tickets_out, entries};
 }
 
 __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uint32_t* job_target,
@@ -500,15 +509,15 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
   const uint32_t* const jobs_completed_lo = reinterpret_cast<const uint32_t*>(&st->jobs_completed);
 
   for (;;) {
-    // (Its rounds of 64 count as deep polls in this launch's figures.)
+    // (Every 64 entries it takes count as one deep poll in this launch's figures.)
     if (storm_next) {
       storm_next = false;
       const StormEnd end = leader_storm(ctl, st, jobs_done, stamps, ring_mask, fixed_per_ticket, s, tickets_out);
       s = same_in_all_lanes(end.s);
       tickets_out = same_in_all_lanes(end.tickets_out);
       entries += end.entries;
-      polls += end.rounds;
-      deep_polls += end.rounds;
+      polls += (end.entries + (kDeepGroups + 1) * kPollEntries - 1) / ((kDeepGroups + 1) * kPollEntries);
+      deep_polls += (end.entries + (kDeepGroups + 1) * kPollEntries - 1) / ((kDeepGroups + 1) * kPollEntries);
       deep = ring_allows_deep;
     }
     // What depends on the lane is worked out afresh in every pass (the empty statement hides from the compiler that
