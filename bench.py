@@ -713,7 +713,7 @@ def main():
             "requests_timed": n_storm * (storm_reps - 1),
             "latency": "publish of a request's slot -> host poller observes its completion word",
             "leader": "a poll fetches 16 submission entries, 64 after a poll that found all sixteen; with 192 or more published "
-            "ahead the leader keeps four groups of sixteen in flight instead, and each round of up to 64 entries counts as a poll of 64",
+            "ahead the leader keeps five groups of sixteen in flight instead, and every 64 entries taken that way count as a poll of 64",
             "best": {k: best[k] for k in ("requests_in_flight", "requests_per_s", "payload_GBps")},
             "sweep": sweep,
         }

@@ -186,8 +186,8 @@ int tcpxuEngineCompleted(tcpxuEngine* engine, uint64_t* completed);
 /* Counters since creation.  The leader's are written by the kernel when it leaves (stop or idle exit), so they
  * are current after tcpxuEngineStop: polls of the submission ring, entries those polls consumed, and how many of
  * the polls fetched 64 entries instead of 16 (the leader does that after a poll that found all sixteen there; with
- * hundreds of entries published ahead of it the leader keeps four groups of sixteen in flight instead of polling,
- * and every round of up to 64 entries taken that way counts as one such poll). */
+ * hundreds of entries published ahead of it the leader keeps several groups of sixteen in flight instead of
+ * polling, and every 64 entries taken that way count as one such poll). */
 typedef struct tcpxuEngineStats {
   uint64_t launches;
   uint64_t submissions;
