@@ -82,7 +82,7 @@ def cpu_baseline(oracle, descs, dst_bytes, pool, threads, budget_s):
     return payload / med / 1e9, iters
 
 
-def plugin_path(pkg, hip, torch, workloads, pool, helper_thread=False, rx_bindings=None):
+def plugin_path(pkg, hip, torch, workloads, pool, helper_thread=False, rx_bindings=None, what="8 MiB chunks"):
     """The same chunks through the whole plugin (libnccl-net.so): irecv -> control messages -> synthetic recvmsg
     with its control messages -> descriptor builder -> slot -> engine -> test() -> iflush -> irecvConsumed, driven by
     the request loop inside the library.  The host builds one descriptor per fragment here, so this is a host-bound
@@ -130,7 +130,7 @@ def plugin_path(pkg, hip, torch, workloads, pool, helper_thread=False, rx_bindin
     payload = 2 * len(workloads) * chunk_bytes
     return {
         "max_slots_at_gpu": int(stats.max_slots_at_gpu),
-        "what": "8 MiB chunks through ncclNet_v7 (irecv/test/iflush/irecvConsumed) with the synthetic devmem socket, "
+        "what": what + " through ncclNet_v7 (irecv/test/iflush/irecvConsumed) with the synthetic devmem socket, "
         + ("the proxy thread plus the plugin's socket thread" if helper_thread else "one proxy thread"),
         "payload_GBps": round(payload / seconds / 1e9, 2),
         "host_ns_per_fragment": round(seconds / frags * 1e9, 1),
@@ -800,6 +800,16 @@ def main():
         # out near 46-57 GB/s or near 11 GB/s accordingly).  So it runs three times as the machine places the threads,
         # median beside all three, and once each with the proxy thread on one CPU and the socket thread bound
         # (NCCL_GPUDIRECTTCPX_RX_BINDINGS, the reference's flag for this) to the CPU nearest to it and farthest from it.
+        # The same surface fed as the reference's sender feeds it: chunks of 128 KiB, 32 fragments to the control message,
+        # the task and the recvmsg (the bulk workload: whole pages, eight flows, runs of 32 fragments per flow).  On the
+        # headline workload every fragment is a chunk of its own, because the contract interleaves its flows fragment
+        # by fragment, and the host's time per fragment is a time per task.
+        bulk = pkg.Workload(4, seed=0xC0FFEE04, shrink=1)  # 128 MiB in 32 requests of 4 MiB from a 512 MiB pool
+        bulk_pool = np.empty(int(bulk.info.pool_bytes), dtype=np.uint8)
+        bulk.fill_window(0, bulk_pool)
+        result["plugin_path"]["in_chunks_of_32_fragments"] = plugin_path(
+            pkg, hip, torch, [bulk], bulk_pool, what="a 128 MiB message of whole pages in 4 MiB requests, eight flows, chunks of 128 KiB,")
+        del bulk_pool
         some = workloads[: min(8, args.chunks)]
         legs = [plugin_path(pkg, hip, torch, some, pool, helper_thread=True) for _ in range(3)]
         legs.sort(key=lambda leg: leg.get("payload_GBps", 0.0))

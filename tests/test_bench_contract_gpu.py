@@ -81,6 +81,9 @@ def test_bench_extras_report_latency_and_the_storm_sweep():
     assert all(0 < x["leader_entries_per_poll"] <= 64 and x["leader_polls_per_us"] > 0 for x in sweep)
     assert r["storm_64KiB"]["best"]["requests_per_s"] == max(x["requests_per_s"] for x in sweep)
     assert 1 <= r["plugin_path"]["max_slots_at_gpu"] <= 16
+    # the same surface with 32 fragments to the chunk, as the reference's sender cuts a message
+    bulk = r["plugin_path"]["in_chunks_of_32_fragments"]
+    assert bulk["payload_GBps"] > 0 and 0 < bulk["host_ns_per_fragment"] and 1 <= bulk["max_slots_at_gpu"] <= 16
     assert r["single_comm"]["value"] > 0 and r["plugin_path"]["payload_GBps"] > 0 and r["plain_copy_kernel"]["rw_GBps"] > 0
     assert sorted(r["other_configs"]) == ["config_1", "config_4", "config_5"]
     assert all(v["payload_GBps"] > 0 for v in r["other_configs"].values())
