@@ -303,14 +303,22 @@ def test_engine_stream_depths(pkg, hip, oracle, depth, benchlib):
     e.destroy()
 
 
-@pytest.mark.parametrize("depth", [256, 2048])
-def test_engine_storm_of_small_requests_many_in_flight(pkg, hip, oracle, depth, benchlib):
+@pytest.mark.parametrize(
+    "depth,per_ticket,ring",
+    [(256, 0, 0), (2048, 0, 0), (2048, 16, 0), (1024, 8, 0), (256, 0, 512)],
+    ids=["256", "2048", "2048-tickets-of-16", "1024-two-tickets-each", "256-ring-of-512"],
+)
+def test_engine_storm_of_small_requests_many_in_flight(pkg, hip, oracle, depth, per_ticket, ring, benchlib):
     """The small-message storm with hundreds to 2048 requests in flight (the unpack queues of 128 comms): the
-    leader then fetches 64 submission entries per poll and turns runs of sixteen into tickets at a stroke, the host
-    publishes in batches.  Every request twice, byte-exact; every submission consumed by exactly one poll."""
+    leader then fetches 64 submission entries per poll and turns runs of sixteen into tickets at a stroke -- with
+    hundreds published ahead of it, in its rolling loop -- and the host publishes in batches.  Also with the ticket
+    size fixed at the requests' sixteen descriptors (one ticket each, as when sized by the backlog) and at eight (two
+    tickets each: none of this applies, the ordinary way with a thousand waiting), and with a submission ring of 512
+    entries, the smallest that the rolling loop takes, wrapped every 512 requests.  Every request twice, byte-exact;
+    every submission consumed by exactly one poll."""
     import torch
 
-    wl = pkg.Workload(3, seed=0x5708A + depth, shrink=1)  # 1024 requests of 16 x 4 KiB, 256 MiB pool
+    wl = pkg.Workload(3, seed=0x5708A + depth + per_ticket + ring, shrink=1)  # 1024 requests of 16 x 4 KiB, 256 MiB pool
     info = wl.info
     pool = np.empty(info.pool_bytes, dtype=np.uint8)
     wl.fill_window(0, pool)
@@ -330,8 +338,8 @@ def test_engine_storm_of_small_requests_many_in_flight(pkg, hip, oracle, depth, 
         items[i].descs_host = descs.ctypes.data + 16 * first
         items[i].n_descs = cnt
         items[i].payload_bytes = int(r["bytes"])
-    e = Engine(pkg, hip)
-    print("engine storm case: depth=%d items=%d" % (depth, 2 * n), flush=True)
+    e = Engine(pkg, hip, descs_per_ticket=per_ticket, ring_entries=ring)
+    print("engine storm case: depth=%d tickets of %d ring %d items=%d" % (depth, per_ticket, ring, 2 * n), flush=True)
     wall, kern = ctypes.c_double(), ctypes.c_double()
     lat = (ctypes.c_double * (2 * n))()
     pkg.check(benchlib.tcpxuEngineRunTimed(e.h, items, 2 * n, 0, depth, 20000, ctypes.byref(wall), ctypes.byref(kern), lat), "tcpxuEngineRunTimed")
