@@ -391,6 +391,7 @@ __device__ __attribute__((noinline)) StormEnd leader_storm(HostCtl* ctl_in, DevS
   uint32_t feeding = kGroups;
   u32x4 sc[kGroups];
   uint32_t ax[kGroups], tickets_done;
+  bool queue_deep = false;
   // The first groups, from s on, and the running count of finished tickets: one round trip, waited for whole.
   auto arm = [&]() {
     feeding = kGroups;
@@ -401,6 +402,8 @@ __device__ __attribute__((noinline)) StormEnd leader_storm(HostCtl* ctl_in, DevS
 #pragma unroll
     for (uint32_t g = 0; g < kGroups; ++g) asm volatile("" : "+v"(sc[g]), "+v"(ax[g]) : : "memory");
     tickets_done = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(tickets_done)));
+    // The first group's probe: the 16 x (kGroups + 1) entries from s on are published, so the queue at the leader is deep.
+    queue_deep = lane_value(ax[0], 2) == static_cast<uint32_t>(s + (kGroups + 1) * kPollEntries);
   };
   // One group through; false when the storm is over: nothing more in flight, or the group was not there whole or not
   // all of one ticket each (then whatever is in flight is dropped, and the leader's next poll asks again).
@@ -425,7 +428,7 @@ __device__ __attribute__((noinline)) StormEnd leader_storm(HostCtl* ctl_in, DevS
       more.sane = ((okm >> (4 * k_of_lane)) & 0xFull) == 0xFull && more.n - 1u < kMaxDescsPerSubmission;
       more.slot_free = quad_value<0>(ax) == more.target_prev;
       more.slot = static_cast<uint32_t>(s_g + k_of_lane) & ring_mask;
-      const uint32_t one_ticket = fixed_per_ticket != 0 ? fixed_per_ticket : kSmallSubmission;
+      const uint32_t one_ticket = fixed_per_ticket != 0 ? fixed_per_ticket : queue_deep ? kMaxDescsPerTicket : kSmallSubmission;
       if (__ballot(more.sane && more.n > one_ticket) == 0) run = write_single_tickets_of_group(st, job_target, stamps, tickets_out, lane, more, sc, left);
     }
     consumed += run;
@@ -497,6 +500,7 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
   // The next poll fetches 64 entries.  (A ring of fewer entries than that never has them.)
   bool deep = false;
   bool storm_next = false;
+  uint32_t storm_backoff = 0, storm_backoff_len = 4;  // polls until the rolling loop is next tried from the several-tickets way
   const bool ring_allows_deep = ring_mask + 1u >= (kDeepGroups + 1) * kPollEntries;
   const bool ring_allows_storm = ring_mask + 1u >= 2 * ((kDeepGroups + 1) * kPollEntries + kStormBacklog);
   // Fixed per-lane roles in the auxiliary load (second load of every poll), so that both loads of a poll are
@@ -519,6 +523,12 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
       polls += (end.entries + (kDeepGroups + 1) * kPollEntries - 1) / ((kDeepGroups + 1) * kPollEntries);
       deep_polls += (end.entries + (kDeepGroups + 1) * kPollEntries - 1) / ((kDeepGroups + 1) * kPollEntries);
       deep = ring_allows_deep;
+      // Nothing taken: the queue was not deep, or what waits is not for that loop.  Wait longer each time before
+      // asking again (an attempt costs a round trip), and start over once it has worked.
+      storm_backoff_len = end.entries != 0 ? 4u : std::min(2u * storm_backoff_len, 256u);
+      storm_backoff = end.entries != 0 ? 0u : storm_backoff_len;
+    } else if (storm_backoff != 0) {
+      --storm_backoff;
     }
     // What depends on the lane is worked out afresh in every pass (the empty statement hides from the compiler that
     // the lane is the same each time): a dozen per-lane addresses kept in registers for the life of the loop are
@@ -703,6 +713,9 @@ __device__ void leader_loop(HostCtl* ctl, DevState* st, uint32_t* jobs_done, uin
           }
           tickets_out += static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(total)));
           consumed = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(run)));
+          // Sixteen entries of a few tickets each, the first of them of no more descriptors than one ticket holds: if
+          // hundreds more wait, the rolling loop makes one ticket of each such entry (asked once in a while).
+          storm_next = consumed == kPollEntries && n_first <= kMaxDescsPerTicket && ring_allows_storm && storm_backoff == 0;
         }
       }
     }

@@ -513,6 +513,11 @@ STORM_MIXED = [.05, .1, .05, .05, .1, .05, .05, .2, .05, .05, .1, .03, .03, .03,
 STORM_MOSTLY_ONE_TICKET = [.001, .1, .05, .05, .1, .05, .05, .3, .05, .05, .196, .001, .001, .001, 0, 0]
 
 
+# Mostly just over one ticket of the usual size and up to what one ticket can hold (33, 40, 64 descriptors), some of one
+# ticket anyway, a few empty.
+STORM_UP_TO_64 = [.005, .02, 0, 0, .05, 0, 0, .1, 0, 0, .1, .25, .25, .225, 0, 0]
+
+
 def storm_workload(pkg, oracle, seed, n_submissions=3000, p=STORM_MIXED):
     """Submissions of 0 to 300 ragged fragments in random order, each owning a stretch of one destination buffer:
     (pool on the device, sentinel-filled destination on the device, stream items, expected bytes, descriptor count)."""
@@ -622,6 +627,33 @@ def test_engine_long_runs_of_one_ticket_submissions_broken_by_others(pkg, hip, o
             assert 0xFFFFFFFFFFFFFFFF not in t and t[0] <= t[1] + slack and t[1] <= t[2] <= t[3], (len(items) - last + i, t)
             assert (t[3] - t[0]) / rate.value < 1e6, "microseconds, not a second"
     e.destroy()
+
+
+@pytest.mark.parametrize("depth", [1024, 96])
+def test_engine_deep_queue_of_submissions_of_up_to_64_fragments(pkg, hip, oracle, benchlib, depth):
+    """Submissions of 33 to 64 ragged fragments need several tickets of the usual size.  With a thousand in flight the
+    leader finds sixteen of them in a poll, asks its rolling loop, and that loop -- seeing more than a hundred
+    entries published ahead -- makes one ticket of up to 64 descriptors of each; with 96 in flight the queue is never
+    that deep, the loop hands back at once and is asked again only after longer and longer pauses.  Either way every
+    byte must be the oracle's and every submission consumed exactly once."""
+    assert abs(sum(STORM_UP_TO_64) - 1) < 1e-9
+    pool_d, dst_d, items, expect, descs = storm_workload(pkg, oracle, 0x64D + depth, 6000, STORM_UP_TO_64)
+    e = Engine(pkg, hip)
+    print("engine deep-queue case: depth=%d submissions=%d descriptors=%d" % (depth, len(items), len(descs)), flush=True)
+    wall, kern = ctypes.c_double(), ctypes.c_double()
+    lat = (ctypes.c_double * len(items))()
+    pkg.check(benchlib.tcpxuEngineRunTimed(e.h, items, len(items), 0, depth, 20000, ctypes.byref(wall), ctypes.byref(kern), lat), "tcpxuEngineRunTimed")
+    stats = pkg.EngineStats()
+    pkg.check(hip.tcpxuEngineGetStats(e.h, ctypes.byref(stats)), "tcpxuEngineGetStats")
+    print("engine deep-queue case: %.2f M submissions/s, %d entries in %d polls of which %d of 64"
+          % (len(items) / wall.value, stats.leader_entries, stats.leader_polls, stats.leader_deep_polls), flush=True)  # fmt: skip
+    assert e.completed() == len(items) and min(lat) > 0
+    assert stats.submissions == stats.leader_entries == len(items) and stats.leader_deep_polls <= stats.leader_polls
+    if depth >= 1024:
+        assert stats.leader_deep_polls > 0, "the rolling loop took part"
+    e.destroy()
+    got = dst_d.cpu().numpy()
+    assert first_difference(got, expect) is None, "first (index, got, want, count): %r" % (first_difference(got, expect),)
 
 
 def test_engine_sequence_numbers_cross_2_to_the_32(pkg, hip, oracle, benchlib, monkeypatch):
