@@ -240,6 +240,13 @@ template <typename T>
 __device__ __forceinline__ void sys_store(T* p, T v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, SYS);
 }
+// The same for memory that is known to be global (device memory, mapped host memory), said outright: where the
+// compiler cannot see that -- a pointer that arrived as a function's argument -- it would emit a flat_ store, which
+// the hardware is free to complete out of turn among a wavefront's memory instructions.
+template <typename T>
+__device__ __forceinline__ void sys_store_global(T* p, T v) {
+  __hip_atomic_store((TCPXU_GLOBAL T*)p, v, __ATOMIC_RELAXED, SYS);  // (only a C-style cast changes the address space)
+}
 __device__ __forceinline__ void drain_memory_ops() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); }
 
 __device__ __forceinline__ uint32_t bcast(uint32_t v, uint32_t src_lane) {
@@ -286,8 +293,8 @@ __device__ __forceinline__ uint32_t write_single_tickets_of_group(DevState* st, 
       if ((lane & 3u) == 3) {
         out.y = v.n | (v.slot << 8) | kOnlyTicket;
         out.z = target;
-        sys_store(&job_target[v.slot], target);
-        if (stamps) sys_store(&stamps[kStampsPerJob * v.slot], clock_now());
+        sys_store_global(&job_target[v.slot], target);
+        if (stamps) sys_store_global(&stamps[kStampsPerJob * v.slot], clock_now());
       }
       store_vec_sys(reinterpret_cast<uint8_t*>(&st->tickets[t & (kTicketRing - 1)]) + 16 * (lane & 3u), out);
     }
@@ -385,8 +392,10 @@ __device__ __attribute__((noinline)) StormEnd leader_storm(HostCtl* ctl_in, DevS
     const uint32_t at_s = static_cast<uint32_t>(s_g);  // (the mask keeps low bits only)
     const uint64_t entry = entry_base + (static_cast<uint64_t>((at_s + k_of_lane) & ring_mask) << 6);
     const uint64_t at = aux_base + (static_cast<uint64_t>((at_s + aux_add) & ring_mask) << aux_shift);
-    asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(sc) : "v"(entry) : "memory");
+    // (The job slots' words first: loads return in the order issued, so entries that are there whole -- every sector
+    // carries its stamp -- vouch for the words that were asked for before them.)
     asm volatile("global_load_dword %0, %1, off sc0 sc1" : "=v"(ax) : "v"(at) : "memory");
+    asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(sc) : "v"(entry) : "memory");
   };
   // kGroups while the loop feeds (that many groups in flight); once it has caught up with the host, the groups still
   // in flight that have not gone through: kGroups - 1, ..., 1, and at 0 the storm is over.
@@ -464,7 +473,7 @@ __device__ __attribute__((noinline)) StormEnd leader_storm(HostCtl* ctl_in, DevS
       s += consumed;
       entries += consumed;
       consumed = 0;
-      if (lane == 0) sys_store(&ctl->head, s);
+      if (lane == 0) sys_store_global(&ctl->head, s);
     }
     // Whatever is still in flight is waited for, so that the registers it lands in are free.
     asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
@@ -474,7 +483,7 @@ __device__ __attribute__((noinline)) StormEnd leader_storm(HostCtl* ctl_in, DevS
       s += consumed;
       entries += consumed;
       consumed = 0;
-      if (lane == 0) sys_store(&ctl->head, s);
+      if (lane == 0) sys_store_global(&ctl->head, s);
     }
     // Caught up with the host, every group in flight gone through whole (16 x kGroups entries at the least since the
     // loop was armed): the host publishes as requests complete, so more is on its way -- ask again from here instead of
