@@ -72,6 +72,8 @@ def test_bench_extras_report_latency_and_the_storm_sweep():
     r = run_bench(["--steps", "200", "--warmup", "20", "--cpu-seconds", "0.2", "--chunks", "8", "--pools", "2"], timeout=300)
     lat = r["latency_us"]["request_64KiB_16_descs"]
     assert 0 < lat["p50"] <= lat["p99"] and r["p50_request_us"] == lat["p50"]
+    deep = r["latency_us"]["budget"]["request_64KiB_16_descs_with_256_in_flight"]
+    assert deep["requests"] > 1000 and deep["p50_with_stamps"] > r["latency_us"]["budget"]["request_64KiB_16_descs"]["p50_with_stamps"]
     sweep = r["storm_64KiB"]["sweep"]
     assert [x["requests_in_flight"] for x in sweep] == [4, 8, 16, 32, 64, 128, 256, 512, 1024, 2048]  # up to "2048 concurrent"
     assert r["storm_64KiB"]["requests"] == 16 * 2048 and r["storm_64KiB"]["requests_timed"] == 15 * 2048
